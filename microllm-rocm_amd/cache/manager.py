@@ -1,0 +1,247 @@
+"""The cache manager: pages of keys and values with a block table per request, and state slots.
+
+Run entries of the model declare what they need: keys and values in pages
+(``PagedKVNeed``, perhaps with a window) or per-request state of fixed size
+(``StateNeed``). Entries with equal paged needs form a group; a group has a pool
+and page arrays of its own, one pair ``[pages, kv_heads, page_size, head_dim]``
+per entry, and every request has one block table per group. Pages are taken when
+a request's tokens cross a page's edge, given back when the request is closed,
+and, in a group with a window, as soon as every position on them is older than
+any later query can see. Nothing is cleared on reuse: lengths, not contents,
+say what is valid. The reference has no pages: one ``[slots, kv_heads, capacity,
+head_dim]`` tensor per layer, zero-filled on release (src/inference/kv_cache.cpp:11-64).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import torch
+
+from ..parts.base import CacheNeed, PagedKVNeed, StateNeed
+from .pages import OutOfPages, PagePool, SlotPool
+
+RELEASED = -1  # block-table entry of a page that a window has passed
+
+
+@dataclass
+class PagedBinding:
+    """What a mixer gets for paged keys and values: its entry's page arrays and its group."""
+    group: int
+    need: PagedKVNeed
+    k: Optional[torch.Tensor]
+    v: Optional[torch.Tensor]
+    owned: bool = True
+
+
+@dataclass
+class StateBinding:
+    """What a mixer gets for per-request state: ``state[slot]`` is the request's, zero when it opens."""
+    need: StateNeed
+    state: Optional[torch.Tensor]
+    owned: bool = True
+
+
+@dataclass
+class RequestCache:
+    request_id: Hashable
+    slot: int
+    num_tokens: int = 0                      # positions whose keys, values and state are in the cache
+    reserved: int = 0                        # positions beyond num_tokens that already have pages
+    pages: List[List[int]] = field(default_factory=list)  # per group: page of every block, RELEASED if given back
+    closed: bool = False
+
+
+class CacheGroup:
+    def __init__(self, index: int, need: PagedKVNeed, num_pages: int, page_size: int):
+        self.index = index
+        self.need = need
+        self.page_size = page_size
+        self.pool = PagePool(num_pages)
+        self.entries: List[int] = []
+
+    def first_needed_block(self, num_tokens: int) -> int:
+        """Blocks below this index hold no key that a query at ``num_tokens`` or later can see."""
+        if self.need.window is None:
+            return 0
+        oldest_visible = num_tokens - self.need.window + 1
+        return max(0, oldest_visible) // self.page_size
+
+
+class CacheManager:
+    def __init__(self, needs: Sequence[CacheNeed], reads: Sequence[Optional[int]], page_size: int,
+                 num_pages: int, max_requests: int, dtype: torch.dtype = torch.float32,
+                 device: Optional[torch.device] = None):
+        if page_size <= 0:
+            raise ValueError("page_size must be positive")
+        if len(needs) != len(reads):
+            raise ValueError("one need and one read source per run entry")
+        self.page_size = page_size
+        self.max_requests = max_requests
+        self.dtype = dtype
+        self.device = device
+        self.groups: List[CacheGroup] = []
+        self.slots = SlotPool(max_requests)
+        self.requests: Dict[Hashable, RequestCache] = {}
+        self._bindings: List[object] = [None] * len(needs)
+        self._state_tensors: List[torch.Tensor] = []
+        by_need: Dict[PagedKVNeed, CacheGroup] = {}
+        for entry, need in enumerate(needs):
+            if reads[entry] is not None:
+                continue
+            if isinstance(need, PagedKVNeed):
+                group = by_need.get(need)
+                if group is None:
+                    group = CacheGroup(len(self.groups), need, num_pages, page_size)
+                    self.groups.append(group)
+                    by_need[need] = group
+                group.entries.append(entry)
+                k = v = None
+                if device is not None:
+                    shape = (num_pages, need.kv_heads, page_size, need.head_dim)
+                    k = torch.empty(shape, dtype=dtype, device=device)
+                    v = torch.empty(shape, dtype=dtype, device=device)
+                self._bindings[entry] = PagedBinding(group.index, need, k, v, owned=True)
+            elif isinstance(need, StateNeed):
+                state = None
+                if device is not None:
+                    state = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
+                    self._state_tensors.append(state)
+                self._bindings[entry] = StateBinding(need, state, owned=True)
+            elif need is not None:
+                raise TypeError(f"run entry {entry} declares an unknown cache need {need!r}")
+        for entry, source in enumerate(reads):
+            if source is None:
+                continue
+            binding = self._bindings[source]
+            if binding is None:
+                raise ValueError(f"run entry {entry} reads the cache of entry {source}, which has none")
+            if isinstance(binding, PagedBinding):
+                self._bindings[entry] = PagedBinding(binding.group, binding.need, binding.k, binding.v, owned=False)
+            else:
+                self._bindings[entry] = StateBinding(binding.need, binding.state, owned=False)
+
+    # ---- what the model sees -------------------------------------------------------------
+    def bindings(self) -> List[object]:
+        return list(self._bindings)
+
+    # ---- requests ------------------------------------------------------------------------
+    def open(self, request_id: Hashable) -> RequestCache:
+        if request_id in self.requests:
+            raise KeyError(f"request {request_id!r} is already open")
+        slot = self.slots.take_one()
+        for state in self._state_tensors:
+            state[slot].zero_()
+        request = RequestCache(request_id, slot, pages=[[] for _ in self.groups])
+        self.requests[request_id] = request
+        return request
+
+    def get(self, request_id: Hashable) -> RequestCache:
+        try:
+            return self.requests[request_id]
+        except KeyError:
+            raise KeyError(f"request {request_id!r} is not open") from None
+
+    def blocks_for(self, tokens: int) -> int:
+        return (tokens + self.page_size - 1) // self.page_size
+
+    def pages_needed(self, request: RequestCache, count: int) -> List[int]:
+        """Pages each group would have to take to hold ``count`` more positions."""
+        total = request.num_tokens + request.reserved + count
+        return [max(0, self.blocks_for(total) - len(request.pages[group.index])) for group in self.groups]
+
+    def can_reserve(self, request: RequestCache, count: int) -> bool:
+        return all(need <= group.pool.num_free
+                   for need, group in zip(self.pages_needed(request, count), self.groups))
+
+    def reserve(self, request: RequestCache, count: int) -> None:
+        """Take the pages for ``count`` more positions in every group, or none at all."""
+        if request.closed:
+            raise KeyError(f"request {request.request_id!r} is closed")
+        if count < 0:
+            raise ValueError("cannot reserve a negative number of positions")
+        needed = self.pages_needed(request, count)
+        for need, group in zip(needed, self.groups):
+            if need > group.pool.num_free:
+                raise OutOfPages(f"request {request.request_id!r} needs {need} pages in group {group.index}, "
+                                 f"{group.pool.num_free} free of {group.pool.num_pages}")
+        for need, group in zip(needed, self.groups):
+            request.pages[group.index].extend(group.pool.take(need))
+        request.reserved += count
+
+    def cancel_reservation(self, request: RequestCache) -> None:
+        """Give back pages that only a reservation needed (a step that did not run)."""
+        keep = self.blocks_for(request.num_tokens)
+        for group in self.groups:
+            pages = request.pages[group.index]
+            extra = [page for page in pages[keep:] if page != RELEASED]
+            group.pool.give(extra)
+            del pages[keep:]
+        request.reserved = 0
+
+    def commit(self, request: RequestCache, count: int) -> None:
+        """``count`` reserved positions now hold keys and values; pages a window has passed go back."""
+        if count > request.reserved:
+            raise ValueError("cannot commit more positions than were reserved")
+        request.num_tokens += count
+        request.reserved -= count
+        for group in self.groups:
+            first = group.first_needed_block(request.num_tokens)
+            pages = request.pages[group.index]
+            passed = [index for index in range(min(first, len(pages))) if pages[index] != RELEASED]
+            if passed:
+                group.pool.give(pages[index] for index in passed)
+                for index in passed:
+                    pages[index] = RELEASED
+
+    def close(self, request_id: Hashable) -> None:
+        request = self.requests.pop(request_id, None)
+        if request is None:
+            raise KeyError(f"request {request_id!r} is not open")
+        for group in self.groups:
+            group.pool.give(page for page in request.pages[group.index] if page != RELEASED)
+            request.pages[group.index] = []
+        self.slots.give([request.slot])
+        request.closed = True
+
+    # ---- accounting ----------------------------------------------------------------------
+    def free_pages(self) -> List[int]:
+        return [group.pool.num_free for group in self.groups]
+
+    def held_pages(self) -> List[int]:
+        return [group.pool.num_held for group in self.groups]
+
+    def bytes_per_page(self, group: CacheGroup) -> int:
+        element = torch.empty((), dtype=self.dtype).element_size()
+        return 2 * len(group.entries) * group.need.kv_heads * self.page_size * group.need.head_dim * element
+
+    def allocated_bytes(self) -> int:
+        return sum(self.bytes_per_page(group) * group.pool.num_pages for group in self.groups)
+
+    def active_bytes(self) -> int:
+        return sum(self.bytes_per_page(group) * group.pool.num_held for group in self.groups)
+
+    def check(self) -> None:
+        """Every page is either free or held by exactly one request; every slot likewise."""
+        for group in self.groups:
+            seen: Dict[int, Hashable] = {}
+            for request in self.requests.values():
+                for page in request.pages[group.index]:
+                    if page == RELEASED:
+                        continue
+                    if page in seen:
+                        raise AssertionError(f"page {page} of group {group.index} is held by "
+                                             f"{seen[page]!r} and {request.request_id!r}")
+                    seen[page] = request.request_id
+            free = group.pool.free_pages()
+            if len(set(free)) != len(free):
+                raise AssertionError(f"group {group.index}: a page is on the free list twice")
+            if set(free) & set(seen):
+                raise AssertionError(f"group {group.index}: a held page is on the free list")
+            if len(free) + len(seen) != group.pool.num_pages:
+                raise AssertionError(f"group {group.index}: {group.pool.num_pages - len(free) - len(seen)} pages lost")
+        slots = [request.slot for request in self.requests.values()]
+        if len(set(slots)) != len(slots):
+            raise AssertionError("two requests share a state slot")
+        if len(slots) + self.slots.num_free != self.max_requests:
+            raise AssertionError("a state slot is lost")

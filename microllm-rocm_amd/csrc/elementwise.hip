@@ -1,0 +1,259 @@
+// Row-wise kernels around the matrix products: embedding gather, RMSNorm with the residual
+// sum, bias + rotation + page write of the attention projections, and SiLU-mul.
+#include "common.h"
+#include "microllm_hip.h"
+
+namespace mll {
+
+static thread_local std::string g_error;
+void set_error(const std::string& text) { g_error = text; }
+int fail(const std::string& text) {
+    g_error = text;
+    return 1;
+}
+
+// ---------------------------------------------------------------------------------------------
+template <typename W>
+__global__ void embedding_kernel(const W* __restrict__ table, const int32_t* __restrict__ ids,
+                                 float* __restrict__ out, int width, int vocab) {
+    const int token = blockIdx.x;
+    const int id = ids[token];
+    float* row_out = out + static_cast<int64_t>(token) * width;
+    if (id < 0 || id >= vocab) {
+        for (int column = threadIdx.x; column < width; column += blockDim.x) row_out[column] = NAN;
+        return;
+    }
+    const W* row = table + static_cast<int64_t>(id) * width;
+    for (int column = threadIdx.x; column < width; column += blockDim.x) row_out[column] = to_float(row[column]);
+}
+
+// ---------------------------------------------------------------------------------------------
+// One block per output row. The sum of squares is taken in float32: per-thread strided partial
+// sums, a butterfly inside each wave, then the waves in ascending order.
+template <typename T>
+__global__ void rms_norm_kernel(float* __restrict__ h, const T* __restrict__ delta,
+                                const int32_t* __restrict__ rows, const float* __restrict__ weight,
+                                float eps, T* __restrict__ out, int width, int write_h) {
+    __shared__ float scratch[16];
+    const int index = blockIdx.x;
+    const int64_t source = rows ? rows[index] : index;
+    float* h_row = h + source * width;
+    const T* delta_row = delta ? delta + source * width : nullptr;
+    T* out_row = out + static_cast<int64_t>(index) * width;
+
+    float partial = 0.0f;
+    for (int column = threadIdx.x; column < width; column += blockDim.x) {
+        float value = h_row[column];
+        if (delta_row) value += to_float(delta_row[column]);
+        if (write_h) h_row[column] = value;
+        partial += value * value;
+    }
+    const float total = block_sum(partial, scratch);
+    const float inverse_rms = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
+    for (int column = threadIdx.x; column < width; column += blockDim.x) {
+        float value = h_row[column];  // already holds the sum when write_h
+        if (delta_row && !write_h) value += to_float(delta_row[column]);
+        out_row[column] = from_float<T>(value * inverse_rms * weight[column]);
+    }
+}
+
+template <typename T>
+__global__ void residual_add_kernel(float* __restrict__ h, const T* __restrict__ delta, int64_t count) {
+    const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (index < count) h[index] += to_float(delta[index]);
+}
+
+// ---------------------------------------------------------------------------------------------
+// One block per token. Angles are position * inv_freq in float64, so cos and sin are the
+// correctly rounded float32 values for any position; they are computed once per token into LDS
+// and shared by all heads.
+constexpr int kMaxHeadDim = 512;
+
+template <typename T>
+__global__ void qkv_rope_store_kernel(const T* __restrict__ qkv, const float* __restrict__ bias,
+                                      const int32_t* __restrict__ positions,
+                                      const int32_t* __restrict__ slot_mapping,
+                                      const double* __restrict__ inv_freq, int n_freq,
+                                      T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                      int heads, int kv_heads, int head_dim, int page_size) {
+    __shared__ float cos_table[kMaxHeadDim / 2];
+    __shared__ float sin_table[kMaxHeadDim / 2];
+    const int token = blockIdx.x;
+    const int position = positions[token];
+    for (int index = threadIdx.x; index < n_freq; index += blockDim.x) {
+        const double angle = static_cast<double>(position) * inv_freq[index];
+        cos_table[index] = static_cast<float>(cos(angle));
+        sin_table[index] = static_cast<float>(sin(angle));
+    }
+    __syncthreads();
+
+    const int half = head_dim / 2;
+    const int total_heads = heads + 2 * kv_heads;
+    const int64_t in_row = static_cast<int64_t>(token) * total_heads * head_dim;
+    const int slot = slot_mapping ? slot_mapping[token] : -1;
+    const int64_t page = slot >= 0 ? slot / page_size : 0;
+    const int offset = slot >= 0 ? slot % page_size : 0;
+
+    for (int item = threadIdx.x; item < total_heads * half; item += blockDim.x) {
+        const int head = item / half;
+        const int pair = item % half;
+        const bool is_value = head >= heads + kv_heads;
+        int first, second;
+        bool rotate;
+        if (pair < n_freq) {
+            first = pair;
+            second = pair + n_freq;
+            rotate = !is_value;
+        } else {  // dims beyond the rotary part pass through, two per item
+            first = 2 * n_freq + 2 * (pair - n_freq);
+            second = first + 1;
+            rotate = false;
+        }
+        const int column = head * head_dim;
+        float x1 = to_float(qkv[in_row + column + first]);
+        float x2 = to_float(qkv[in_row + column + second]);
+        if (bias) {
+            x1 += bias[column + first];
+            x2 += bias[column + second];
+        }
+        float y1 = x1, y2 = x2;
+        if (rotate) {
+            const float c = cos_table[pair], s = sin_table[pair];
+            y1 = x1 * c - x2 * s;
+            y2 = x1 * s + x2 * c;
+        }
+        if (head < heads) {
+            T* q_row = q_out + (static_cast<int64_t>(token) * heads + head) * head_dim;
+            q_row[first] = from_float<T>(y1);
+            q_row[second] = from_float<T>(y2);
+        } else if (slot >= 0) {
+            const int kv_head = is_value ? head - heads - kv_heads : head - heads;
+            T* cache = is_value ? v_cache : k_cache;
+            T* row = cache + ((page * kv_heads + kv_head) * page_size + offset) * head_dim;
+            row[first] = from_float<T>(y1);
+            row[second] = from_float<T>(y2);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+__device__ inline float stable_sigmoid(float value) {
+    if (value >= 0.0f) return 1.0f / (1.0f + expf(-value));
+    const float e = expf(value);
+    return e / (1.0f + e);
+}
+
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gate, const T* __restrict__ up, int64_t in_stride,
+                                T* __restrict__ out, int width) {
+    const int token = blockIdx.y;
+    const int column = blockIdx.x * blockDim.x + threadIdx.x;
+    if (column >= width) return;
+    const float g = to_float(gate[token * in_stride + column]);
+    const float u = to_float(up[token * in_stride + column]);
+    out[static_cast<int64_t>(token) * width + column] = from_float<T>(g * stable_sigmoid(g) * u);
+}
+
+}  // namespace mll
+
+using namespace mll;
+
+extern "C" {
+
+const char* mll_last_error() { return g_error.c_str(); }
+int mll_version() { return 1; }
+
+int mll_embedding(const void* table, int table_dtype, const int32_t* ids, float* out,
+                  int n_tokens, int width, int vocab, hipStream_t stream) {
+    MLL_REQUIRE(n_tokens >= 0 && width > 0 && vocab > 0, "embedding: sizes must be positive");
+    if (n_tokens == 0) return 0;
+    if (table_dtype == kF32) {
+        embedding_kernel<float><<<n_tokens, 256, 0, stream>>>(static_cast<const float*>(table), ids, out, width, vocab);
+    } else if (table_dtype == kBF16) {
+        embedding_kernel<bf16><<<n_tokens, 256, 0, stream>>>(static_cast<const bf16*>(table), ids, out, width, vocab);
+    } else {
+        return fail("embedding: unknown table dtype");
+    }
+    return check_launch("embedding");
+}
+
+int mll_rms_norm(float* h, const void* delta, const int32_t* rows, const float* weight, float eps,
+                 void* out, int dtype, int n_rows, int width, int write_h, hipStream_t stream) {
+    MLL_REQUIRE(n_rows >= 0 && width > 0, "rms_norm: sizes must be positive");
+    MLL_REQUIRE(eps > 0.0f, "rms_norm: eps must be positive");
+    MLL_REQUIRE(!(write_h && rows), "rms_norm: cannot write h through a row selection");
+    if (n_rows == 0) return 0;
+    const int threads = width >= 2048 ? 512 : 256;
+    if (dtype == kF32) {
+        rms_norm_kernel<float><<<n_rows, threads, 0, stream>>>(h, static_cast<const float*>(delta), rows, weight, eps,
+                                                               static_cast<float*>(out), width, write_h);
+    } else if (dtype == kBF16) {
+        rms_norm_kernel<bf16><<<n_rows, threads, 0, stream>>>(h, static_cast<const bf16*>(delta), rows, weight, eps,
+                                                              static_cast<bf16*>(out), width, write_h);
+    } else {
+        return fail("rms_norm: unknown dtype");
+    }
+    return check_launch("rms_norm");
+}
+
+int mll_residual_add(float* h, const void* delta, int dtype, int n_rows, int width, hipStream_t stream) {
+    const int64_t count = static_cast<int64_t>(n_rows) * width;
+    if (count == 0) return 0;
+    const int blocks = static_cast<int>((count + 255) / 256);
+    if (dtype == kF32) {
+        residual_add_kernel<float><<<blocks, 256, 0, stream>>>(h, static_cast<const float*>(delta), count);
+    } else if (dtype == kBF16) {
+        residual_add_kernel<bf16><<<blocks, 256, 0, stream>>>(h, static_cast<const bf16*>(delta), count);
+    } else {
+        return fail("residual_add: unknown dtype");
+    }
+    return check_launch("residual_add");
+}
+
+int mll_qkv_rope_store(const void* qkv, int dtype, const float* bias, const int32_t* positions,
+                       const int32_t* slot_mapping, const double* inv_freq, int n_freq,
+                       void* q_out, void* k_cache, void* v_cache,
+                       int n_tokens, int heads, int kv_heads, int head_dim, int page_size,
+                       hipStream_t stream) {
+    MLL_REQUIRE(heads > 0 && kv_heads >= 0 && head_dim > 0, "qkv_rope_store: sizes must be positive");
+    MLL_REQUIRE(head_dim % 2 == 0 && head_dim <= kMaxHeadDim, "qkv_rope_store: head_dim must be even and at most 512");
+    MLL_REQUIRE(n_freq >= 0 && 2 * n_freq <= head_dim, "qkv_rope_store: rotary part exceeds head_dim");
+    MLL_REQUIRE(inv_freq != nullptr || n_freq == 0, "qkv_rope_store: n_freq without a frequency table");
+    MLL_REQUIRE(slot_mapping == nullptr || (k_cache && v_cache && page_size > 0),
+                "qkv_rope_store: slot_mapping needs both caches and a page size");
+    if (n_tokens == 0) return 0;
+    if (dtype == kF32) {
+        qkv_rope_store_kernel<float><<<n_tokens, 256, 0, stream>>>(
+            static_cast<const float*>(qkv), bias, positions, slot_mapping, inv_freq, n_freq,
+            static_cast<float*>(q_out), static_cast<float*>(k_cache), static_cast<float*>(v_cache),
+            heads, kv_heads, head_dim, page_size);
+    } else if (dtype == kBF16) {
+        qkv_rope_store_kernel<bf16><<<n_tokens, 256, 0, stream>>>(
+            static_cast<const bf16*>(qkv), bias, positions, slot_mapping, inv_freq, n_freq,
+            static_cast<bf16*>(q_out), static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache),
+            heads, kv_heads, head_dim, page_size);
+    } else {
+        return fail("qkv_rope_store: unknown dtype");
+    }
+    return check_launch("qkv_rope_store");
+}
+
+int mll_silu_mul(const void* gate, const void* up, int64_t in_stride, void* out, int dtype,
+                 int n_tokens, int width, hipStream_t stream) {
+    MLL_REQUIRE(n_tokens >= 0 && width > 0 && in_stride >= width, "silu_mul: bad sizes");
+    if (n_tokens == 0) return 0;
+    MLL_REQUIRE(n_tokens <= 65535, "silu_mul: more than 65535 tokens in one call");
+    const dim3 grid((width + 255) / 256, n_tokens);
+    if (dtype == kF32) {
+        silu_mul_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(gate), static_cast<const float*>(up),
+                                                         in_stride, static_cast<float*>(out), width);
+    } else if (dtype == kBF16) {
+        silu_mul_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(gate), static_cast<const bf16*>(up),
+                                                        in_stride, static_cast<bf16*>(out), width);
+    } else {
+        return fail("silu_mul: unknown dtype");
+    }
+    return check_launch("silu_mul");
+}
+
+}  // extern "C"

@@ -1,0 +1,69 @@
+// C interface of libmicrollm_hip: every function launches on `stream`, returns 0 or a
+// non-zero code, and leaves a text for mll_last_error() when it refuses its arguments.
+// Pointers are device pointers unless a comment says otherwise. `dtype` is 0 for float32 and
+// 1 for bfloat16 and names the element type of activations, cache pages and, where stated,
+// weights. Statistics, softmax and accumulators are float32 in every kernel.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+extern "C" {
+
+const char* mll_last_error();
+int mll_version();
+
+// out[t, :] = table[ids[t], :] widened to float32. An id outside [0, vocab) gives a row of NaN.
+int mll_embedding(const void* table, int table_dtype, const int32_t* ids, float* out,
+                  int n_tokens, int width, int vocab, hipStream_t stream);
+
+// For i < n_rows, r = rows ? rows[i] : i:  v = h[r] + (delta ? delta[r] : 0);
+// if write_h, h[r] = v;  out[i] = v * rsqrt(mean(v^2) + eps) * weight.
+// h is the float32 residual stream; delta and out have element type `dtype`.
+int mll_rms_norm(float* h, const void* delta, const int32_t* rows, const float* weight, float eps,
+                 void* out, int dtype, int n_rows, int width, int write_h, hipStream_t stream);
+
+// Adds a pending delta into the residual stream: h[r] += delta[r] for all rows.
+int mll_residual_add(float* h, const void* delta, int dtype, int n_rows, int width, hipStream_t stream);
+
+// Splits fused projections qkv[t] = [q (H*hd) | k (KVH*hd) | v (KVH*hd)], adds `bias` (nullable),
+// rotates q and k by the split-half rule with angle position * inv_freq[i] in float64 (inv_freq nullable:
+// no rotation; rotary_dim = 2 * n_freq <= hd), writes q to q_out[t] and k, v into the pages:
+// slot = slot_mapping[t] (negative: not stored) addresses [page, kv_head, offset, :] with
+// page = slot / page_size.  k_cache / v_cache nullable together with slot_mapping.
+int mll_qkv_rope_store(const void* qkv, int dtype, const float* bias, const int32_t* positions,
+                       const int32_t* slot_mapping, const double* inv_freq, int n_freq,
+                       void* q_out, void* k_cache, void* v_cache,
+                       int n_tokens, int heads, int kv_heads, int head_dim, int page_size,
+                       hipStream_t stream);
+
+// Attention of every query token over its request's pages, one wave per (token, head).
+// Key j is visible to a query at position p iff j <= p and (window <= 0 or p - j < window).
+// block_table[seq, j / page_size] gives the page of key j. Reduction order depends only on
+// (p, window), so the result does not depend on how tokens were cut into steps.
+int mll_paged_attention_rowwise(const void* q, int dtype, const void* k_cache, const void* v_cache,
+                                const int32_t* block_table, int table_width,
+                                const int32_t* seq_of_token, const int32_t* positions, void* out,
+                                float scale, int window, int n_tokens, int heads, int kv_heads,
+                                int head_dim, int page_size, hipStream_t stream);
+
+// out[t, c] = silu(gate[t, c]) * up[t, c]; gate and up rows are `in_stride` elements apart.
+int mll_silu_mul(const void* gate, const void* up, int64_t in_stride, void* out, int dtype,
+                 int n_tokens, int width, hipStream_t stream);
+
+// C[m, n] = sum_k A[m, k] * W[n, k] (+ bias[n]), all float32, k summed in ascending order by one
+// thread per output element, so a row's result does not depend on the other rows.
+int mll_gemm_f32(const float* a, const float* w, const float* bias, float* c,
+                 int m, int n, int k, hipStream_t stream);
+
+// Index of the first maximum of each row; a row that holds a non-finite value gives -1.
+int mll_argmax(const float* logits, int32_t* out, int n_rows, int vocab, hipStream_t stream);
+
+// Draws one token per row from softmax(logits / temperature) restricted to the top_k largest
+// logits (top_k <= 0: all; ties at the k-th value go to the lower token ids), by inverse CDF in
+// token order with the given uniform in [0, 1). temperature == 0 or top_k == 1 gives the
+// argmax. A non-finite logit gives -1. top_k may be null.
+int mll_sample(const float* logits, const float* temperature, const int32_t* top_k,
+               const float* uniform, int32_t* out, int n_rows, int vocab, hipStream_t stream);
+
+}  // extern "C"

@@ -1,0 +1,134 @@
+"""The batch of one step: a flat list of tokens with, for every request in it, where its portion starts.
+
+A step holds portions of prompts beside single decoded tokens. Everything a
+kernel needs to find a token's request, position and pages is packed into one
+int32 buffer on the host and copied to the device in one transfer (the reference
+packs tokens, positions and rows the same way, src/model/model.cpp:1522-1538).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager, RELEASED, RequestCache
+
+
+@dataclass
+class StepEntry:
+    """One request's next tokens and the places among them whose logits are wanted."""
+    request_id: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class PagedView:
+    """One cache group as the step sees it."""
+    block_table: torch.Tensor   # int32 [requests, width]; RELEASED where a window has passed
+    slot_mapping: torch.Tensor  # int32 [tokens]: page * page_size + offset of every token's key and value
+    page_size: int
+    width: int
+
+
+@dataclass
+class StepContext:
+    n_tokens: int
+    n_seqs: int
+    tokens: torch.Tensor        # int32 [tokens]
+    positions: torch.Tensor     # int32 [tokens]: absolute position of every token in its request
+    seq_of_token: torch.Tensor  # int32 [tokens]: index into this step's requests
+    cu_tokens: torch.Tensor     # int32 [requests + 1]: where each request's portion starts in the flat list
+    seq_start: torch.Tensor     # int32 [requests]: position of the portion's first token
+    seq_total: torch.Tensor     # int32 [requests]: positions in the cache once this step is done
+    slots: torch.Tensor         # int32 [requests]: state slot of every request
+    want_rows: Optional[torch.Tensor]  # int32 [wanted]: rows of the flat list whose logits are wanted
+    paged: List[PagedView]
+    # the same on the host, for parts written in Python and for choosing kernels
+    starts: List[int] = field(default_factory=list)
+    counts: List[int] = field(default_factory=list)
+    host_slots: List[int] = field(default_factory=list)
+    max_count: int = 0
+    max_total: int = 0
+
+
+class BatchBuilder:
+    """Packs a step's metadata and moves it to the device through one pinned staging buffer."""
+
+    def __init__(self, cache: CacheManager, device: torch.device):
+        self.cache = cache
+        self.device = device
+        self._staging: Optional[torch.Tensor] = None
+        self._device_buffer: Optional[torch.Tensor] = None
+        self._copied = None
+
+    def _buffers(self, size: int):
+        if self._staging is None or self._staging.numel() < size:
+            capacity = max(4096, 1 << (size - 1).bit_length())
+            self._staging = torch.empty(capacity, dtype=torch.int32, pin_memory=True)
+            self._device_buffer = torch.empty(capacity, dtype=torch.int32, device=self.device)
+            self._copied = None
+        if self._copied is not None:
+            self._copied.synchronize()  # the last step's copy has left the staging buffer
+        return self._staging, self._device_buffer
+
+    def build(self, requests: Sequence[RequestCache], token_lists: Sequence[Sequence[int]],
+              wants: Sequence[Sequence[int]]) -> StepContext:
+        page_size = self.cache.page_size
+        counts = [len(tokens) for tokens in token_lists]
+        starts = [request.num_tokens for request in requests]
+        n_seqs = len(requests)
+        n_tokens = sum(counts)
+        totals = [start + count for start, count in zip(starts, counts)]
+        cu = np.zeros(n_seqs + 1, dtype=np.int32)
+        np.cumsum(counts, out=cu[1:])
+        tokens = np.concatenate([np.asarray(t, dtype=np.int32) for t in token_lists]) if n_tokens else np.zeros(0, np.int32)
+        positions = np.concatenate([np.arange(s, s + c, dtype=np.int32) for s, c in zip(starts, counts)]) \
+            if n_tokens else np.zeros(0, np.int32)
+        seq_of_token = np.repeat(np.arange(n_seqs, dtype=np.int32), counts)
+        want_rows = np.asarray([cu[index] + place for index, want in enumerate(wants) for place in want],
+                               dtype=np.int32)
+        tables, mappings, widths = [], [], []
+        for group in self.cache.groups:
+            width = max(1, max(len(request.pages[group.index]) for request in requests))
+            table = np.full((n_seqs, width), RELEASED, dtype=np.int32)
+            for row, request in enumerate(requests):
+                pages = request.pages[group.index]
+                table[row, :len(pages)] = pages
+            mapping = table[seq_of_token, positions // page_size] * page_size + positions % page_size
+            tables.append(table)
+            mappings.append(mapping.astype(np.int32))
+            widths.append(width)
+        slots = np.asarray([request.slot for request in requests], dtype=np.int32)
+        pieces = [tokens, positions, seq_of_token, cu, np.asarray(starts, np.int32), np.asarray(totals, np.int32),
+                  slots, want_rows]
+        for table, mapping in zip(tables, mappings):
+            pieces += [table.reshape(-1), mapping]
+        offsets, cursor = [], 0
+        for piece in pieces:
+            offsets.append(cursor)
+            cursor += (piece.size + 3) // 4 * 4  # keep every piece 16-byte aligned
+        staging, device_buffer = self._buffers(max(cursor, 1))
+        host = staging.numpy()
+        for offset, piece in zip(offsets, pieces):
+            host[offset:offset + piece.size] = piece
+        device_buffer[:cursor].copy_(staging[:cursor], non_blocking=True)
+        self._copied = torch.cuda.Event()
+        self._copied.record()
+
+        def piece_at(index: int, shape=None) -> torch.Tensor:
+            view = device_buffer[offsets[index]:offsets[index] + pieces[index].size]
+            return view if shape is None else view.view(shape)
+
+        paged = []
+        for g, group in enumerate(self.cache.groups):
+            paged.append(PagedView(piece_at(8 + 2 * g, (n_seqs, widths[g])), piece_at(9 + 2 * g),
+                                   page_size, widths[g]))
+        return StepContext(
+            n_tokens=n_tokens, n_seqs=n_seqs, tokens=piece_at(0), positions=piece_at(1), seq_of_token=piece_at(2),
+            cu_tokens=piece_at(3), seq_start=piece_at(4), seq_total=piece_at(5), slots=piece_at(6),
+            want_rows=piece_at(7) if want_rows.size else None, paged=paged,
+            starts=list(starts), counts=counts, host_slots=[request.slot for request in requests],
+            max_count=max(counts) if counts else 0, max_total=max(totals) if totals else 0)

@@ -1,0 +1,144 @@
+"""The engine: a model, its cache and the one step function.
+
+``step`` takes a batch of (request, its next tokens, wanted places): portions of
+prompts beside single decoded tokens, cut anywhere. It runs only those tokens,
+as one batch, against what earlier steps left in the cache, and returns the
+float32 logits at the wanted places. The reference has five entry points, each
+with its own batch shape (src/model/model.cpp:1091-1135, 1263-1303, 1316-1354,
+1419-1439, 1448-1572); this is the one that replaces them.
+"""
+from __future__ import annotations
+
+import os
+from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Union
+
+import torch
+
+from ..cache.manager import CacheManager, RequestCache
+from ..cache.pages import OutOfPages
+from ..config.registry import architecture_named, load_config
+from ..ops import library
+from ..parts import Model, ModelSpec, Runtime
+from ..weights import load_folder, place_all, random_tensors
+from .batch import BatchBuilder, StepContext, StepEntry
+
+_DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": torch.bfloat16, "bf16": torch.bfloat16}
+
+
+def parse_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
+    if isinstance(dtype, torch.dtype):
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"the engine runs in float32 or bfloat16, not {dtype}")
+        return dtype
+    if dtype not in _DTYPES:
+        raise ValueError(f"unknown dtype {dtype!r}; use float32 or bfloat16")
+    return _DTYPES[dtype]
+
+
+class Engine:
+    def __init__(self, spec: ModelSpec, tensors: Mapping[str, torch.Tensor], dtype: Union[str, torch.dtype] = "bfloat16",
+                 device: Union[str, torch.device] = "cuda:0", page_size: int = 16,
+                 max_tokens: Optional[int] = None, num_pages: Optional[int] = None, max_requests: int = 64,
+                 tensors_placed: bool = False):
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU is visible; this engine has no CPU path")
+        library.load()  # fail now, and loudly, if the kernels are missing and cannot be built
+        self.dtype = parse_dtype(dtype)
+        self.device = torch.device(device)
+        torch.cuda.set_device(self.device)
+        self.spec = spec
+        self.runtime = Runtime(dtype=self.dtype, device=self.device)
+        self.model = Model(spec, self.runtime)
+        decls = self.model.tensors()
+        if not tensors_placed:
+            tensors = place_all(tensors, decls, self.dtype, self.device)
+        self.model.bind(tensors)
+        del tensors
+        if num_pages is None:
+            if max_tokens is None:
+                raise ValueError("give max_tokens or num_pages: the cache pool is sized once")
+            num_pages = max(1, -(-max_tokens // page_size))
+        reads = [entry.reads_cache_of for entry in spec.order]
+        self.cache = CacheManager(self.model.cache_needs(), reads, page_size, num_pages, max_requests,
+                                  dtype=self.dtype, device=self.device)
+        self._bindings = self.cache.bindings()
+        self._builder = BatchBuilder(self.cache, self.device)
+        self.steps_run = 0
+
+    # ---- construction --------------------------------------------------------------------
+    @classmethod
+    def from_folder(cls, folder: str, dtype: Union[str, torch.dtype] = "bfloat16", device="cuda:0", **options) -> "Engine":
+        """Read ``config.json``, choose the model by its architecture name, load ``model.safetensors``."""
+        architecture, config = load_config(folder)
+        spec = architecture.build_spec(config)
+        engine_dtype = parse_dtype(dtype)
+        probe = Model(spec, Runtime(dtype=engine_dtype, device=torch.device("cpu")))
+        tensors = load_folder(folder, probe.tensors(), engine_dtype, torch.device(device))
+        engine = cls(spec, tensors, dtype=engine_dtype, device=device, tensors_placed=True, **options)
+        engine.config = config
+        return engine
+
+    @classmethod
+    def from_random(cls, config, seed: int = 0, dtype: Union[str, torch.dtype] = "bfloat16", device="cuda:0",
+                    stds: Optional[Mapping[str, float]] = None, on_device: bool = False, **options) -> "Engine":
+        """Random weights drawn in memory (on the GPU when ``on_device``: for sizes too large to draw on the host)."""
+        architecture = architecture_named(config.architecture)
+        spec = architecture.build_spec(config)
+        engine_dtype = parse_dtype(dtype)
+        probe = Model(spec, Runtime(dtype=engine_dtype, device=torch.device("cpu")))
+        tensors = random_tensors(probe.tensors(), architecture.init_rules(config), seed, dtype=torch.bfloat16,
+                                 stds=stds, device=device if on_device else "cpu")
+        engine = cls(spec, tensors, dtype=engine_dtype, device=device, **options)
+        engine.config = config
+        return engine
+
+    # ---- requests ------------------------------------------------------------------------
+    def open(self, request_id: Hashable) -> RequestCache:
+        return self.cache.open(request_id)
+
+    def close(self, request_id: Hashable) -> None:
+        self.cache.close(request_id)
+
+    def is_open(self, request_id: Hashable) -> bool:
+        return request_id in self.cache.requests
+
+    # ---- the step ------------------------------------------------------------------------
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Run one batch; returns float32 logits ``[wanted, vocab]`` in the order of entries and of ``want``."""
+        entries = [entry if isinstance(entry, StepEntry) else StepEntry(*entry) for entry in entries]
+        if not entries:
+            return None
+        requests: List[RequestCache] = []
+        seen = set()
+        for entry in entries:
+            if entry.request_id in seen:
+                raise ValueError(f"request {entry.request_id!r} appears twice in one step")
+            seen.add(entry.request_id)
+            request = self.cache.get(entry.request_id)
+            count = len(entry.tokens)
+            if count == 0:
+                raise ValueError(f"request {entry.request_id!r} brings no tokens")
+            for token in entry.tokens:
+                if not 0 <= int(token) < self.spec.vocab_size:
+                    raise ValueError(f"token {token} of request {entry.request_id!r} is outside the vocabulary")
+            if request.num_tokens + count > self.spec.max_positions:
+                raise ValueError(f"request {entry.request_id!r} would pass max positions {self.spec.max_positions}")
+            for place in entry.want:
+                if not 0 <= place < count:
+                    raise ValueError(f"wanted place {place} of request {entry.request_id!r} is outside its {count} tokens")
+            requests.append(request)
+        reserved: List[RequestCache] = []
+        try:
+            for request, entry in zip(requests, entries):
+                self.cache.reserve(request, len(entry.tokens))
+                reserved.append(request)
+        except OutOfPages:
+            for request in reserved:
+                self.cache.cancel_reservation(request)
+            raise
+        ctx = self._builder.build(requests, [entry.tokens for entry in entries], [entry.want for entry in entries])
+        logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
+        for request, entry in zip(requests, entries):
+            self.cache.commit(request, len(entry.tokens))
+        self.steps_run += 1
+        return logits

@@ -1,0 +1,268 @@
+"""Python bindings of the HIP kernels: shape and type checks on the host, then one launch.
+
+Every function takes torch tensors on the GPU, launches on torch's current HIP
+stream and returns the output tensor. Checks happen here, before the launch, so
+a kernel never sees operands that do not fit what its grid assumes.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import library
+from .library import KernelLibraryError
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype not in _CODES:
+        raise KernelLibraryError(f"kernels take float32 or bfloat16, got {dtype}")
+    return _CODES[dtype]
+
+
+def _ptr(tensor: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if tensor is None else tensor.data_ptr())
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(status: int, lib) -> None:
+    if status != 0:
+        raise KernelLibraryError(lib.mll_last_error().decode("utf-8", "replace"))
+
+
+def _need(condition: bool, text: str) -> None:
+    if not condition:
+        raise KernelLibraryError(text)
+
+
+def _device_tensor(tensor: torch.Tensor, name: str, dtype: Optional[torch.dtype] = None) -> None:
+    _need(tensor.is_cuda, f"{name} must live on the GPU")
+    _need(tensor.is_contiguous(), f"{name} must be contiguous")
+    if dtype is not None:
+        _need(tensor.dtype == dtype, f"{name} must be {dtype}, got {tensor.dtype}")
+
+
+def embedding(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    lib = library.load()
+    _device_tensor(table, "embedding table")
+    _device_tensor(ids, "token ids", torch.int32)
+    _need(table.dim() == 2 and ids.dim() == 1, "embedding takes a [vocab, width] table and [tokens] ids")
+    vocab, width = table.shape
+    if out is None:
+        out = torch.empty((ids.shape[0], width), dtype=torch.float32, device=table.device)
+    _device_tensor(out, "embedding output", torch.float32)
+    _need(tuple(out.shape) == (ids.shape[0], width), "embedding output has the wrong shape")
+    _check(lib.mll_embedding(_ptr(table), _code(table.dtype), _ptr(ids), _ptr(out),
+                             ids.shape[0], width, vocab, _stream()), lib)
+    return out
+
+
+def rms_norm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+             delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
+             write_h: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out = rms_norm(h[rows] + delta[rows]) * weight``; with ``write_h`` the sum replaces ``h``."""
+    lib = library.load()
+    _device_tensor(h, "residual stream", torch.float32)
+    _device_tensor(weight, "norm weight", torch.float32)
+    _need(h.dim() == 2 and weight.dim() == 1 and weight.shape[0] == h.shape[1],
+          "rms_norm weight must match the last dimension")
+    width = h.shape[1]
+    if delta is not None:
+        _device_tensor(delta, "delta", out_dtype)
+        _need(tuple(delta.shape) == tuple(h.shape), "delta must have the residual stream's shape")
+    if rows is not None:
+        _device_tensor(rows, "row selection", torch.int32)
+        _need(not write_h, "cannot write h through a row selection")
+        n_rows = rows.shape[0]
+    else:
+        n_rows = h.shape[0]
+    if out is None:
+        out = torch.empty((n_rows, width), dtype=out_dtype, device=h.device)
+    _device_tensor(out, "norm output", out_dtype)
+    _need(tuple(out.shape) == (n_rows, width), "norm output has the wrong shape")
+    _check(lib.mll_rms_norm(_ptr(h), _ptr(delta), _ptr(rows), _ptr(weight), ctypes.c_float(eps), _ptr(out),
+                            _code(out_dtype), n_rows, width, int(write_h), _stream()), lib)
+    return out
+
+
+def residual_add(h: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+    lib = library.load()
+    _device_tensor(h, "residual stream", torch.float32)
+    _device_tensor(delta, "delta")
+    _need(tuple(delta.shape) == tuple(h.shape) and h.dim() == 2, "delta must have the residual stream's shape")
+    _check(lib.mll_residual_add(_ptr(h), _ptr(delta), _code(delta.dtype), h.shape[0], h.shape[1], _stream()), lib)
+    return h
+
+
+def qkv_rope_store(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
+                   slot_mapping: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor],
+                   k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                   heads: int, kv_heads: int, head_dim: int, page_size: int,
+                   q_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Bias, rotation and page write of fused projections ``[tokens, (heads + 2 kv_heads) * head_dim]``."""
+    lib = library.load()
+    _device_tensor(qkv, "qkv")
+    n_tokens = qkv.shape[0]
+    total = (heads + 2 * kv_heads) * head_dim
+    _need(qkv.dim() == 2 and qkv.shape[1] == total, f"qkv must be [tokens, {total}]")
+    if bias is not None:
+        _device_tensor(bias, "qkv bias", torch.float32)
+        _need(tuple(bias.shape) == (total,), "qkv bias has the wrong size")
+    _device_tensor(positions, "positions", torch.int32)
+    _need(tuple(positions.shape) == (n_tokens,), "positions must hold one entry per token")
+    n_freq = 0
+    if inv_freq is not None:
+        _device_tensor(inv_freq, "inverse frequencies", torch.float64)
+        n_freq = inv_freq.shape[0]
+    if slot_mapping is not None:
+        _device_tensor(slot_mapping, "slot mapping", torch.int32)
+        _need(tuple(slot_mapping.shape) == (n_tokens,), "slot mapping must hold one entry per token")
+        _need(k_cache is not None and v_cache is not None, "slot mapping needs both caches")
+        for cache in (k_cache, v_cache):
+            _device_tensor(cache, "cache pages", qkv.dtype)
+            _need(cache.dim() == 4 and tuple(cache.shape[1:]) == (kv_heads, page_size, head_dim),
+                  "cache pages must be [pages, kv_heads, page_size, head_dim]")
+    if q_out is None:
+        q_out = torch.empty((n_tokens, heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    _device_tensor(q_out, "q output", qkv.dtype)
+    _need(tuple(q_out.shape) == (n_tokens, heads * head_dim), "q output has the wrong shape")
+    _check(lib.mll_qkv_rope_store(_ptr(qkv), _code(qkv.dtype), _ptr(bias), _ptr(positions), _ptr(slot_mapping),
+                                  _ptr(inv_freq), n_freq, _ptr(q_out), _ptr(k_cache), _ptr(v_cache),
+                                  n_tokens, heads, kv_heads, head_dim, page_size, _stream()), lib)
+    return q_out
+
+
+def _check_paged(q, k_cache, v_cache, block_table, heads, kv_heads, head_dim) -> int:
+    _device_tensor(q, "queries")
+    _need(q.dim() == 2 and q.shape[1] == heads * head_dim, "queries must be [tokens, heads * head_dim]")
+    for cache in (k_cache, v_cache):
+        _device_tensor(cache, "cache pages", q.dtype)
+        _need(cache.dim() == 4 and cache.shape[1] == kv_heads and cache.shape[3] == head_dim,
+              "cache pages must be [pages, kv_heads, page_size, head_dim]")
+    _need(k_cache.shape == v_cache.shape, "key and value pages must have one shape")
+    _device_tensor(block_table, "block table", torch.int32)
+    _need(block_table.dim() == 2, "block table must be [requests, pages]")
+    return k_cache.shape[2]
+
+
+def paged_attention_rowwise(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                            block_table: torch.Tensor, seq_of_token: torch.Tensor, positions: torch.Tensor,
+                            scale: float, window: int, heads: int, kv_heads: int, head_dim: int,
+                            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    lib = library.load()
+    page_size = _check_paged(q, k_cache, v_cache, block_table, heads, kv_heads, head_dim)
+    n_tokens = q.shape[0]
+    _device_tensor(seq_of_token, "request of token", torch.int32)
+    _device_tensor(positions, "positions", torch.int32)
+    _need(seq_of_token.shape[0] == n_tokens and positions.shape[0] == n_tokens,
+          "request-of-token and positions must hold one entry per token")
+    if out is None:
+        out = torch.empty_like(q)
+    _device_tensor(out, "attention output", q.dtype)
+    _need(out.shape == q.shape, "attention output must have the queries' shape")
+    _check(lib.mll_paged_attention_rowwise(_ptr(q), _code(q.dtype), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
+                                           block_table.shape[1], _ptr(seq_of_token), _ptr(positions), _ptr(out),
+                                           ctypes.c_float(scale), int(window), n_tokens, heads, kv_heads, head_dim,
+                                           page_size, _stream()), lib)
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``silu(gate) * up`` of fused rows ``[tokens, 2 * width]`` (gate first)."""
+    lib = library.load()
+    _device_tensor(gate_up, "gate/up")
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "gate/up must be [tokens, 2 * width]")
+    n_tokens, double = gate_up.shape
+    width = double // 2
+    if out is None:
+        out = torch.empty((n_tokens, width), dtype=gate_up.dtype, device=gate_up.device)
+    _device_tensor(out, "silu_mul output", gate_up.dtype)
+    _need(tuple(out.shape) == (n_tokens, width), "silu_mul output has the wrong shape")
+    element = gate_up.element_size()
+    for start in range(0, n_tokens, 65535):
+        count = min(65535, n_tokens - start)
+        gate_ptr = gate_up.data_ptr() + start * double * element
+        _check(lib.mll_silu_mul(ctypes.c_void_p(gate_ptr), ctypes.c_void_p(gate_ptr + width * element),
+                                ctypes.c_int64(double), ctypes.c_void_p(out.data_ptr() + start * width * element),
+                                _code(gate_up.dtype), count, width, _stream()), lib)
+    return out
+
+
+def gemm_f32(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``a @ weight.T (+ bias)`` in true float32 with a fixed order of additions per element."""
+    lib = library.load()
+    _device_tensor(a, "gemm input", torch.float32)
+    _device_tensor(weight, "gemm weight", torch.float32)
+    _need(a.dim() == 2 and weight.dim() == 2 and a.shape[1] == weight.shape[1],
+          "gemm takes [m, k] and [n, k]")
+    m, k = a.shape
+    n = weight.shape[0]
+    if bias is not None:
+        _device_tensor(bias, "gemm bias", torch.float32)
+        _need(tuple(bias.shape) == (n,), "gemm bias has the wrong size")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    _device_tensor(out, "gemm output", torch.float32)
+    _need(tuple(out.shape) == (m, n), "gemm output has the wrong shape")
+    step = 65535 * 64
+    for start in range(0, max(m, 1), step):
+        count = min(step, m - start)
+        _check(lib.mll_gemm_f32(ctypes.c_void_p(a.data_ptr() + start * k * 4), _ptr(weight), _ptr(bias),
+                                ctypes.c_void_p(out.data_ptr() + start * n * 4), count, n, k, _stream()), lib)
+    return out
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    lib = library.load()
+    _device_tensor(logits, "logits", torch.float32)
+    _need(logits.dim() == 2, "logits must be [rows, vocab]")
+    out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
+    _check(lib.mll_argmax(_ptr(logits), _ptr(out), logits.shape[0], logits.shape[1], _stream()), lib)
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: Optional[torch.Tensor],
+           uniform: torch.Tensor) -> torch.Tensor:
+    lib = library.load()
+    _device_tensor(logits, "logits", torch.float32)
+    _need(logits.dim() == 2, "logits must be [rows, vocab]")
+    rows = logits.shape[0]
+    _device_tensor(temperature, "temperature", torch.float32)
+    _device_tensor(uniform, "uniform", torch.float32)
+    _need(temperature.shape[0] == rows and uniform.shape[0] == rows, "one temperature and uniform per row")
+    if top_k is not None:
+        _device_tensor(top_k, "top_k", torch.int32)
+        _need(top_k.shape[0] == rows, "one top_k per row")
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    _check(lib.mll_sample(_ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(uniform), _ptr(out),
+                          rows, logits.shape[1], _stream()), lib)
+    return out
+
+
+def gemm_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """``x @ weight.T`` for bfloat16 operands with float32 accumulation.
+
+    The product itself is the library's (hipBLASLt through ``torch.mm``), as the
+    reference uses the library for its large linears (src/ops/optimized.cpp:94-450).
+    """
+    _device_tensor(x, "gemm input", torch.bfloat16)
+    _device_tensor(weight, "gemm weight", torch.bfloat16)
+    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "gemm takes [m, k] and [n, k]")
+    if out_dtype == torch.bfloat16:
+        return torch.mm(x, weight.t())
+    return torch.mm(x, weight.t(), out_dtype=out_dtype)
+
+
+def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, view, ctx,
+                    scale: float, window: int, heads: int, kv_heads: int, head_dim: int) -> torch.Tensor:
+    """Attention of the step's queries over their requests' pages; chooses the kernel for the batch's shape."""
+    return paged_attention_rowwise(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
+                                   scale, window, heads, kv_heads, head_dim)

@@ -1,0 +1,103 @@
+"""Grouped-query attention over paged keys and values.
+
+``q = x Wq + bq`` (likewise k, v), rotation of q and k after the bias, scores
+``(q . k_j) * scale`` over the visible keys, softmax in float32, ``o = sum p_j v_j``,
+then the output projection without bias (src/model/model.cpp:472-520;
+src/ops/ops.cpp:2348-2383). Query head ``h`` uses kv head ``h // (heads / kv_heads)``.
+With a window ``W`` key ``j`` is visible to a query at ``p`` iff ``j <= p`` and
+``p - j < W``; the reference has no window (src/model/huggingface.cpp:159-161).
+The three projections are stacked into one weight at bind time.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Mapping, Optional
+
+import torch
+
+from ..ops import kernels
+from .base import MATRIX, Mixer, PagedKVNeed, Runtime, TensorDecl, VECTOR
+from .linear import linear
+from .registry import build_part, register_part
+from .spec import PartSpec
+
+
+class PagedAttention(Mixer):
+    def __init__(self, spec: PartSpec, runtime: Runtime):
+        super().__init__(spec, runtime)
+        p = spec.params
+        self.hidden = int(p["hidden_size"])
+        self.heads = int(p["num_heads"])
+        self.kv_heads = int(p["num_kv_heads"])
+        self.head_dim = int(p["head_dim"])
+        self.qkv_bias = bool(p.get("qkv_bias", False))
+        self.window = p.get("window")
+        self.scale = float(p.get("scale", 1.0 / math.sqrt(self.head_dim)))
+        self.owns_kv = bool(p.get("owns_kv", True))  # False: only q is projected, another entry's pages are read
+        if self.heads % self.kv_heads != 0:
+            raise ValueError("num_heads must divide into num_kv_heads groups")
+        position = p.get("position")
+        self.position = build_part("position", position, runtime) if position is not None else None
+        self.qkv_weight: Optional[torch.Tensor] = None
+        self.qkv_bias_vector: Optional[torch.Tensor] = None
+        self.o_weight: Optional[torch.Tensor] = None
+
+    # ---- tensors -------------------------------------------------------------------------
+    def _projections(self):
+        out = [("q", self.heads * self.head_dim)]
+        if self.owns_kv:
+            out += [("k", self.kv_heads * self.head_dim), ("v", self.kv_heads * self.head_dim)]
+        return out
+
+    def tensors(self) -> Dict[str, TensorDecl]:
+        decls = {}
+        for role, width in self._projections():
+            decls[self.name(f"{role}_proj.weight")] = TensorDecl((width, self.hidden), MATRIX)
+            if self.qkv_bias:
+                decls[self.name(f"{role}_proj.bias")] = TensorDecl((width,), VECTOR)
+        decls[self.name("o_proj.weight")] = TensorDecl((self.hidden, self.heads * self.head_dim), MATRIX)
+        return decls
+
+    def bind(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        weights = [tensors[self.name(f"{role}_proj.weight")] for role, _ in self._projections()]
+        if len({w.dtype for w in weights}) != 1:
+            raise TypeError("the q, k and v weights of one layer must share a dtype to be stacked")
+        self.qkv_weight = torch.cat(weights, dim=0).contiguous() if len(weights) > 1 else weights[0]
+        if self.qkv_bias:
+            biases = [tensors[self.name(f"{role}_proj.bias")] for role, _ in self._projections()]
+            self.qkv_bias_vector = torch.cat(biases, dim=0).contiguous() if len(biases) > 1 else biases[0]
+        self.o_weight = tensors[self.name("o_proj.weight")]
+
+    def cache_need(self):
+        if not self.owns_kv:
+            return None
+        return PagedKVNeed(self.kv_heads, self.head_dim, self.window)
+
+    # ---- forward -------------------------------------------------------------------------
+    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+        view = ctx.paged[cache.group]
+        kv_heads = cache.need.kv_heads
+        qkv = linear(x, self.qkv_weight)
+        stored_heads = self.kv_heads if self.owns_kv else 0
+        slot_mapping = view.slot_mapping if self.owns_kv else None
+        k_pages = cache.k if self.owns_kv else None
+        v_pages = cache.v if self.owns_kv else None
+        bias = self.qkv_bias_vector
+        inv_freq = None
+        if self.position is not None:
+            if self.position.fused_split_half:
+                inv_freq = self.position.inv_freq
+            else:
+                if bias is not None:
+                    qkv = (qkv.float() + bias).to(qkv.dtype)
+                    bias = None
+                qkv = self.position.apply(qkv, ctx.positions, self.heads, stored_heads, self.head_dim).contiguous()
+        q = kernels.qkv_rope_store(qkv, bias, ctx.positions, slot_mapping, inv_freq, k_pages, v_pages,
+                                   self.heads, stored_heads, self.head_dim, view.page_size)
+        window = int(self.window) if self.window else 0
+        o = kernels.paged_attention(q, cache.k, cache.v, view, ctx, self.scale, window,
+                                    self.heads, kv_heads, self.head_dim)
+        return linear(o, self.o_weight)
+
+
+register_part("mixer", "paged_attention", PagedAttention)

@@ -1,0 +1,108 @@
+"""What every part is: sizes and constants in, tensor declarations out, one forward.
+
+A part is built from a ``PartSpec`` and a ``Runtime`` and knows nothing of the
+model it sits in: its sizes, constants and the names of its tensors all come
+with the spec. Categories are ``norm``, ``position``, ``mixer``, ``ffn``,
+``block``, ``embedding`` and ``head``; each has a registry in ``parts.registry``.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, Mapping, Optional, Tuple, Union
+
+import torch
+
+from .spec import PartSpec
+
+MATRIX = "matrix"   # a float matrix or table: float32 stays float32, bfloat16 stays bfloat16 in a bfloat16 engine
+VECTOR = "vector"   # a float vector read by kernels as float32 (norm weights, biases)
+INT_TABLE = "int_table"  # integers, held as int32
+
+
+@dataclass(frozen=True)
+class TensorDecl:
+    shape: Tuple[int, ...]
+    kind: str = MATRIX
+
+
+@dataclass(frozen=True)
+class Runtime:
+    """What a part needs of the engine: the element type of activations and pages, and the device."""
+    dtype: torch.dtype
+    device: torch.device
+
+
+@dataclass(frozen=True)
+class PagedKVNeed:
+    """Keys and values in pages; ``window`` is None when every key stays needed."""
+    kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Per-request state of fixed size: one slot of ``shape`` and ``dtype`` per live request."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+CacheNeed = Union[PagedKVNeed, StateNeed, None]
+
+
+class Part:
+    category = "part"
+
+    def __init__(self, spec: PartSpec, runtime: Runtime):
+        self.spec = spec
+        self.runtime = runtime
+
+    def tensors(self) -> Dict[str, TensorDecl]:
+        """File name of every tensor this part needs, with its shape and kind."""
+        return {}
+
+    def bind(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        """Take the loaded tensors (by file name); called once, before the first forward."""
+
+    def name(self, role: str) -> str:
+        try:
+            return self.spec.names[role]
+        except KeyError:
+            raise KeyError(f"{type(self).__name__} needs a tensor name for {role!r}") from None
+
+
+class Mixer(Part):
+    """Mixes information between the positions of one request (attention, or a layer with state)."""
+    category = "mixer"
+
+    def cache_need(self) -> CacheNeed:
+        return None
+
+    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:  # [tokens, hidden] -> [tokens, hidden]
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    category = "ffn"
+
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Norm(Part):
+    category = "norm"
+
+    def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor] = None, write_h: bool = True,
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Normalise ``h + delta`` (float32 residual stream); with ``write_h`` the sum replaces ``h``."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    category = "position"
+    fused_split_half = False  # True: the mixer's fused kernel applies it from ``inv_freq``
+
+    def apply(self, qkv: torch.Tensor, positions: torch.Tensor, heads: int, kv_heads: int,
+              head_dim: int) -> torch.Tensor:
+        """Encode positions into the q and k parts of fused projections ``[tokens, (heads + 2 kv) * hd]``."""
+        raise NotImplementedError

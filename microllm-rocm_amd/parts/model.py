@@ -1,0 +1,123 @@
+"""The model a ``ModelSpec`` describes: embedding, layers run in the spec's order, final norm, head.
+
+Nothing here names an architecture. The run order is data: an entry names a
+layer (perhaps one that an earlier entry named too) and either owns a cache or
+reads an earlier entry's. Logits are computed in float32 for the wanted rows only
+(the reference projects the last row only, src/model/model.cpp:1118-1128).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Mapping, Optional
+
+import torch
+
+from ..ops import kernels
+from .base import CacheNeed, MATRIX, Part, Runtime, TensorDecl
+from .block import Block, build_block
+from .linear import linear
+from .registry import build_part, register_part
+from .spec import ModelSpec, PartSpec
+
+
+class TokenEmbedding(Part):
+    """``h0[t] = E[id_t]`` widened to float32 (src/model/model.cpp:1111)."""
+    category = "embedding"
+
+    def __init__(self, spec: PartSpec, runtime: Runtime):
+        super().__init__(spec, runtime)
+        self.vocab = int(spec.params["vocab_size"])
+        self.width = int(spec.params["hidden_size"])
+        self.table: Optional[torch.Tensor] = None
+
+    def tensors(self):
+        return {self.name("weight"): TensorDecl((self.vocab, self.width), MATRIX)}
+
+    def bind(self, tensors):
+        self.table = tensors[self.name("weight")]
+
+    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+        return kernels.embedding(self.table, ids)
+
+
+class LMHead(Part):
+    """``logits = x W^T`` in float32; a tied head names the embedding's table as its weight
+    (src/model/model.cpp:1121-1128)."""
+    category = "head"
+
+    def __init__(self, spec: PartSpec, runtime: Runtime):
+        super().__init__(spec, runtime)
+        self.vocab = int(spec.params["vocab_size"])
+        self.width = int(spec.params["hidden_size"])
+        self.weight: Optional[torch.Tensor] = None
+
+    def tensors(self):
+        return {self.name("weight"): TensorDecl((self.vocab, self.width), MATRIX)}
+
+    def bind(self, tensors):
+        self.weight = tensors[self.name("weight")]
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return linear(x, self.weight, out_dtype=torch.float32)
+
+
+register_part("embedding", "token_embedding", TokenEmbedding)
+register_part("head", "lm_head", LMHead)
+
+
+class Model:
+    def __init__(self, spec: ModelSpec, runtime: Runtime):
+        spec.validate()
+        self.spec = spec
+        self.runtime = runtime
+        self.embedding = build_part("embedding", spec.embedding, runtime)
+        self.blocks: List[Block] = [build_block(layer, runtime) for layer in spec.layers]
+        self.final_norm = build_part("norm", spec.final_norm, runtime)
+        self.head = build_part("head", spec.head, runtime)
+
+    # ---- tensors -------------------------------------------------------------------------
+    def tensors(self) -> Dict[str, TensorDecl]:
+        decls: Dict[str, TensorDecl] = {}
+
+        def add(new: Mapping[str, TensorDecl]) -> None:
+            for name, decl in new.items():
+                if name in decls and decls[name] != decl:
+                    raise ValueError(f"tensor {name!r} is declared twice with different shapes or kinds")
+                decls[name] = decl
+
+        add(self.embedding.tensors())
+        for block in self.blocks:
+            add(block.tensors())
+        add(self.final_norm.tensors())
+        add(self.head.tensors())
+        return decls
+
+    def bind(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.embedding.bind(tensors)
+        for block in self.blocks:
+            block.bind(tensors)
+        self.final_norm.bind(tensors)
+        self.head.bind(tensors)
+
+    def cache_needs(self) -> List[CacheNeed]:
+        """The cache need of every run entry; None for an entry that owns none."""
+        needs: List[CacheNeed] = []
+        for entry in self.spec.order:
+            need = self.blocks[entry.layer].mixer.cache_need()
+            needs.append(None if entry.reads_cache_of is not None else need)
+        return needs
+
+    # ---- forward -------------------------------------------------------------------------
+    def forward(self, ctx, caches, want_rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+        """Run the step's tokens through every entry; logits ``[wanted, vocab]`` in float32.
+
+        ``caches[i]`` is the cache binding of run entry ``i`` (its own, or the one it reads).
+        ``want_rows`` indexes the step's flat token list; None or empty skips the head.
+        """
+        h = self.embedding.forward(ctx.tokens)
+        pending = None
+        for index, entry in enumerate(self.spec.order):
+            pending = self.blocks[entry.layer].forward(h, pending, ctx, caches[index])
+        if want_rows is None or want_rows.numel() == 0:
+            return None
+        x = self.final_norm.forward(h, delta=pending, write_h=False, rows=want_rows)
+        return self.head.forward(x)
