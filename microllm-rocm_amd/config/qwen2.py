@@ -127,7 +127,7 @@ class Qwen2Config:
                 if kind not in (FULL_ATTENTION, SLIDING_ATTENTION):
                     raise ConfigError(f"unknown layer type {kind!r}")
         windowed = any(window is not None for window in self.layer_windows())
-        if windowed:
+        if windowed or self.use_sliding_window:
             if self.sliding_window is None or self.sliding_window <= 0:
                 raise ConfigError("sliding_window must be positive when a layer uses the window")
         if self.use_sliding_window and self.layer_types is None:

@@ -30,15 +30,15 @@ __global__ void embedding_kernel(const W* __restrict__ table, const int32_t* __r
 // ---------------------------------------------------------------------------------------------
 // One block per output row. The sum of squares is taken in float32: per-thread strided partial
 // sums, a butterfly inside each wave, then the waves in ascending order.
-template <typename T>
-__global__ void rms_norm_kernel(float* __restrict__ h, const T* __restrict__ delta,
+template <typename T, typename D>
+__global__ void rms_norm_kernel(float* __restrict__ h, const D* __restrict__ delta,
                                 const int32_t* __restrict__ rows, const float* __restrict__ weight,
                                 float eps, T* __restrict__ out, int width, int write_h) {
     __shared__ float scratch[16];
     const int index = blockIdx.x;
     const int64_t source = rows ? rows[index] : index;
     float* h_row = h + source * width;
-    const T* delta_row = delta ? delta + source * width : nullptr;
+    const D* delta_row = delta ? delta + source * width : nullptr;
     T* out_row = out + static_cast<int64_t>(index) * width;
 
     float partial = 0.0f;
@@ -69,8 +69,8 @@ __global__ void residual_add_kernel(float* __restrict__ h, const T* __restrict__
 // and shared by all heads.
 constexpr int kMaxHeadDim = 512;
 
-template <typename T>
-__global__ void qkv_rope_store_kernel(const T* __restrict__ qkv, const float* __restrict__ bias,
+template <typename In, typename T>
+__global__ void qkv_rope_store_kernel(const In* __restrict__ qkv, const float* __restrict__ bias,
                                       const int32_t* __restrict__ positions,
                                       const int32_t* __restrict__ slot_mapping,
                                       const double* __restrict__ inv_freq, int n_freq,
@@ -177,21 +177,24 @@ int mll_embedding(const void* table, int table_dtype, const int32_t* ids, float*
     return check_launch("embedding");
 }
 
-int mll_rms_norm(float* h, const void* delta, const int32_t* rows, const float* weight, float eps,
+int mll_rms_norm(float* h, const void* delta, int delta_dtype, const int32_t* rows, const float* weight, float eps,
                  void* out, int dtype, int n_rows, int width, int write_h, hipStream_t stream) {
     MLL_REQUIRE(n_rows >= 0 && width > 0, "rms_norm: sizes must be positive");
     MLL_REQUIRE(eps > 0.0f, "rms_norm: eps must be positive");
     MLL_REQUIRE(!(write_h && rows), "rms_norm: cannot write h through a row selection");
     if (n_rows == 0) return 0;
     const int threads = width >= 2048 ? 512 : 256;
-    if (dtype == kF32) {
-        rms_norm_kernel<float><<<n_rows, threads, 0, stream>>>(h, static_cast<const float*>(delta), rows, weight, eps,
-                                                               static_cast<float*>(out), width, write_h);
-    } else if (dtype == kBF16) {
-        rms_norm_kernel<bf16><<<n_rows, threads, 0, stream>>>(h, static_cast<const bf16*>(delta), rows, weight, eps,
-                                                              static_cast<bf16*>(out), width, write_h);
+    if (dtype == kF32 && delta_dtype == kF32) {
+        rms_norm_kernel<float, float><<<n_rows, threads, 0, stream>>>(
+            h, static_cast<const float*>(delta), rows, weight, eps, static_cast<float*>(out), width, write_h);
+    } else if (dtype == kBF16 && delta_dtype == kF32) {
+        rms_norm_kernel<bf16, float><<<n_rows, threads, 0, stream>>>(
+            h, static_cast<const float*>(delta), rows, weight, eps, static_cast<bf16*>(out), width, write_h);
+    } else if (dtype == kBF16 && delta_dtype == kBF16) {
+        rms_norm_kernel<bf16, bf16><<<n_rows, threads, 0, stream>>>(
+            h, static_cast<const bf16*>(delta), rows, weight, eps, static_cast<bf16*>(out), width, write_h);
     } else {
-        return fail("rms_norm: unknown dtype");
+        return fail("rms_norm: unsupported combination of output and delta dtypes");
     }
     return check_launch("rms_norm");
 }
@@ -210,7 +213,7 @@ int mll_residual_add(float* h, const void* delta, int dtype, int n_rows, int wid
     return check_launch("residual_add");
 }
 
-int mll_qkv_rope_store(const void* qkv, int dtype, const float* bias, const int32_t* positions,
+int mll_qkv_rope_store(const void* qkv, int in_dtype, int dtype, const float* bias, const int32_t* positions,
                        const int32_t* slot_mapping, const double* inv_freq, int n_freq,
                        void* q_out, void* k_cache, void* v_cache,
                        int n_tokens, int heads, int kv_heads, int head_dim, int page_size,
@@ -222,18 +225,23 @@ int mll_qkv_rope_store(const void* qkv, int dtype, const float* bias, const int3
     MLL_REQUIRE(slot_mapping == nullptr || (k_cache && v_cache && page_size > 0),
                 "qkv_rope_store: slot_mapping needs both caches and a page size");
     if (n_tokens == 0) return 0;
-    if (dtype == kF32) {
-        qkv_rope_store_kernel<float><<<n_tokens, 256, 0, stream>>>(
+    if (dtype == kF32 && in_dtype == kF32) {
+        qkv_rope_store_kernel<float, float><<<n_tokens, 256, 0, stream>>>(
             static_cast<const float*>(qkv), bias, positions, slot_mapping, inv_freq, n_freq,
             static_cast<float*>(q_out), static_cast<float*>(k_cache), static_cast<float*>(v_cache),
             heads, kv_heads, head_dim, page_size);
-    } else if (dtype == kBF16) {
-        qkv_rope_store_kernel<bf16><<<n_tokens, 256, 0, stream>>>(
+    } else if (dtype == kBF16 && in_dtype == kF32) {
+        qkv_rope_store_kernel<float, bf16><<<n_tokens, 256, 0, stream>>>(
+            static_cast<const float*>(qkv), bias, positions, slot_mapping, inv_freq, n_freq,
+            static_cast<bf16*>(q_out), static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache),
+            heads, kv_heads, head_dim, page_size);
+    } else if (dtype == kBF16 && in_dtype == kBF16) {
+        qkv_rope_store_kernel<bf16, bf16><<<n_tokens, 256, 0, stream>>>(
             static_cast<const bf16*>(qkv), bias, positions, slot_mapping, inv_freq, n_freq,
             static_cast<bf16*>(q_out), static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache),
             heads, kv_heads, head_dim, page_size);
     } else {
-        return fail("qkv_rope_store: unknown dtype");
+        return fail("qkv_rope_store: unsupported combination of input and output dtypes");
     }
     return check_launch("qkv_rope_store");
 }

@@ -19,8 +19,9 @@ int mll_embedding(const void* table, int table_dtype, const int32_t* ids, float*
 
 // For i < n_rows, r = rows ? rows[i] : i:  v = h[r] + (delta ? delta[r] : 0);
 // if write_h, h[r] = v;  out[i] = v * rsqrt(mean(v^2) + eps) * weight.
-// h is the float32 residual stream; delta and out have element type `dtype`.
-int mll_rms_norm(float* h, const void* delta, const int32_t* rows, const float* weight, float eps,
+// h is the float32 residual stream; out has element type `dtype`, delta `delta_dtype`
+// (float32, or the same as out).
+int mll_rms_norm(float* h, const void* delta, int delta_dtype, const int32_t* rows, const float* weight, float eps,
                  void* out, int dtype, int n_rows, int width, int write_h, hipStream_t stream);
 
 // Adds a pending delta into the residual stream: h[r] += delta[r] for all rows.
@@ -30,8 +31,9 @@ int mll_residual_add(float* h, const void* delta, int dtype, int n_rows, int wid
 // rotates q and k by the split-half rule with angle position * inv_freq[i] in float64 (inv_freq nullable:
 // no rotation; rotary_dim = 2 * n_freq <= hd), writes q to q_out[t] and k, v into the pages:
 // slot = slot_mapping[t] (negative: not stored) addresses [page, kv_head, offset, :] with
-// page = slot / page_size.  k_cache / v_cache nullable together with slot_mapping.
-int mll_qkv_rope_store(const void* qkv, int dtype, const float* bias, const int32_t* positions,
+// page = slot / page_size.  k_cache / v_cache nullable together with slot_mapping. qkv has element type
+// `in_dtype` (float32, or the same as `dtype`); q_out and the pages have `dtype`.
+int mll_qkv_rope_store(const void* qkv, int in_dtype, int dtype, const float* bias, const int32_t* positions,
                        const int32_t* slot_mapping, const double* inv_freq, int n_freq,
                        void* q_out, void* k_cache, void* v_cache,
                        int n_tokens, int heads, int kv_heads, int head_dim, int page_size,

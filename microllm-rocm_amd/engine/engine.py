@@ -103,8 +103,11 @@ class Engine:
         return request_id in self.cache.requests
 
     # ---- the step ------------------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
-        """Run one batch; returns float32 logits ``[wanted, vocab]`` in the order of entries and of ``want``."""
+    def step(self, entries: Sequence[StepEntry], reserved: bool = False) -> Optional[torch.Tensor]:
+        """Run one batch; returns float32 logits ``[wanted, vocab]`` in the order of entries and of ``want``.
+
+        With ``reserved`` the caller (a scheduler) has already taken the pages for every portion.
+        """
         entries = [entry if isinstance(entry, StepEntry) else StepEntry(*entry) for entry in entries]
         if not entries:
             return None
@@ -127,15 +130,20 @@ class Engine:
                 if not 0 <= place < count:
                     raise ValueError(f"wanted place {place} of request {entry.request_id!r} is outside its {count} tokens")
             requests.append(request)
-        reserved: List[RequestCache] = []
-        try:
+        if reserved:
             for request, entry in zip(requests, entries):
-                self.cache.reserve(request, len(entry.tokens))
-                reserved.append(request)
-        except OutOfPages:
-            for request in reserved:
-                self.cache.cancel_reservation(request)
-            raise
+                if request.reserved < len(entry.tokens):
+                    raise ValueError(f"request {entry.request_id!r} has no pages reserved for its portion")
+        else:
+            taken: List[RequestCache] = []
+            try:
+                for request, entry in zip(requests, entries):
+                    self.cache.reserve(request, len(entry.tokens))
+                    taken.append(request)
+            except OutOfPages:
+                for request in taken:
+                    self.cache.cancel_reservation(request)
+                raise
         ctx = self._builder.build(requests, [entry.tokens for entry in entries], [entry.want for entry in entries])
         logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
         for request, entry in zip(requests, entries):

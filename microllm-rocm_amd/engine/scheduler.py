@@ -1,0 +1,316 @@
+"""Continuous batching above the step function.
+
+Each scheduler step builds one batch: every running request that is decoding
+brings its one token, requests still in their prompt bring a portion of it, and
+waiting requests are admitted first come first served while the step's token
+budget, the request slots and the free pages allow. A request whose portion ends
+its known tokens gets logits, a token is selected, and it finishes on a stop
+token or at its length. States and reasons are the reference's
+(include/microllm/inference/scheduler.h:15-27); its continuous scheduler
+(src/inference/scheduler.cpp:464-1069) prefills whole prompts of equal length
+into fixed slots and reserves capacity up front, so it has neither a token budget
+nor a way to run out of cache.
+
+When pages run out: the running request that was admitted last is preempted. Its
+pages and slot go back, it returns to the head of the waiting queue, and when it
+is admitted again its prompt and the tokens it had generated are run again in
+portions (recomputation); sampling draws are indexed by the number of generated
+tokens, so it continues with the same stream. A request that is alone and still
+cannot get pages would never fit; ``submit`` refuses such a request.
+"""
+from __future__ import annotations
+
+import enum
+import time
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Deque, Dict, Hashable, List, Optional, Sequence
+
+from ..cache.pages import OutOfPages
+from ..sampling import Sampler, SamplingParams
+from .batch import StepEntry
+
+
+class RequestState(enum.Enum):
+    PENDING_PREFILL = "pending_prefill"   # waiting, or admitted and still inside its known tokens
+    DECODING = "decoding"
+    COMPLETED = "completed"
+    CANCELLED = "cancelled"
+
+
+class CompletionReason(enum.Enum):
+    NONE = "none"
+    LENGTH = "length"
+    STOP_TOKEN = "stop_token"
+    CANCELLED = "cancelled"
+
+
+@dataclass
+class Request:
+    id: int
+    prompt: List[int]
+    params: SamplingParams
+    arrival_step: int
+    state: RequestState = RequestState.PENDING_PREFILL
+    completion_reason: CompletionReason = CompletionReason.NONE
+    generated: List[int] = field(default_factory=list)
+    computed: int = 0            # tokens of prompt + generated whose keys and values are in the cache
+    admitted: bool = False
+    admission_order: int = -1
+    completion_step: int = -1
+    preemptions: int = 0
+    submit_time: float = 0.0
+    first_token_time: float = -1.0
+    completion_time: float = -1.0
+
+    @property
+    def known(self) -> int:
+        return len(self.prompt) + len(self.generated)
+
+    def token_at(self, index: int) -> int:
+        return self.prompt[index] if index < len(self.prompt) else self.generated[index - len(self.prompt)]
+
+    @property
+    def terminal(self) -> bool:
+        return self.state in (RequestState.COMPLETED, RequestState.CANCELLED)
+
+
+@dataclass
+class SchedulerMetrics:
+    scheduler_steps: int = 0
+    submitted_requests: int = 0
+    completed_requests: int = 0
+    cancelled_requests: int = 0
+    stop_completed_requests: int = 0
+    admissions: int = 0
+    preemptions: int = 0
+    prefill_tokens: int = 0
+    decode_tokens: int = 0
+    batched_tokens: int = 0
+    engine_steps: int = 0
+    peak_active_requests: int = 0
+    peak_held_pages: int = 0
+
+
+@dataclass
+class Portion:
+    """What one request brings to a step."""
+    request: Request
+    start: int
+    count: int
+    wants_logits: bool
+
+
+class Scheduler:
+    def __init__(self, engine, max_batched_tokens: int = 2048, prefill_chunk: int = 512,
+                 max_requests: Optional[int] = None, sampler: Optional[Sampler] = None):
+        if max_batched_tokens <= 0 or prefill_chunk <= 0:
+            raise ValueError("max_batched_tokens and prefill_chunk must be positive")
+        self.engine = engine
+        self.cache = engine.cache
+        self.max_batched_tokens = max_batched_tokens
+        self.prefill_chunk = prefill_chunk
+        self.max_requests = min(max_requests or self.cache.max_requests, self.cache.max_requests)
+        self.sampler = sampler or Sampler()
+        self.requests: Dict[int, Request] = {}
+        self.waiting: Deque[Request] = deque()
+        self.running: List[Request] = []     # in admission order
+        self.metrics = SchedulerMetrics()
+        self.current_step = 0
+        self._next_id = 0
+        self._admissions = 0
+
+    # ---- submitting ----------------------------------------------------------------------
+    def submit(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
+               arrival_step: Optional[int] = None) -> int:
+        params = params or SamplingParams()
+        vocab = self.engine.spec.vocab_size
+        params.validate(vocab)
+        prompt = [int(token) for token in prompt]
+        if not prompt:
+            raise ValueError("a prompt needs at least one token")
+        for token in prompt:
+            if not 0 <= token < vocab:
+                raise ValueError(f"prompt token {token} is outside the vocabulary")
+        total = len(prompt) + params.max_new_tokens
+        if total > self.engine.spec.max_positions:
+            raise ValueError(f"prompt plus max_new_tokens is {total}, beyond max positions {self.engine.spec.max_positions}")
+        for group in self.cache.groups:
+            if self.cache.blocks_for(total) > group.pool.num_pages:
+                raise ValueError(f"prompt plus max_new_tokens is {total} tokens, more than the cache holds "
+                                 f"({group.pool.num_pages * self.cache.page_size})")
+        request = Request(self._next_id, prompt, params, arrival_step if arrival_step is not None else self.current_step,
+                          submit_time=time.perf_counter())
+        self._next_id += 1
+        self.requests[request.id] = request
+        self.metrics.submitted_requests += 1
+        if params.max_new_tokens == 0:   # completes at once, src/inference/scheduler.cpp:876-881
+            self._finish(request, CompletionReason.LENGTH)
+        else:
+            self.waiting.append(request)
+        return request.id
+
+    def cancel(self, request_id: int) -> bool:
+        """Terminal and idempotent: False when the request had already ended (src/inference/scheduler.cpp:885-896)."""
+        if request_id not in self.requests:
+            raise KeyError(f"unknown request {request_id}")
+        request = self.requests[request_id]
+        if request.terminal:
+            return False
+        if request in self.running:
+            self.running.remove(request)
+            self._release(request)
+        else:
+            self.waiting.remove(request)
+        request.state = RequestState.CANCELLED
+        request.completion_reason = CompletionReason.CANCELLED
+        request.completion_step = self.current_step
+        request.completion_time = time.perf_counter()
+        self.metrics.cancelled_requests += 1
+        return True
+
+    # ---- one step ------------------------------------------------------------------------
+    def has_work(self) -> bool:
+        return bool(self.running or self.waiting)
+
+    def plan(self) -> List[Portion]:
+        """Decide what this step runs. Takes pages (a reservation per portion); may preempt."""
+        budget = self.max_batched_tokens
+        portions: List[Portion] = []
+
+        def portion_of(request: Request, budget_left: int) -> int:
+            remaining = request.known - request.computed
+            return min(remaining, self.prefill_chunk if remaining > 1 else 1, budget_left)
+
+        # Running requests first: decodes, then prompts that are under way, each in admission order.
+        ordered = sorted(self.running, key=lambda r: (r.known - r.computed > 1, r.admission_order))
+        for request in ordered:
+            if request not in self.running:      # preempted while an earlier one was placed
+                continue
+            if budget <= 0:
+                break
+            count = portion_of(request, budget)
+            while True:
+                try:
+                    self.cache.reserve(self.cache.get(request.id), count)
+                    break
+                except OutOfPages:
+                    victim = self.running[-1]
+                    was_planned = [p for p in portions if p.request is victim]
+                    for planned in was_planned:
+                        portions.remove(planned)
+                        budget += planned.count
+                    self._preempt(victim)
+                    if victim is request:
+                        count = 0
+                        break
+            if count > 0:
+                portions.append(Portion(request, request.computed, count, request.computed + count == request.known))
+                budget -= count
+
+        # Then admissions, first come first served; a request that does not fit stops the queue.
+        while self.waiting and budget > 0 and len(self.running) < self.max_requests:
+            request = self.waiting[0]
+            if request.arrival_step > self.current_step:
+                break
+            count = portion_of(request, budget)
+            handle = self.cache.open(request.id)
+            try:
+                self.cache.reserve(handle, count)
+            except OutOfPages:
+                self.cache.close(request.id)
+                break
+            self.waiting.popleft()
+            request.admitted = True
+            request.admission_order = self._admissions
+            self._admissions += 1
+            self.metrics.admissions += 1
+            self.running.append(request)
+            portions.append(Portion(request, request.computed, count, request.computed + count == request.known))
+            budget -= count
+        return portions
+
+    def step(self) -> List[int]:
+        """Run one batch; returns the ids of requests that got a token in this step."""
+        portions = self.plan()
+        self.metrics.scheduler_steps += 1
+        self.metrics.peak_active_requests = max(self.metrics.peak_active_requests, len(self.running))
+        if self.cache.groups:
+            self.metrics.peak_held_pages = max(self.metrics.peak_held_pages, max(self.cache.held_pages()))
+        produced: List[int] = []
+        if portions:
+            entries = []
+            for portion in portions:
+                request = portion.request
+                tokens = [request.token_at(index) for index in range(portion.start, portion.start + portion.count)]
+                entries.append(StepEntry(request.id, tokens, [portion.count - 1] if portion.wants_logits else []))
+                if portion.count == 1 and request.state == RequestState.DECODING:
+                    self.metrics.decode_tokens += 1
+                else:
+                    self.metrics.prefill_tokens += portion.count
+                self.metrics.batched_tokens += portion.count
+            logits = self.engine.step(entries, reserved=True)
+            self.metrics.engine_steps += 1
+            for portion in portions:
+                portion.request.computed += portion.count
+            wanting = [portion.request for portion in portions if portion.wants_logits]
+            if wanting:
+                tokens = self.sampler.select(logits, [r.params for r in wanting], [len(r.generated) for r in wanting])
+                now = time.perf_counter()
+                for request, token in zip(wanting, tokens):
+                    request.generated.append(int(token))
+                    request.state = RequestState.DECODING
+                    if request.first_token_time < 0:
+                        request.first_token_time = now
+                    produced.append(request.id)
+                    if int(token) in request.params.stop_tokens:      # emitted, then stop
+                        self._complete(request, CompletionReason.STOP_TOKEN)
+                    elif len(request.generated) >= request.params.max_new_tokens:
+                        self._complete(request, CompletionReason.LENGTH)
+        self.current_step += 1
+        return produced
+
+    def run_until_idle(self, maximum_steps: int = -1) -> None:
+        """Step until nothing runs or waits; more than ``maximum_steps`` is an error
+        (src/inference/scheduler.cpp:1002-1005)."""
+        steps = 0
+        while self.has_work():
+            if 0 <= maximum_steps <= steps:
+                raise RuntimeError(f"scheduler did not become idle within {maximum_steps} steps")
+            self.step()
+            steps += 1
+
+    # ---- endings -------------------------------------------------------------------------
+    def _release(self, request: Request) -> None:
+        if self.cache.requests.get(request.id) is not None:
+            self.cache.close(request.id)
+
+    def _preempt(self, request: Request) -> None:
+        self.running.remove(request)
+        self._release(request)
+        request.computed = 0
+        request.admitted = False
+        request.preemptions += 1
+        request.state = RequestState.PENDING_PREFILL
+        self.metrics.preemptions += 1
+        self.waiting.appendleft(request)
+
+    def _complete(self, request: Request, reason: CompletionReason) -> None:
+        self.running.remove(request)
+        self._release(request)
+        self._finish(request, reason)
+
+    def _finish(self, request: Request, reason: CompletionReason) -> None:
+        request.state = RequestState.COMPLETED
+        request.completion_reason = reason
+        request.completion_step = self.current_step
+        request.completion_time = time.perf_counter()
+        self.metrics.completed_requests += 1
+        if reason == CompletionReason.STOP_TOKEN:
+            self.metrics.stop_completed_requests += 1
+
+    # ---- looking -------------------------------------------------------------------------
+    def request(self, request_id: int) -> Request:
+        if request_id not in self.requests:
+            raise KeyError(f"unknown request {request_id}")
+        return self.requests[request_id]

@@ -74,9 +74,12 @@ def rms_norm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch
     _need(h.dim() == 2 and weight.dim() == 1 and weight.shape[0] == h.shape[1],
           "rms_norm weight must match the last dimension")
     width = h.shape[1]
+    delta_code = F32
     if delta is not None:
-        _device_tensor(delta, "delta", out_dtype)
+        _device_tensor(delta, "delta")
+        _need(delta.dtype in (torch.float32, out_dtype), "delta must be float32 or have the output's dtype")
         _need(tuple(delta.shape) == tuple(h.shape), "delta must have the residual stream's shape")
+        delta_code = _code(delta.dtype)
     if rows is not None:
         _device_tensor(rows, "row selection", torch.int32)
         _need(not write_h, "cannot write h through a row selection")
@@ -87,7 +90,7 @@ def rms_norm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch
         out = torch.empty((n_rows, width), dtype=out_dtype, device=h.device)
     _device_tensor(out, "norm output", out_dtype)
     _need(tuple(out.shape) == (n_rows, width), "norm output has the wrong shape")
-    _check(lib.mll_rms_norm(_ptr(h), _ptr(delta), _ptr(rows), _ptr(weight), ctypes.c_float(eps), _ptr(out),
+    _check(lib.mll_rms_norm(_ptr(h), _ptr(delta), delta_code, _ptr(rows), _ptr(weight), ctypes.c_float(eps), _ptr(out),
                             _code(out_dtype), n_rows, width, int(write_h), _stream()), lib)
     return out
 
@@ -104,11 +107,14 @@ def residual_add(h: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
 def qkv_rope_store(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
                    slot_mapping: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor],
                    k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                   heads: int, kv_heads: int, head_dim: int, page_size: int,
+                   heads: int, kv_heads: int, head_dim: int, page_size: int, out_dtype: torch.dtype,
                    q_out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Bias, rotation and page write of fused projections ``[tokens, (heads + 2 kv_heads) * head_dim]``."""
+    """Bias, rotation and page write of fused projections ``[tokens, (heads + 2 kv_heads) * head_dim]``.
+
+    ``qkv`` is float32 or ``out_dtype``; the rotated queries and the pages have ``out_dtype``."""
     lib = library.load()
     _device_tensor(qkv, "qkv")
+    _need(qkv.dtype in (torch.float32, out_dtype), "qkv must be float32 or have the output's dtype")
     n_tokens = qkv.shape[0]
     total = (heads + 2 * kv_heads) * head_dim
     _need(qkv.dim() == 2 and qkv.shape[1] == total, f"qkv must be [tokens, {total}]")
@@ -126,14 +132,14 @@ def qkv_rope_store(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: t
         _need(tuple(slot_mapping.shape) == (n_tokens,), "slot mapping must hold one entry per token")
         _need(k_cache is not None and v_cache is not None, "slot mapping needs both caches")
         for cache in (k_cache, v_cache):
-            _device_tensor(cache, "cache pages", qkv.dtype)
+            _device_tensor(cache, "cache pages", out_dtype)
             _need(cache.dim() == 4 and tuple(cache.shape[1:]) == (kv_heads, page_size, head_dim),
                   "cache pages must be [pages, kv_heads, page_size, head_dim]")
     if q_out is None:
-        q_out = torch.empty((n_tokens, heads * head_dim), dtype=qkv.dtype, device=qkv.device)
-    _device_tensor(q_out, "q output", qkv.dtype)
+        q_out = torch.empty((n_tokens, heads * head_dim), dtype=out_dtype, device=qkv.device)
+    _device_tensor(q_out, "q output", out_dtype)
     _need(tuple(q_out.shape) == (n_tokens, heads * head_dim), "q output has the wrong shape")
-    _check(lib.mll_qkv_rope_store(_ptr(qkv), _code(qkv.dtype), _ptr(bias), _ptr(positions), _ptr(slot_mapping),
+    _check(lib.mll_qkv_rope_store(_ptr(qkv), _code(qkv.dtype), _code(out_dtype), _ptr(bias), _ptr(positions), _ptr(slot_mapping),
                                   _ptr(inv_freq), n_freq, _ptr(q_out), _ptr(k_cache), _ptr(v_cache),
                                   n_tokens, heads, kv_heads, head_dim, page_size, _stream()), lib)
     return q_out

@@ -77,7 +77,7 @@ class PagedAttention(Mixer):
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
         view = ctx.paged[cache.group]
         kv_heads = cache.need.kv_heads
-        qkv = linear(x, self.qkv_weight)
+        qkv = linear(x, self.qkv_weight, out_dtype=torch.float32)   # rounded once, after bias and rotation
         stored_heads = self.kv_heads if self.owns_kv else 0
         slot_mapping = view.slot_mapping if self.owns_kv else None
         k_pages = cache.k if self.owns_kv else None
@@ -89,15 +89,15 @@ class PagedAttention(Mixer):
                 inv_freq = self.position.inv_freq
             else:
                 if bias is not None:
-                    qkv = (qkv.float() + bias).to(qkv.dtype)
+                    qkv = qkv + bias
                     bias = None
                 qkv = self.position.apply(qkv, ctx.positions, self.heads, stored_heads, self.head_dim).contiguous()
         q = kernels.qkv_rope_store(qkv, bias, ctx.positions, slot_mapping, inv_freq, k_pages, v_pages,
-                                   self.heads, stored_heads, self.head_dim, view.page_size)
+                                   self.heads, stored_heads, self.head_dim, view.page_size, self.runtime.dtype)
         window = int(self.window) if self.window else 0
         o = kernels.paged_attention(q, cache.k, cache.v, view, ctx, self.scale, window,
                                     self.heads, kv_heads, self.head_dim)
-        return linear(o, self.o_weight)
+        return linear(o, self.o_weight, out_dtype=torch.float32)        # summed into the residual stream in float32
 
 
 register_part("mixer", "paged_attention", PagedAttention)

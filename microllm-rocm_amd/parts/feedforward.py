@@ -42,7 +42,7 @@ class SwiGLU(FeedForward):
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         gate_up = linear(x, self.gate_up_weight)
-        return linear(kernels.silu_mul(gate_up), self.down_weight)
+        return linear(kernels.silu_mul(gate_up), self.down_weight, out_dtype=torch.float32)
 
 
 register_part("ffn", "swiglu", SwiGLU)

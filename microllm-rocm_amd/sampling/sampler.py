@@ -1,0 +1,84 @@
+"""Choosing the next token: greedy, temperature and top-k, on the device.
+
+Rules follow the reference's ``sample_token`` (src/inference/generator.cpp:36-69):
+temperature 0 or top_k 1 gives the first maximum; otherwise the top_k largest
+logits (all when top_k is 0) are weighed by ``exp(l/T - max/T)`` and one is drawn;
+non-finite logits are an error. The reference draws with ``mt19937_64`` and
+``std::discrete_distribution``, whose algorithm the C++ library defines; here the
+draw is by inverse CDF in token order with one uniform per token from a
+counter-based rule keyed by (seed, index of the draw), so that the device kernel,
+a plain implementation and a preempted request that is run again all see the
+same stream. Defaults are the reference's (include/microllm/inference/generator.h:11-23).
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+from typing import List, Sequence, Tuple
+
+import torch
+
+from ..ops import kernels
+
+_MASK = (1 << 64) - 1
+
+
+@dataclass(frozen=True)
+class SamplingParams:
+    max_new_tokens: int = 32
+    temperature: float = 1.0
+    top_k: int = 0
+    seed: int = 1
+    stop_tokens: Tuple[int, ...] = ()
+
+    @property
+    def greedy(self) -> bool:
+        return self.temperature == 0.0 or self.top_k == 1
+
+    def validate(self, vocab_size: int) -> None:
+        """The checks of src/inference/scheduler.cpp:32-63."""
+        if self.max_new_tokens < 0:
+            raise ValueError("max_new_tokens must be non-negative")
+        if not math.isfinite(self.temperature) or self.temperature < 0.0:
+            raise ValueError("sampling temperature must be finite and non-negative")
+        if not 0 <= self.top_k <= vocab_size:
+            raise ValueError("top_k is outside the vocabulary")
+        if len(set(self.stop_tokens)) != len(self.stop_tokens):
+            raise ValueError("stop tokens must be unique")
+        for token in self.stop_tokens:
+            if not 0 <= token < vocab_size:
+                raise ValueError(f"stop token {token} is outside the vocabulary")
+
+
+def uniform_for(seed: int, draw: int) -> float:
+    """The uniform in [0, 1) for a request's ``draw``-th sampled token (splitmix64 finaliser, top 24 bits)."""
+    z = (seed * 0x9E3779B97F4A7C15 + (draw + 1) * 0xBF58476D1CE4E5B9) & _MASK
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _MASK
+    z ^= z >> 31
+    return (z >> 40) / float(1 << 24)
+
+
+class NonFiniteLogits(RuntimeError):
+    """A row of logits held NaN or infinity (the reference throws too, src/inference/scheduler.cpp:918-920)."""
+
+
+class Sampler:
+    """Selects one token per row of logits on the device; one transfer of the chosen ids back."""
+
+    def select(self, logits: torch.Tensor, params: Sequence[SamplingParams], draws: Sequence[int]) -> List[int]:
+        if logits.shape[0] != len(params) or len(params) != len(draws):
+            raise ValueError("one SamplingParams and one draw index per row of logits")
+        if all(p.greedy for p in params):
+            chosen = kernels.argmax(logits)
+        else:
+            device = logits.device
+            temperature = torch.tensor([0.0 if p.greedy else p.temperature for p in params], dtype=torch.float32, device=device)
+            top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32, device=device)
+            uniform = torch.tensor([uniform_for(p.seed, d) for p, d in zip(params, draws)], dtype=torch.float32, device=device)
+            chosen = kernels.sample(logits, temperature, top_k, uniform)
+        tokens = chosen.tolist()
+        for row, token in enumerate(tokens):
+            if token < 0:
+                raise NonFiniteLogits(f"row {row} of the logits is not finite")
+        return tokens

@@ -1,0 +1,157 @@
+"""Trace replay on the GPU against the plain implementation: whole, prefill then decode, changing portions and
+mixed batches with reused pages, in float32 and in bfloat16, on tiny configurations that differ in every size."""
+import io
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from replay_tools import (PlainModel, collect, compare, mixed, portions, prefill_then_decode, round_up, to_lines,
+                          whole)
+from tiny import CONFIGS, make_folder, random_tokens
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SHARP = {"std": 0.12, "norm_std": 0.1}   # sharper attention and larger biases than N(0, 0.02) gives
+DTYPES = ["float32", "bfloat16"]
+CASES = [("A", None), ("B", None), ("A", SHARP), ("B", SHARP), ("C", SHARP)]
+_models = {}
+
+
+def model_for(tmp_path_factory, which, stds):
+    key = (which, bool(stds))
+    if key not in _models:
+        folder = make_folder(tmp_path_factory.mktemp(f"model_{which}_{'sharp' if stds else 'std'}"), which, stds)
+        _models[key] = (folder, PlainModel(folder))
+    return _models[key]
+
+
+def run_trace(folder, dtype, steps, out_dir, max_tokens):
+    """In-process replay: the same ``replay`` that bin/trace_run calls, on a fresh engine."""
+    from microllm_rocm_amd.engine import Engine
+    from microllm_rocm_amd.engine.replay import replay
+    engine = Engine.from_folder(folder, dtype=dtype, max_tokens=max_tokens, max_requests=8)
+    report = io.StringIO()
+    replay(engine, io.StringIO(to_lines(steps)), str(out_dir), report)
+    assert report.getvalue().split() == [word for step in steps for word in ("done", str(step["step"]))]
+    engine.cache.check()
+    assert not engine.cache.requests, "every request of a trace is ended"
+    assert all(free == group.pool.num_pages for free, group in zip(engine.cache.free_pages(), engine.cache.groups))
+    return engine
+
+
+def requests_for(config, lengths, seed):
+    return {f"r{index}": random_tokens(seed + index, length, config.vocab_size) for index, length in enumerate(lengths)}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which,stds", CASES)
+def test_every_cut_matches_the_plain_implementation(tmp_path_factory, tmp_path, which, stds, dtype):
+    config = CONFIGS[which]
+    folder, plain_model = model_for(tmp_path_factory, which, stds)
+    lengths = [100, 64, 37] if which != "C" else [300, 129, 64]
+    requests = requests_for(config, lengths, seed=10)
+    vocab = config.vocab_size
+    results = {}
+
+    steps = whole(requests)
+    run_trace(folder, dtype, steps, tmp_path / "whole", max_tokens=round_up(max(lengths), 64))
+    results["whole"] = collect(steps, tmp_path / "whole", vocab)
+    compare(results["whole"], requests, plain_model, dtype)
+
+    for rid, tokens in requests.items():
+        steps = prefill_then_decode(rid, tokens, tail=32)
+        run_trace(folder, dtype, steps, tmp_path / f"decode_{rid}", max_tokens=round_up(len(tokens), 64))
+        results[f"decode_{rid}"] = collect(steps, tmp_path / f"decode_{rid}", vocab)
+        compare(results[f"decode_{rid}"], {rid: tokens}, plain_model, dtype)
+
+        steps = portions(rid, tokens, sizes=[7, 2, 5, 16, 3, 2, 33, 2, 17])
+        run_trace(folder, dtype, steps, tmp_path / f"portions_{rid}", max_tokens=round_up(len(tokens), 64))
+        results[f"portions_{rid}"] = collect(steps, tmp_path / f"portions_{rid}", vocab)
+        compare(results[f"portions_{rid}"], {rid: tokens}, plain_model, dtype)
+
+    if dtype == "float32":
+        # In 32-bit every kernel sums in an order that depends on the row alone: the cuts agree bit for bit.
+        for name, rows in results.items():
+            if name == "whole":
+                continue
+            for key, row in rows.items():
+                assert np.array_equal(row, results["whole"][key]), f"{name}: {key} differs from the whole run"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which,stds", [("A", SHARP), ("B", SHARP), ("C", SHARP)])
+def test_mixed_batches_with_reused_pages(tmp_path_factory, tmp_path, which, stds, dtype):
+    config = CONFIGS[which]
+    folder, plain_model = model_for(tmp_path_factory, which, stds)
+    lengths = [70, 45, 90, 33, 64, 50, 81] if which != "C" else [200, 70, 150, 64, 260, 90]
+    requests = requests_for(config, lengths, seed=20)
+    steps, peak = mixed(requests, seed=3)
+    assert max(len(step["entries"]) for step in steps) == 4
+    assert any(len(e["tokens"]) == 1 for s in steps for e in s["entries"]) and any(len(e["tokens"]) == 2 for s in steps for e in s["entries"])
+    engine = run_trace(folder, dtype, steps, tmp_path / "mixed", max_tokens=peak)
+    pool = engine.cache.groups[0].pool
+    assert pool.total_taken > pool.num_pages, "the pool is small enough for pages to be used again"
+    got = collect(steps, tmp_path / "mixed", config.vocab_size)
+    compare(got, requests, plain_model, dtype)
+    if dtype == "float32":
+        alone = whole(requests)
+        run_trace(folder, dtype, alone, tmp_path / "alone", max_tokens=round_up(max(lengths), 64))
+        reference = collect(alone, tmp_path / "alone", config.vocab_size)
+        for key, row in got.items():
+            assert np.array_equal(row, reference[key]), f"mixed: {key} differs from the request run alone"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_first_tokens_and_long_decoding(tmp_path_factory, tmp_path, dtype):
+    config = CONFIGS["C"]
+    folder, plain_model = model_for(tmp_path_factory, "C", SHARP)
+    tokens = random_tokens(77, 400, config.vocab_size)
+    # the first tokens of a sequence, one by one from an empty cache, then a long run of decoding past the window
+    steps = prefill_then_decode("long", tokens, tail=399)
+    run_trace(folder, dtype, steps, tmp_path / "long", max_tokens=round_up(len(tokens), 64))
+    got = collect(steps, tmp_path / "long", config.vocab_size)
+    compare(got, {"long": tokens}, plain_model, dtype)
+    for count in (1, 2, 3):
+        steps = whole({"first": tokens[:count]})
+        run_trace(folder, dtype, steps, tmp_path / f"first{count}", max_tokens=64)
+        compare(collect(steps, tmp_path / f"first{count}", config.vocab_size), {"first": tokens[:count]}, plain_model, dtype)
+
+
+def test_logits_only_where_wanted_and_requests_left_out(tmp_path_factory, tmp_path):
+    config = CONFIGS["B"]
+    folder, plain_model = model_for(tmp_path_factory, "B", SHARP)
+    a, b = random_tokens(1, 40, config.vocab_size), random_tokens(2, 30, config.vocab_size)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:20], "want": []}], "end": []},
+        {"step": 1, "entries": [{"id": "b", "tokens": b[:30], "want": [29, 0]}], "end": ["b"]},
+        {"step": 2, "entries": [{"id": "a", "tokens": a[20:40], "want": [19]}], "end": ["a"]},
+    ]
+    run_trace(folder, "float32", steps, tmp_path / "out", max_tokens=128)
+    assert not os.path.exists(tmp_path / "out" / "0.f32")
+    rows = np.fromfile(tmp_path / "out" / "1.f32", dtype="<f4").reshape(2, config.vocab_size)
+    reference = plain_model.logits(b)
+    scale = np.abs(reference).max()
+    assert np.abs(rows[0] - reference[29]).max() <= 2e-5 * scale and np.abs(rows[1] - reference[0]).max() <= 2e-5 * scale
+    last = np.fromfile(tmp_path / "out" / "2.f32", dtype="<f4")
+    assert np.abs(last - plain_model.logits(a)[39]).max() <= 2e-5 * np.abs(plain_model.logits(a)).max()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_program_itself(tmp_path_factory, tmp_path, dtype):
+    """bin/trace_run as a user calls it: a process, steps on standard input, files in --out."""
+    config = CONFIGS["B"]
+    folder, plain_model = model_for(tmp_path_factory, "B", SHARP)
+    requests = requests_for(config, [50, 64, 33, 40, 70], seed=40)
+    steps, peak = mixed(requests, seed=5)
+    out_dir = tmp_path / "program"
+    result = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                             "--out", str(out_dir), "--max-tokens", str(peak)],
+                            input=to_lines(steps), capture_output=True, text=True, timeout=300)
+    assert result.returncode == 0, result.stderr
+    assert result.stdout.split() == [word for step in steps for word in ("done", str(step["step"]))]
+    compare(collect(steps, out_dir, config.vocab_size), requests, plain_model, dtype)
