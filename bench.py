@@ -1,0 +1,101 @@
+"""Decode and prefill throughput of the engine at Qwen2-7B size with random weights on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+A step is one decode step of the engine's own loop: one token of every request through `Engine.step`,
+greedy selection on the device, the chosen ids back to the host. Prints one JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+BF16_PEAK_FLOPS = 2.5e15       # MI355X dense bf16 MFMA, published
+FP32_PEAK_FLOPS = 157.3e12
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=64)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--context", type=int, default=4096)
+    parser.add_argument("--layers", type=int, default=28, help="fewer than 28 only where memory or time needs it")
+    parser.add_argument("--prefill-tokens", type=int, default=2048)
+    parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    parser.add_argument("--points", default="1,64", help="other decode batch sizes to report")
+    parser.add_argument("--no-prefill", action="store_true")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
+        return 2
+
+    import torch
+    from microllm_rocm_amd import Engine, Qwen2Config
+    from microllm_rocm_amd.engine.benchmark import decode_throughput, prefill_throughput, step_bytes, step_flops
+
+    full_layers = 28
+    config = Qwen2Config(vocab_size=152064, hidden_size=3584, num_hidden_layers=args.layers, num_attention_heads=28,
+                         num_key_value_heads=4, head_dim=128, intermediate_size=18944, max_position_embeddings=32768,
+                         rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False)
+    page_size = 16
+    points = sorted({int(b) for b in args.points.split(",") if b} | {args.batch})
+    largest = max(points)
+    per_request = args.context + args.steps + args.warmup + 2 * page_size
+    max_tokens = max(largest * per_request, args.prefill_tokens + page_size)
+    engine = Engine.from_random(config, seed=0, dtype=args.dtype, device="cuda:0", on_device=True,
+                                page_size=page_size, max_tokens=max_tokens, max_requests=max(largest, 4))
+    peak_flops = BF16_PEAK_FLOPS if args.dtype == "bfloat16" else FP32_PEAK_FLOPS
+
+    results = {}
+    for batch in points:
+        results[batch] = decode_throughput(engine, batch, args.context, args.steps, args.warmup, seed=batch)
+    main_result = results[args.batch]
+    bytes_step = step_bytes(engine, args.batch, args.context + args.warmup + args.steps // 2)
+    achieved = bytes_step / (main_result["ms_per_step"] * 1e-3) / 1e9
+
+    line = {
+        "metric": "decode tok/s (ctx 4096) Qwen2-7B bf16",
+        "value": round(main_result["tokens_per_second"], 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(main_result["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: random N(0,0.02) weights, uniform-random token ids, caches filled with random keys and values",
+        "config": {
+            "model": "Qwen2-7B size", "layers": args.layers, "layers_of_full_model": full_layers,
+            "hidden_size": config.hidden_size, "heads": config.num_attention_heads,
+            "kv_heads": config.num_key_value_heads, "head_dim": config.head_dim,
+            "intermediate_size": config.intermediate_size, "vocab_size": config.vocab_size,
+            "tie_word_embeddings": False, "global_batch": args.batch, "seq_len": args.context,
+            "kv_block_size": page_size, "prefill_tokens": args.prefill_tokens, "parallelism": "single GPU",
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "points": {f"decode_b{batch}": round(results[batch]["tokens_per_second"], 2) for batch in points if batch != args.batch},
+    }
+    if not args.no_prefill:
+        prefill = prefill_throughput(engine, args.prefill_tokens, repeats=3)
+        flops = step_flops(engine, args.prefill_tokens)
+        line["prefill"] = {"value": round(prefill["tokens_per_second"], 1), "tokens": args.prefill_tokens,
+                           "ms": round(prefill["ms"], 3),
+                           "frac": round(flops / (prefill["ms"] * 1e-3) / peak_flops, 4)}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

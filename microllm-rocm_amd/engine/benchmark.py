@@ -1,0 +1,129 @@
+"""Timed workloads shared by ``bench.py`` and the command line: steady decoding and one prefill.
+
+Decoding is measured the way the reference's "steady" mode is (apps/hf_infer.cpp:352-361): every
+timed token runs one forward. Caches are filled with random keys and values instead of by a
+prefill of the context, which changes no byte that a decode step reads or writes.
+"""
+from __future__ import annotations
+
+import time
+from typing import Dict
+
+import numpy as np
+import torch
+
+from ..cache.manager import PagedBinding
+from ..sampling import Sampler, SamplingParams
+from .batch import StepEntry
+from .engine import Engine
+
+
+def _fill_random(engine: Engine) -> None:
+    for binding in engine.cache.bindings():
+        if isinstance(binding, PagedBinding) and binding.owned:
+            binding.k.normal_(0.0, 1.0)
+            binding.v.normal_(0.0, 1.0)
+
+
+def decode_throughput(engine: Engine, batch: int, context: int, steps: int, warmup: int, seed: int = 0) -> Dict[str, float]:
+    """``batch`` requests that each hold ``context`` positions decode ``warmup + steps`` tokens, greedily."""
+    rng = np.random.default_rng(seed)
+    sampler = Sampler()
+    params = [SamplingParams(temperature=0.0)] * batch
+    ids = [("bench", batch, index) for index in range(batch)]
+    for request_id in ids:
+        request = engine.open(request_id)
+        engine.cache.reserve(request, context)
+        engine.cache.commit(request, context)
+    _fill_random(engine)
+    tokens = rng.integers(0, engine.spec.vocab_size, size=batch).tolist()
+
+    def one_step(current):
+        logits = engine.step([StepEntry(request_id, [token], [0]) for request_id, token in zip(ids, current)])
+        return sampler.select(logits, params, [0] * batch)
+
+    try:
+        for _ in range(warmup):
+            tokens = one_step(tokens)
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        for _ in range(steps):
+            tokens = one_step(tokens)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+    finally:
+        for request_id in ids:
+            engine.close(request_id)
+    return {"tokens_per_second": batch * steps / elapsed, "ms_per_step": elapsed / steps * 1e3}
+
+
+def prefill_throughput(engine: Engine, tokens: int, repeats: int = 3, seed: int = 0) -> Dict[str, float]:
+    """One request's prompt of ``tokens`` ids in one step, logits at its last position; the best of ``repeats``."""
+    rng = np.random.default_rng(seed)
+    prompt = rng.integers(0, engine.spec.vocab_size, size=tokens).tolist()
+    best = float("inf")
+    for repeat in range(repeats + 1):   # the first run warms up
+        request_id = ("prefill", repeat)
+        engine.open(request_id)
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        logits = engine.step([StepEntry(request_id, prompt, [tokens - 1])])
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+        engine.close(request_id)
+        assert torch.isfinite(logits).all()
+        if repeat > 0:
+            best = min(best, elapsed)
+    return {"tokens_per_second": tokens / best, "ms": best * 1e3}
+
+
+def weight_bytes(engine: Engine) -> int:
+    """Bytes of every weight a decode step reads once: all layers, the final norm and the head (an embedding
+    table that is not the head's is read one row per token, which is counted apart)."""
+    seen, total = set(), 0
+    embedding_only = None
+    model = engine.model
+    if model.embedding.table.data_ptr() != model.head.weight.data_ptr():
+        embedding_only = model.embedding.table.data_ptr()
+    tensors = [model.final_norm.weight, model.head.weight]
+    for block in model.blocks:
+        for part in block.parts():
+            tensors += [value for value in vars(part).values() if isinstance(value, torch.Tensor)]
+            position = getattr(part, "position", None)
+            if position is not None:
+                tensors += [value for value in vars(position).values() if isinstance(value, torch.Tensor)]
+    for tensor in tensors:
+        if tensor.data_ptr() in seen or tensor.data_ptr() == embedding_only:
+            continue
+        seen.add(tensor.data_ptr())
+        total += tensor.numel() * tensor.element_size()
+    return total
+
+
+def step_bytes(engine: Engine, batch: int, context: int) -> int:
+    """What a decode step has to read: every weight once, the cache of the live requests, one embedding row each."""
+    element = torch.empty((), dtype=engine.dtype).element_size()
+    cache = 0
+    for group in engine.cache.groups:
+        visible = context if group.need.window is None else min(context, group.need.window)
+        cache += 2 * len(group.entries) * group.need.kv_heads * group.need.head_dim * visible * element
+    row = engine.spec.hidden_size * engine.model.embedding.table.element_size()
+    return weight_bytes(engine) + batch * (cache + row)
+
+
+def step_flops(engine: Engine, tokens: int) -> float:
+    """Floating-point operations of one prompt of ``tokens`` ids: 2 per multiply-add of every matrix product over
+    all tokens (the head for one row) and of causal attention (scores and values)."""
+    flops = 0.0
+    for block in engine.model.blocks:
+        for part in block.parts():
+            for name, value in vars(part).items():
+                if isinstance(value, torch.Tensor) and value.dim() == 2:
+                    flops += 2.0 * value.numel() * tokens
+        mixer = block.mixer
+        if hasattr(mixer, "heads"):
+            window = mixer.window or tokens
+            pairs = sum(min(position + 1, window) for position in range(tokens))
+            flops += 4.0 * mixer.heads * mixer.head_dim * pairs
+    flops += 2.0 * engine.model.head.weight.numel()
+    return flops
