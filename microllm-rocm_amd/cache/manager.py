@@ -3,8 +3,8 @@
 Run entries of the model declare what they need: keys and values in pages
 (``PagedKVNeed``, perhaps with a window) or per-request state of fixed size
 (``StateNeed``). Entries with equal paged needs form a group; a group has a pool
-and page arrays of its own, one pair ``[pages, kv_heads, page_size, head_dim]``
-per entry, and every request has one block table per group. Pages are taken when
+and page arrays of its own, keys ``[pages, kv_heads, page_size, head_dim]`` and values
+``[pages, kv_heads, head_dim, page_size]`` per entry, and every request has one block table per group. Pages are taken when
 a request's tokens cross a page's edge, given back when the request is closed,
 and, in a group with a window, as soon as every position on them is older than
 any later query can see. Nothing is cleared on reuse: lengths, not contents,
@@ -98,9 +98,10 @@ class CacheManager:
                 group.entries.append(entry)
                 k = v = None
                 if device is not None:
-                    shape = (num_pages, need.kv_heads, page_size, need.head_dim)
-                    k = torch.empty(shape, dtype=dtype, device=device)
-                    v = torch.empty(shape, dtype=dtype, device=device)
+                    # Values are kept transposed so that one dim's keys are contiguous for the MFMA kernels.
+                    # Zeroed once: a kernel may read a whole page whose tail was never written.
+                    k = torch.zeros((num_pages, need.kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
+                    v = torch.zeros((num_pages, need.kv_heads, need.head_dim, page_size), dtype=dtype, device=device)
                 self._bindings[entry] = PagedBinding(group.index, need, k, v, owned=True)
             elif isinstance(need, StateNeed):
                 state = None

@@ -1,0 +1,285 @@
+// Paged attention for single query tokens (decoding) in bfloat16: split over the keys, MFMA for both
+// products, online softmax in float32, a second kernel that joins the splits.
+//
+// One workgroup (4 waves) takes one token, one kv head (with up to 16 of its query heads) and one split
+// of the visible keys. A wave walks pairs of 16-key tiles. Scores are computed transposed,
+// S^T = K . Q^T (v_mfma_f32_16x16x32_bf16: A = 16 keys x 32 dims straight from the page, B = Q^T), so
+// that a lane ends up with 8 keys of one head: exactly the B operand of O^T = V^T . P^T, whose A operand
+// comes straight from the value pages, which are stored transposed ([page, kv_head, dim, key]) for this.
+// Nothing passes through LDS but the final join of the 4 waves.
+#include "common.h"
+#include "microllm_hip.h"
+
+namespace mll {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kDecodeWaves = 4;
+constexpr int kDecodeThreads = kDecodeWaves * kWave;
+
+union Frag8 {
+    bf16x8 v;
+    bf16x4 h[2];
+    uint4 raw;
+};
+
+template <int HD_TILES>
+__global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+    const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ seq_of_token,
+    const int32_t* __restrict__ positions, bf16* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, float scale, int window, int heads, int kv_heads, int page_size, int n_splits) {
+    constexpr int HD = HD_TILES * 16;
+    constexpr int K_STEPS = (HD + 31) / 32;
+    __shared__ float o_shared[16][HD + 4];
+    __shared__ float m_shared[16];
+    __shared__ float l_shared[16];
+
+    const int token = blockIdx.x;
+    const int group = heads / kv_heads;
+    const int chunks = (group + 15) / 16;
+    const int kv_head = blockIdx.y / chunks;
+    const int chunk = blockIdx.y % chunks;
+    const int split = blockIdx.z;
+    const int head0 = kv_head * group + chunk * 16;
+    const int heads_here = min(16, group - chunk * 16);
+
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int col = lane % 16;   // head (B operands, results) or key/dim row (A operands)
+    const int quad = lane / 16;  // which 8 of the 32 k-slots this lane supplies
+
+    const int seq = seq_of_token[token];
+    const int position = positions[token];
+    const int low = window > 0 ? max(0, position - window + 1) : 0;
+    const int32_t* table = block_table + static_cast<int64_t>(seq) * table_width;
+
+    const int first_pair = low / 32, last_pair = position / 32;
+    const int total_pairs = last_pair - first_pair + 1;
+    const int pairs_per_split = (total_pairs + n_splits - 1) / n_splits;
+    const int pair_begin = first_pair + split * pairs_per_split;
+    const int pair_end = min(pair_begin + pairs_per_split, last_pair + 1);
+
+    // Q^T fragments: head `col`, dims ks * 32 + quad * 8 ... + 7.
+    Frag8 q_frag[K_STEPS];
+#pragma unroll
+    for (int ks = 0; ks < K_STEPS; ++ks) {
+        const int dim = ks * 32 + quad * 8;
+        q_frag[ks].raw = make_uint4(0, 0, 0, 0);
+        if (col < heads_here && dim < HD) {
+            q_frag[ks].raw = *reinterpret_cast<const uint4*>(
+                q + (static_cast<int64_t>(token) * heads + head0 + col) * HD + dim);
+        }
+    }
+
+    floatx4 o_acc[HD_TILES];
+#pragma unroll
+    for (int d = 0; d < HD_TILES; ++d) o_acc[d] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    float running_max = -INFINITY, running_sum = 0.0f;
+
+    for (int pair = pair_begin + wave; pair < pair_end; pair += kDecodeWaves) {
+        const int key0 = pair * 32;
+        bool tile_live[2];
+        int64_t k_row[2], v_row[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int tile_key = key0 + 16 * t;
+            tile_live[t] = tile_key <= position && tile_key + 15 >= low;
+            k_row[t] = v_row[t] = 0;
+            if (tile_live[t]) {
+                const int64_t page = table[tile_key / page_size];
+                const int offset = tile_key % page_size;
+                k_row[t] = ((page * kv_heads + kv_head) * page_size + offset + col) * HD;       // key `col` of the tile
+                v_row[t] = ((page * kv_heads + kv_head) * HD + col) * page_size + offset;       // dim `col` of a dim tile
+            }
+        }
+        // Keys: A operand, row = key, 8 dims per lane.
+        Frag8 k_frag[2][K_STEPS];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int ks = 0; ks < K_STEPS; ++ks) {
+                const int dim = ks * 32 + quad * 8;
+                k_frag[t][ks].raw = make_uint4(0, 0, 0, 0);
+                if (tile_live[t] && dim < HD)
+                    k_frag[t][ks].raw = *reinterpret_cast<const uint4*>(k_cache + k_row[t] + dim);
+            }
+        // Values: A operand of the second product, row = dim, k-slots = keys 4*quad..+3 of tile 0, then of tile 1.
+        Frag8 v_frag[HD_TILES];
+#pragma unroll
+        for (int d = 0; d < HD_TILES; ++d) {
+            v_frag[d].raw = make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                if (tile_live[t])
+                    v_frag[d].h[t] = *reinterpret_cast<const bf16x4*>(
+                        v_cache + v_row[t] + static_cast<int64_t>(d) * 16 * page_size + quad * 4);
+        }
+
+        // S^T = K . Q^T: lane holds head `col`, keys 4*quad + i of each tile.
+        float score[8];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            floatx4 s = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int ks = 0; ks < K_STEPS; ++ks)
+                s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_frag[t][ks].v, q_frag[ks].v, s, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = key0 + 16 * t + 4 * quad + i;
+                score[4 * t + i] = (key >= low && key <= position) ? s[i] * scale : -INFINITY;
+            }
+        }
+        // A pair that straddles an end of the visible range may hold stale values: they must not reach
+        // the product, where 0 * NaN would be NaN.
+        if (key0 < low || key0 + 31 > position) {
+#pragma unroll
+            for (int d = 0; d < HD_TILES; ++d)
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (score[j] == -INFINITY) v_frag[d].v[j] = static_cast<__bf16>(0.0f);
+        }
+
+        float tile_max = score[0];
+#pragma unroll
+        for (int j = 1; j < 8; ++j) tile_max = fmaxf(tile_max, score[j]);
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+        const float new_max = fmaxf(running_max, tile_max);   // finite: every pair holds a visible key
+        const float rescale = __expf(running_max - new_max);
+        Frag8 p_frag;
+        float tile_sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float p = __expf(score[j] - new_max);
+            tile_sum += p;
+            p_frag.v[j] = static_cast<__bf16>(p);
+        }
+        tile_sum += __shfl_xor(tile_sum, 16, kWave);
+        tile_sum += __shfl_xor(tile_sum, 32, kWave);
+        running_sum = running_sum * rescale + tile_sum;
+        running_max = new_max;
+#pragma unroll
+        for (int d = 0; d < HD_TILES; ++d) {
+            o_acc[d] *= rescale;
+            o_acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_frag[d].v, p_frag.v, o_acc[d], 0, 0, 0);
+        }
+    }
+
+    // Join the 4 waves, one after the other, in LDS: o_shared[head][dim].
+    for (int w = 0; w < kDecodeWaves; ++w) {
+        __syncthreads();
+        if (wave != w) continue;
+        float old_max = w == 0 ? -INFINITY : m_shared[col];
+        float old_sum = w == 0 ? 0.0f : l_shared[col];
+        const float new_max = fmaxf(old_max, running_max);
+        const float keep = (old_max == -INFINITY) ? 0.0f : __expf(old_max - new_max);
+        const float add = (running_max == -INFINITY) ? 0.0f : __expf(running_max - new_max);
+#pragma unroll
+        for (int d = 0; d < HD_TILES; ++d)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int dim = d * 16 + quad * 4 + i;
+                const float before = w == 0 ? 0.0f : o_shared[col][dim];
+                o_shared[col][dim] = before * keep + o_acc[d][i] * add;
+            }
+        if (quad == 0) {
+            m_shared[col] = new_max;
+            l_shared[col] = old_sum * keep + running_sum * add;
+        }
+    }
+    __syncthreads();
+
+    for (int index = threadIdx.x; index < heads_here * HD; index += kDecodeThreads) {
+        const int h = index / HD, dim = index % HD;
+        const int64_t row = static_cast<int64_t>(token) * heads + head0 + h;
+        if (n_splits == 1) {
+            out[row * HD + dim] = from_float<bf16>(o_shared[h][dim] / l_shared[h]);
+        } else {
+            part_o[(row * n_splits + split) * HD + dim] = o_shared[h][dim];
+        }
+    }
+    if (n_splits > 1 && threadIdx.x < heads_here) {
+        const int64_t row = static_cast<int64_t>(token) * heads + head0 + threadIdx.x;
+        part_ml[(row * n_splits + split) * 2 + 0] = m_shared[threadIdx.x];
+        part_ml[(row * n_splits + split) * 2 + 1] = l_shared[threadIdx.x];
+    }
+}
+
+// Joins the splits of one (token, head): out = sum_s w_s O_s / sum_s w_s l_s with w_s = exp(m_s - max m).
+__global__ void paged_attention_join_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                            bf16* __restrict__ out, int head_dim, int n_splits) {
+    const int64_t row = blockIdx.x;
+    const float* ml = part_ml + row * n_splits * 2;
+    float top = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) top = fmaxf(top, ml[2 * s]);
+    for (int dim = threadIdx.x; dim < head_dim; dim += blockDim.x) {
+        float total = 0.0f, weight_sum = 0.0f;
+        for (int s = 0; s < n_splits; ++s) {
+            const float m = ml[2 * s];
+            if (m == -INFINITY) continue;   // a split without keys
+            const float weight = __expf(m - top);
+            total += weight * part_o[(row * n_splits + s) * head_dim + dim];
+            weight_sum += weight * ml[2 * s + 1];
+        }
+        out[row * head_dim + dim] = from_float<bf16>(total / weight_sum);
+    }
+}
+
+template <int HD_TILES>
+static int launch_decode(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
+                         int table_width, const int32_t* seq_of_token, const int32_t* positions, void* out,
+                         float* part_o, float* part_ml, float scale, int window, int n_tokens, int heads, int kv_heads,
+                         int page_size, int n_splits, hipStream_t stream) {
+    const int group = heads / kv_heads;
+    const dim3 grid(n_tokens, kv_heads * ((group + 15) / 16), n_splits);
+    paged_attention_decode_kernel<HD_TILES><<<grid, kDecodeThreads, 0, stream>>>(
+        static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), block_table,
+        table_width, seq_of_token, positions, static_cast<bf16*>(out), part_o, part_ml, scale, window, heads, kv_heads,
+        page_size, n_splits);
+    return check_launch("paged_attention_decode");
+}
+
+}  // namespace mll
+
+using namespace mll;
+
+extern "C" int mll_paged_attention_decode(const void* q, const void* k_cache, const void* v_cache,
+                                          const int32_t* block_table, int table_width, const int32_t* seq_of_token,
+                                          const int32_t* positions, void* out, float* part_o, float* part_ml,
+                                          float scale, int window, int n_tokens, int heads, int kv_heads, int head_dim,
+                                          int page_size, int n_splits, hipStream_t stream) {
+    MLL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "paged_attention_decode: heads must divide into kv_heads groups");
+    MLL_REQUIRE(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256,
+                "paged_attention_decode: head_dim must be a multiple of 16 in [16, 256]");
+    MLL_REQUIRE(page_size > 0 && page_size % 16 == 0, "paged_attention_decode: page_size must be a multiple of 16");
+    MLL_REQUIRE(n_splits >= 1 && n_splits <= 65535, "paged_attention_decode: bad number of splits");
+    MLL_REQUIRE(n_splits == 1 || (part_o && part_ml), "paged_attention_decode: splits need the partial buffers");
+    MLL_REQUIRE(kv_heads * ((heads / kv_heads + 15) / 16) <= 65535, "paged_attention_decode: too many heads");
+    if (n_tokens == 0) return 0;
+    int status = 0;
+#define MLL_DECODE_CASE(TILES)                                                                                        \
+    case TILES:                                                                                                       \
+        status = launch_decode<TILES>(q, k_cache, v_cache, block_table, table_width, seq_of_token, positions, out,    \
+                                      part_o, part_ml, scale, window, n_tokens, heads, kv_heads, page_size, n_splits, \
+                                      stream);                                                                        \
+        break;
+    switch (head_dim / 16) {
+        MLL_DECODE_CASE(1) MLL_DECODE_CASE(2) MLL_DECODE_CASE(3) MLL_DECODE_CASE(4) MLL_DECODE_CASE(5)
+        MLL_DECODE_CASE(6) MLL_DECODE_CASE(7) MLL_DECODE_CASE(8) MLL_DECODE_CASE(9) MLL_DECODE_CASE(10)
+        MLL_DECODE_CASE(11) MLL_DECODE_CASE(12) MLL_DECODE_CASE(13) MLL_DECODE_CASE(14) MLL_DECODE_CASE(15)
+        MLL_DECODE_CASE(16)
+        default: return fail("paged_attention_decode: unsupported head_dim");
+    }
+#undef MLL_DECODE_CASE
+    if (status != 0) return status;
+    if (n_splits > 1) {
+        const int threads = head_dim <= 64 ? 64 : (head_dim <= 128 ? 128 : 256);
+        paged_attention_join_kernel<<<n_tokens * heads, threads, 0, stream>>>(part_o, part_ml, static_cast<bf16*>(out),
+                                                                             head_dim, n_splits);
+        return check_launch("paged_attention_join");
+    }
+    return 0;
+}

@@ -18,7 +18,7 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_kernel(
     int heads, int kv_heads, int head_dim, int page_size) {
     __shared__ float q_shared[kRowwiseMaxHeadDim];
     __shared__ float p_shared[kWave];
-    __shared__ int64_t row_shared[kWave];
+    __shared__ int64_t v_shared[kWave];
 
     const int token = blockIdx.x;
     const int head = blockIdx.y;
@@ -43,11 +43,12 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_kernel(
         const int key = tile + lane;
         const bool visible = key >= low && key <= position;
         float score = -INFINITY;
-        int64_t row = 0;
+        int64_t v_column = 0;
         if (visible) {
             const int64_t page = table[key / page_size];
-            row = ((page * kv_heads + kv_head) * page_size + key % page_size) * head_dim;
-            const T* k_row = k_cache + row;
+            const int offset = key % page_size;
+            const T* k_row = k_cache + ((page * kv_heads + kv_head) * page_size + offset) * head_dim;
+            v_column = (page * kv_heads + kv_head) * head_dim * page_size + offset;  // value pages are [.., dim, offset]
             float dot = 0.0f;
             for (int d = 0; d < head_dim; ++d) dot += q_shared[d] * to_float(k_row[d]);
             score = dot * scale;
@@ -60,7 +61,7 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_kernel(
 
         __syncthreads();  // the previous tile's readers are done
         p_shared[lane] = p;
-        row_shared[lane] = row;
+        v_shared[lane] = v_column;
         __syncthreads();
         const int first = max(low - tile, 0);
         const int last = min(position - tile, kWave - 1);
@@ -69,7 +70,8 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_kernel(
             const int d = lane + i * kWave;
             if (d < head_dim) {
                 float value = acc[i] * rescale;
-                for (int j = first; j <= last; ++j) value += p_shared[j] * to_float(v_cache[row_shared[j] + d]);
+                for (int j = first; j <= last; ++j)
+                    value += p_shared[j] * to_float(v_cache[v_shared[j] + static_cast<int64_t>(d) * page_size]);
                 acc[i] = value;
             }
         }

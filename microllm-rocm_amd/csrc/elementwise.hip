@@ -126,12 +126,16 @@ __global__ void qkv_rope_store_kernel(const In* __restrict__ qkv, const float* _
             T* q_row = q_out + (static_cast<int64_t>(token) * heads + head) * head_dim;
             q_row[first] = from_float<T>(y1);
             q_row[second] = from_float<T>(y2);
-        } else if (slot >= 0) {
-            const int kv_head = is_value ? head - heads - kv_heads : head - heads;
-            T* cache = is_value ? v_cache : k_cache;
-            T* row = cache + ((page * kv_heads + kv_head) * page_size + offset) * head_dim;
+        } else if (slot >= 0 && !is_value) {
+            const int kv_head = head - heads;
+            T* row = k_cache + ((page * kv_heads + kv_head) * page_size + offset) * head_dim;
             row[first] = from_float<T>(y1);
             row[second] = from_float<T>(y2);
+        } else if (slot >= 0) {  // value pages are transposed: [page, kv_head, dim, offset]
+            const int kv_head = head - heads - kv_heads;
+            T* column = v_cache + (page * kv_heads + kv_head) * head_dim * page_size + offset;
+            column[static_cast<int64_t>(first) * page_size] = from_float<T>(y1);
+            column[static_cast<int64_t>(second) * page_size] = from_float<T>(y2);
         }
     }
 }

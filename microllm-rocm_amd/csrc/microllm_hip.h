@@ -30,8 +30,9 @@ int mll_residual_add(float* h, const void* delta, int dtype, int n_rows, int wid
 // Splits fused projections qkv[t] = [q (H*hd) | k (KVH*hd) | v (KVH*hd)], adds `bias` (nullable),
 // rotates q and k by the split-half rule with angle position * inv_freq[i] in float64 (inv_freq nullable:
 // no rotation; rotary_dim = 2 * n_freq <= hd), writes q to q_out[t] and k, v into the pages:
-// slot = slot_mapping[t] (negative: not stored) addresses [page, kv_head, offset, :] with
-// page = slot / page_size.  k_cache / v_cache nullable together with slot_mapping. qkv has element type
+// slot = slot_mapping[t] (negative: not stored) addresses key pages [page, kv_head, offset, dim] and
+// value pages [page, kv_head, dim, offset] (transposed, so that a dim's keys are contiguous) with
+// page = slot / page_size, offset = slot % page_size.  k_cache / v_cache nullable together with slot_mapping. qkv has element type
 // `in_dtype` (float32, or the same as `dtype`); q_out and the pages have `dtype`.
 int mll_qkv_rope_store(const void* qkv, int in_dtype, int dtype, const float* bias, const int32_t* positions,
                        const int32_t* slot_mapping, const double* inv_freq, int n_freq,
@@ -48,6 +49,17 @@ int mll_paged_attention_rowwise(const void* q, int dtype, const void* k_cache, c
                                 const int32_t* seq_of_token, const int32_t* positions, void* out,
                                 float scale, int window, int n_tokens, int heads, int kv_heads,
                                 int head_dim, int page_size, hipStream_t stream);
+
+// out[t, c] = silu(gate[t, c]) * up[t, c]; gate and up rows are `in_stride` elements apart.
+// The same attention for bfloat16 with MFMA, one workgroup per (token, kv head, split of the keys): meant
+// for steps whose requests bring one token each, right for any. head_dim a multiple of 16 up to 256,
+// page_size a multiple of 16. n_splits > 1 needs part_o [tokens, heads, n_splits, head_dim] and
+// part_ml [tokens, heads, n_splits, 2] (float32 device scratch, contents need not be cleared).
+int mll_paged_attention_decode(const void* q, const void* k_cache, const void* v_cache,
+                               const int32_t* block_table, int table_width, const int32_t* seq_of_token,
+                               const int32_t* positions, void* out, float* part_o, float* part_ml,
+                               float scale, int window, int n_tokens, int heads, int kv_heads, int head_dim,
+                               int page_size, int n_splits, hipStream_t stream);
 
 // out[t, c] = silu(gate[t, c]) * up[t, c]; gate and up rows are `in_stride` elements apart.
 int mll_silu_mul(const void* gate, const void* up, int64_t in_stride, void* out, int dtype,

@@ -131,10 +131,12 @@ def qkv_rope_store(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: t
         _device_tensor(slot_mapping, "slot mapping", torch.int32)
         _need(tuple(slot_mapping.shape) == (n_tokens,), "slot mapping must hold one entry per token")
         _need(k_cache is not None and v_cache is not None, "slot mapping needs both caches")
-        for cache in (k_cache, v_cache):
-            _device_tensor(cache, "cache pages", out_dtype)
-            _need(cache.dim() == 4 and tuple(cache.shape[1:]) == (kv_heads, page_size, head_dim),
-                  "cache pages must be [pages, kv_heads, page_size, head_dim]")
+        _device_tensor(k_cache, "key pages", out_dtype)
+        _device_tensor(v_cache, "value pages", out_dtype)
+        _need(k_cache.dim() == 4 and tuple(k_cache.shape[1:]) == (kv_heads, page_size, head_dim),
+              "key pages must be [pages, kv_heads, page_size, head_dim]")
+        _need(v_cache.dim() == 4 and tuple(v_cache.shape) == (k_cache.shape[0], kv_heads, head_dim, page_size),
+              "value pages must be [pages, kv_heads, head_dim, page_size]")
     if q_out is None:
         q_out = torch.empty((n_tokens, heads * head_dim), dtype=out_dtype, device=qkv.device)
     _device_tensor(q_out, "q output", out_dtype)
@@ -148,11 +150,12 @@ def qkv_rope_store(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: t
 def _check_paged(q, k_cache, v_cache, block_table, heads, kv_heads, head_dim) -> int:
     _device_tensor(q, "queries")
     _need(q.dim() == 2 and q.shape[1] == heads * head_dim, "queries must be [tokens, heads * head_dim]")
-    for cache in (k_cache, v_cache):
-        _device_tensor(cache, "cache pages", q.dtype)
-        _need(cache.dim() == 4 and cache.shape[1] == kv_heads and cache.shape[3] == head_dim,
-              "cache pages must be [pages, kv_heads, page_size, head_dim]")
-    _need(k_cache.shape == v_cache.shape, "key and value pages must have one shape")
+    _device_tensor(k_cache, "key pages", q.dtype)
+    _device_tensor(v_cache, "value pages", q.dtype)
+    _need(k_cache.dim() == 4 and k_cache.shape[1] == kv_heads and k_cache.shape[3] == head_dim,
+          "key pages must be [pages, kv_heads, page_size, head_dim]")
+    _need(v_cache.dim() == 4 and tuple(v_cache.shape) == (k_cache.shape[0], kv_heads, head_dim, k_cache.shape[2]),
+          "value pages must be [pages, kv_heads, head_dim, page_size]")
     _device_tensor(block_table, "block table", torch.int32)
     _need(block_table.dim() == 2, "block table must be [requests, pages]")
     return k_cache.shape[2]
@@ -267,8 +270,49 @@ def gemm_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = to
     return torch.mm(x, weight.t(), out_dtype=out_dtype)
 
 
+def decode_splits(n_tokens: int, kv_heads: int, longest: int) -> int:
+    """How many splits of the keys fill the GPU: about a thousand workgroups, at least 128 keys each."""
+    wanted = -(-1024 // max(1, n_tokens * kv_heads))
+    return max(1, min(wanted, -(-longest // 128), 256))
+
+
+def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                           seq_of_token: torch.Tensor, positions: torch.Tensor, scale: float, window: int,
+                           heads: int, kv_heads: int, head_dim: int, n_splits: int,
+                           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The MFMA kernel for bfloat16 queries that each attend alone (one token per request)."""
+    lib = library.load()
+    page_size = _check_paged(q, k_cache, v_cache, block_table, heads, kv_heads, head_dim)
+    _need(q.dtype == torch.bfloat16, "the decode kernel takes bfloat16")
+    _need(head_dim % 16 == 0 and 16 <= head_dim <= 256, "the decode kernel takes head sizes in steps of 16 up to 256")
+    _need(page_size % 16 == 0, "the decode kernel takes page sizes in steps of 16")
+    n_tokens = q.shape[0]
+    _device_tensor(seq_of_token, "request of token", torch.int32)
+    _device_tensor(positions, "positions", torch.int32)
+    _need(seq_of_token.shape[0] == n_tokens and positions.shape[0] == n_tokens,
+          "request-of-token and positions must hold one entry per token")
+    if out is None:
+        out = torch.empty_like(q)
+    part_o = part_ml = None
+    if n_splits > 1:
+        part_o = torch.empty((n_tokens, heads, n_splits, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((n_tokens, heads, n_splits, 2), dtype=torch.float32, device=q.device)
+    _check(lib.mll_paged_attention_decode(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
+                                          _ptr(seq_of_token), _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml),
+                                          ctypes.c_float(scale), int(window), n_tokens, heads, kv_heads, head_dim,
+                                          page_size, n_splits, _stream()), lib)
+    return out
+
+
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, view, ctx,
                     scale: float, window: int, heads: int, kv_heads: int, head_dim: int) -> torch.Tensor:
     """Attention of the step's queries over their requests' pages; chooses the kernel for the batch's shape."""
+    page_size = k_cache.shape[2]
+    mfma_fits = q.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256 and page_size % 16 == 0
+    if mfma_fits and ctx.max_count == 1:
+        visible = min(ctx.max_total, window) if window > 0 else ctx.max_total
+        splits = decode_splits(ctx.n_tokens, kv_heads, visible)
+        return paged_attention_decode(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
+                                      scale, window, heads, kv_heads, head_dim, splits)
     return paged_attention_rowwise(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
                                    scale, window, heads, kv_heads, head_dim)
