@@ -3,8 +3,8 @@
 Run entries of the model declare what they need: keys and values in pages
 (``PagedKVNeed``, perhaps with a window) or per-request state of fixed size
 (``StateNeed``). Entries with equal paged needs form a group; a group has a pool
-and page arrays of its own, keys ``[pages, kv_heads, page_size, head_dim]`` and values
-``[pages, kv_heads, head_dim, page_size]`` per entry, and every request has one block table per group. Pages are taken when
+and page arrays of its own, keys and values per entry (laid out in tiles of 16 positions, see
+``cache.layout``), and every request has one block table per group. Pages are taken when
 a request's tokens cross a page's edge, given back when the request is closed,
 and, in a group with a window, as soon as every position on them is older than
 any later query can see. Nothing is cleared on reuse: lengths, not contents,
@@ -19,6 +19,7 @@ from typing import Dict, Hashable, List, Optional, Sequence
 import torch
 
 from ..parts.base import CacheNeed, PagedKVNeed, StateNeed
+from .layout import check_sizes, key_page_shape, value_page_shape
 from .pages import OutOfPages, PagePool, SlotPool
 
 RELEASED = -1  # block-table entry of a page that a window has passed
@@ -74,6 +75,8 @@ class CacheManager:
                  device: Optional[torch.device] = None):
         if page_size <= 0:
             raise ValueError("page_size must be positive")
+        if device is not None:
+            check_sizes(page_size, 1)   # device pages are tiled by 16 positions; the bookkeeping alone is not
         if len(needs) != len(reads):
             raise ValueError("one need and one read source per run entry")
         self.page_size = page_size
@@ -98,10 +101,9 @@ class CacheManager:
                 group.entries.append(entry)
                 k = v = None
                 if device is not None:
-                    # Values are kept transposed so that one dim's keys are contiguous for the MFMA kernels.
-                    # Zeroed once: a kernel may read a whole page whose tail was never written.
-                    k = torch.zeros((num_pages, need.kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
-                    v = torch.zeros((num_pages, need.kv_heads, need.head_dim, page_size), dtype=dtype, device=device)
+                    # Zeroed once: a kernel may read a whole tile whose tail was never written.
+                    k = torch.zeros(key_page_shape(num_pages, need.kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
+                    v = torch.zeros(value_page_shape(num_pages, need.kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
                 self._bindings[entry] = PagedBinding(group.index, need, k, v, owned=True)
             elif isinstance(need, StateNeed):
                 state = None

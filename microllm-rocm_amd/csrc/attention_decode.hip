@@ -5,8 +5,9 @@
 // of the visible keys. A wave walks pairs of 16-key tiles. Scores are computed transposed,
 // S^T = K . Q^T (v_mfma_f32_16x16x32_bf16: A = 16 keys x 32 dims straight from the page, B = Q^T), so
 // that a lane ends up with 8 keys of one head: exactly the B operand of O^T = V^T . P^T, whose A operand
-// comes straight from the value pages, which are stored transposed ([page, kv_head, dim, key]) for this.
-// Nothing passes through LDS but the final join of the 4 waves.
+// comes straight from the value pages. Pages are laid out in MFMA order (cache_layout.h), so every load of
+// a wave is one contiguous piece. Nothing passes through LDS but the final join of the 4 waves.
+#include "cache_layout.h"
 #include "common.h"
 #include "microllm_hip.h"
 
@@ -33,9 +34,13 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
     float* __restrict__ part_ml, float scale, int window, int heads, int kv_heads, int page_size, int n_splits) {
     constexpr int HD = HD_TILES * 16;
     constexpr int K_STEPS = (HD + 31) / 32;
-    __shared__ float o_shared[16][HD + 4];
-    __shared__ float m_shared[16];
-    __shared__ float l_shared[16];
+    constexpr int K_CHUNKS = HD / 8;
+    // Join buffer: one slot per wave when it fits, else one slot that the waves enter in turn.
+    constexpr bool kParallelJoin = HD_TILES <= 8;
+    constexpr int kSlots = kParallelJoin ? kDecodeWaves : 1;
+    __shared__ float o_shared[kSlots][16][HD + 4];
+    __shared__ float m_shared[kSlots][16];
+    __shared__ float l_shared[kSlots][16];
 
     const int token = blockIdx.x;
     const int group = heads / kv_heads;
@@ -45,6 +50,7 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
     const int split = blockIdx.z;
     const int head0 = kv_head * group + chunk * 16;
     const int heads_here = min(16, group - chunk * 16);
+    const CacheLayout layout(kv_heads, page_size, HD);
 
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
@@ -79,43 +85,47 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
     for (int d = 0; d < HD_TILES; ++d) o_acc[d] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     float running_max = -INFINITY, running_sum = 0.0f;
 
-    for (int pair = pair_begin + wave; pair < pair_end; pair += kDecodeWaves) {
+    // The pages of a pair's two tiles are looked up one iteration ahead of their use.
+    auto page_of = [&](int tile_key) -> int {
+        return (tile_key <= position && tile_key + 15 >= low) ? table[tile_key / page_size] : -1;
+    };
+    int pair = pair_begin + wave;
+    int next_page[2] = {-1, -1};
+    if (pair < pair_end) {
+        next_page[0] = page_of(pair * 32);
+        next_page[1] = page_of(pair * 32 + 16);
+    }
+    for (; pair < pair_end; pair += kDecodeWaves) {
         const int key0 = pair * 32;
-        bool tile_live[2];
-        int64_t k_row[2], v_row[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const int tile_key = key0 + 16 * t;
-            tile_live[t] = tile_key <= position && tile_key + 15 >= low;
-            k_row[t] = v_row[t] = 0;
-            if (tile_live[t]) {
-                const int64_t page = table[tile_key / page_size];
-                const int offset = tile_key % page_size;
-                k_row[t] = ((page * kv_heads + kv_head) * page_size + offset + col) * HD;       // key `col` of the tile
-                v_row[t] = ((page * kv_heads + kv_head) * HD + col) * page_size + offset;       // dim `col` of a dim tile
-            }
+        const int page[2] = {next_page[0], next_page[1]};
+        if (pair + kDecodeWaves < pair_end) {
+            next_page[0] = page_of((pair + kDecodeWaves) * 32);
+            next_page[1] = page_of((pair + kDecodeWaves) * 32 + 16);
         }
-        // Keys: A operand, row = key, 8 dims per lane.
+        // Keys: A operand, row = key `col` of the tile, 8 dims (chunk 4 * ks + quad) per lane.
+        // Values: A operand of the second product, row = dim `col` of a dim tile, k-slots = keys 4*quad..+3 of
+        // tile 0, then of tile 1.
         Frag8 k_frag[2][K_STEPS];
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int ks = 0; ks < K_STEPS; ++ks) {
-                const int dim = ks * 32 + quad * 8;
-                k_frag[t][ks].raw = make_uint4(0, 0, 0, 0);
-                if (tile_live[t] && dim < HD)
-                    k_frag[t][ks].raw = *reinterpret_cast<const uint4*>(k_cache + k_row[t] + dim);
-            }
-        // Values: A operand of the second product, row = dim, k-slots = keys 4*quad..+3 of tile 0, then of tile 1.
         Frag8 v_frag[HD_TILES];
 #pragma unroll
-        for (int d = 0; d < HD_TILES; ++d) {
-            v_frag[d].raw = make_uint4(0, 0, 0, 0);
+        for (int d = 0; d < HD_TILES; ++d) v_frag[d].raw = make_uint4(0, 0, 0, 0);
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
-                if (tile_live[t])
-                    v_frag[d].h[t] = *reinterpret_cast<const bf16x4*>(
-                        v_cache + v_row[t] + static_cast<int64_t>(d) * 16 * page_size + quad * 4);
+        for (int t = 0; t < 2; ++t) {
+            const int offset = (key0 + 16 * t) % page_size;
+            const bf16* k_tile = k_cache + layout.k_tile(max(page[t], 0), kv_head, offset / 16) + col * 8;
+            const bf16* v_tile = v_cache + layout.v_tile(max(page[t], 0), kv_head, offset / 16) + (quad * 16 + col) * 4;
+#pragma unroll
+            for (int ks = 0; ks < K_STEPS; ++ks) {
+                const int piece = ks * 4 + quad;
+                k_frag[t][ks].raw = make_uint4(0, 0, 0, 0);
+                if (page[t] >= 0 && piece < K_CHUNKS)
+                    k_frag[t][ks].raw = *reinterpret_cast<const uint4*>(k_tile + piece * 128);
+            }
+            if (page[t] >= 0) {
+#pragma unroll
+                for (int d = 0; d < HD_TILES; ++d)
+                    v_frag[d].h[t] = *reinterpret_cast<const bf16x4*>(v_tile + d * 256);
+            }
         }
 
         // S^T = K . Q^T: lane holds head `col`, keys 4*quad + i of each tile.
@@ -168,43 +178,65 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
         }
     }
 
-    // Join the 4 waves, one after the other, in LDS: o_shared[head][dim].
-    for (int w = 0; w < kDecodeWaves; ++w) {
-        __syncthreads();
-        if (wave != w) continue;
-        float old_max = w == 0 ? -INFINITY : m_shared[col];
-        float old_sum = w == 0 ? 0.0f : l_shared[col];
-        const float new_max = fmaxf(old_max, running_max);
-        const float keep = (old_max == -INFINITY) ? 0.0f : __expf(old_max - new_max);
-        const float add = (running_max == -INFINITY) ? 0.0f : __expf(running_max - new_max);
+    // Join the 4 waves in LDS: o_shared[slot][head][dim]; lane holds head `col`, dims d*16 + quad*4 + i.
+    if (kParallelJoin) {
 #pragma unroll
         for (int d = 0; d < HD_TILES; ++d)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int dim = d * 16 + quad * 4 + i;
-                const float before = w == 0 ? 0.0f : o_shared[col][dim];
-                o_shared[col][dim] = before * keep + o_acc[d][i] * add;
-            }
+            for (int i = 0; i < 4; ++i) o_shared[wave][col][d * 16 + quad * 4 + i] = o_acc[d][i];
         if (quad == 0) {
-            m_shared[col] = new_max;
-            l_shared[col] = old_sum * keep + running_sum * add;
+            m_shared[wave][col] = running_max;
+            l_shared[wave][col] = running_sum;
         }
+        __syncthreads();
+    } else {
+        for (int w = 0; w < kDecodeWaves; ++w) {
+            __syncthreads();
+            if (wave != w) continue;
+            const float old_max = w == 0 ? -INFINITY : m_shared[0][col];
+            const float old_sum = w == 0 ? 0.0f : l_shared[0][col];
+            const float new_max = fmaxf(old_max, running_max);
+            const float keep = (old_max == -INFINITY) ? 0.0f : __expf(old_max - new_max);
+            const float add = (running_max == -INFINITY) ? 0.0f : __expf(running_max - new_max);
+#pragma unroll
+            for (int d = 0; d < HD_TILES; ++d)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int dim = d * 16 + quad * 4 + i;
+                    const float before = w == 0 ? 0.0f : o_shared[0][col][dim];
+                    o_shared[0][col][dim] = before * keep + o_acc[d][i] * add;
+                }
+            if (quad == 0) {
+                m_shared[0][col] = new_max;
+                l_shared[0][col] = old_sum * keep + running_sum * add;
+            }
+        }
+        __syncthreads();
     }
-    __syncthreads();
 
     for (int index = threadIdx.x; index < heads_here * HD; index += kDecodeThreads) {
         const int h = index / HD, dim = index % HD;
+        float top = m_shared[0][h];
+#pragma unroll
+        for (int w = 1; w < kSlots; ++w) top = fmaxf(top, m_shared[w][h]);
+        float total = 0.0f, sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kSlots; ++w) {
+            const float m = m_shared[w][h];
+            const float weight = (m == -INFINITY) ? 0.0f : __expf(m - top);
+            total += weight * o_shared[w][h][dim];
+            sum += weight * l_shared[w][h];
+        }
         const int64_t row = static_cast<int64_t>(token) * heads + head0 + h;
         if (n_splits == 1) {
-            out[row * HD + dim] = from_float<bf16>(o_shared[h][dim] / l_shared[h]);
+            out[row * HD + dim] = from_float<bf16>(total / sum);
         } else {
-            part_o[(row * n_splits + split) * HD + dim] = o_shared[h][dim];
+            part_o[(row * n_splits + split) * HD + dim] = total;
+            if (dim == 0) {
+                part_ml[(row * n_splits + split) * 2 + 0] = top;
+                part_ml[(row * n_splits + split) * 2 + 1] = sum;
+            }
         }
-    }
-    if (n_splits > 1 && threadIdx.x < heads_here) {
-        const int64_t row = static_cast<int64_t>(token) * heads + head0 + threadIdx.x;
-        part_ml[(row * n_splits + split) * 2 + 0] = m_shared[threadIdx.x];
-        part_ml[(row * n_splits + split) * 2 + 1] = l_shared[threadIdx.x];
     }
 }
 

@@ -2,6 +2,7 @@
 // head size can take, and the float32 path's only attention. Keys are reduced in tiles of 64
 // aligned to absolute positions, with a running maximum and sum, so a query's result depends
 // on its position and its request's keys only: not on the step's cut, the batch or the pages.
+#include "cache_layout.h"
 #include "common.h"
 #include "microllm_hip.h"
 
@@ -19,6 +20,7 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_kernel(
     __shared__ float q_shared[kRowwiseMaxHeadDim];
     __shared__ float p_shared[kWave];
     __shared__ int64_t v_shared[kWave];
+    const CacheLayout layout(kv_heads, page_size, head_dim);
 
     const int token = blockIdx.x;
     const int head = blockIdx.y;
@@ -47,10 +49,10 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_kernel(
         if (visible) {
             const int64_t page = table[key / page_size];
             const int offset = key % page_size;
-            const T* k_row = k_cache + ((page * kv_heads + kv_head) * page_size + offset) * head_dim;
-            v_column = (page * kv_heads + kv_head) * head_dim * page_size + offset;  // value pages are [.., dim, offset]
+            const T* k_tile = k_cache + layout.k_tile(page, kv_head, offset / 16);
+            v_column = layout.v_tile(page, kv_head, offset / 16) + CacheLayout::v_in_tile(offset % 16, 0);
             float dot = 0.0f;
-            for (int d = 0; d < head_dim; ++d) dot += q_shared[d] * to_float(k_row[d]);
+            for (int d = 0; d < head_dim; ++d) dot += q_shared[d] * to_float(k_tile[CacheLayout::k_in_tile(offset % 16, d)]);
             score = dot * scale;
         }
         const float new_max = fmaxf(running_max, wave_max(score));  // every tile holds a visible key
@@ -70,8 +72,8 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_kernel(
             const int d = lane + i * kWave;
             if (d < head_dim) {
                 float value = acc[i] * rescale;
-                for (int j = first; j <= last; ++j)
-                    value += p_shared[j] * to_float(v_cache[v_shared[j] + static_cast<int64_t>(d) * page_size]);
+                const int v_dim = ((d / 16) * 64 + d % 16) * 4;   // CacheLayout::v_in_tile(0, d)
+                for (int j = first; j <= last; ++j) value += p_shared[j] * to_float(v_cache[v_shared[j] + v_dim]);
                 acc[i] = value;
             }
         }
@@ -97,7 +99,8 @@ extern "C" int mll_paged_attention_rowwise(const void* q, int dtype, const void*
                                            int head_dim, int page_size, hipStream_t stream) {
     MLL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "paged_attention: heads must divide into kv_heads groups");
     MLL_REQUIRE(head_dim > 0 && head_dim <= kRowwiseMaxHeadDim, "paged_attention: head_dim must be in [1, 512]");
-    MLL_REQUIRE(page_size > 0 && table_width > 0, "paged_attention: page_size and table width must be positive");
+    MLL_REQUIRE(page_size > 0 && page_size % 16 == 0 && table_width > 0,
+                "paged_attention: page_size must be a multiple of 16 and the table width positive");
     MLL_REQUIRE(heads <= 65535, "paged_attention: more than 65535 heads");
     if (n_tokens == 0) return 0;
     const dim3 grid(n_tokens, heads);

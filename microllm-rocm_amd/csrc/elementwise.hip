@@ -1,5 +1,6 @@
 // Row-wise kernels around the matrix products: embedding gather, RMSNorm with the residual
 // sum, bias + rotation + page write of the attention projections, and SiLU-mul.
+#include "cache_layout.h"
 #include "common.h"
 #include "microllm_hip.h"
 
@@ -32,6 +33,7 @@ __global__ void embedding_kernel(const W* __restrict__ table, const int32_t* __r
 // sums, a butterfly inside each wave, then the waves in ascending order.
 template <typename T, typename D>
 __global__ void rms_norm_kernel(float* __restrict__ h, const D* __restrict__ delta,
+                                int n_partials, int64_t partial_stride,
                                 const int32_t* __restrict__ rows, const float* __restrict__ weight,
                                 float eps, T* __restrict__ out, int width, int write_h) {
     __shared__ float scratch[16];
@@ -44,7 +46,11 @@ __global__ void rms_norm_kernel(float* __restrict__ h, const D* __restrict__ del
     float partial = 0.0f;
     for (int column = threadIdx.x; column < width; column += blockDim.x) {
         float value = h_row[column];
-        if (delta_row) value += to_float(delta_row[column]);
+        if (delta_row) {
+            float sum = to_float(delta_row[column]);
+            for (int part = 1; part < n_partials; ++part) sum += to_float(delta_row[part * partial_stride + column]);
+            value += sum;
+        }
         if (write_h) h_row[column] = value;
         partial += value * value;
     }
@@ -52,8 +58,78 @@ __global__ void rms_norm_kernel(float* __restrict__ h, const D* __restrict__ del
     const float inverse_rms = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
     for (int column = threadIdx.x; column < width; column += blockDim.x) {
         float value = h_row[column];  // already holds the sum when write_h
-        if (delta_row && !write_h) value += to_float(delta_row[column]);
+        if (delta_row && !write_h) {
+            float sum = to_float(delta_row[column]);
+            for (int part = 1; part < n_partials; ++part) sum += to_float(delta_row[part * partial_stride + column]);
+            value += sum;
+        }
         out_row[column] = from_float<T>(value * inverse_rms * weight[column]);
+    }
+}
+
+// The same for rows of float4: one pass, the row kept in registers between the sum of squares and the
+// scaling. Taken when the width is a multiple of 4 and at most 4 * CHUNKS * blockDim.x.
+template <typename T, typename D, int CHUNKS>
+__global__ void rms_norm_vec4_kernel(float* __restrict__ h, const D* __restrict__ delta,
+                                     const int32_t* __restrict__ rows, const float* __restrict__ weight,
+                                     float eps, T* __restrict__ out, int width, int write_h) {
+    __shared__ float scratch[16];
+    const int index = blockIdx.x;
+    const int64_t source = rows ? rows[index] : index;
+    float* h_row = h + source * width;
+    const D* delta_row = delta ? delta + source * width : nullptr;
+    T* out_row = out + static_cast<int64_t>(index) * width;
+    const int quads = width / 4;
+
+    float4 value[CHUNKS];
+    float partial = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int q = threadIdx.x + c * blockDim.x;
+        value[c] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (q < quads) {
+            value[c] = reinterpret_cast<const float4*>(h_row)[q];
+            if (delta_row) {
+                value[c].x += to_float(delta_row[4 * q + 0]);
+                value[c].y += to_float(delta_row[4 * q + 1]);
+                value[c].z += to_float(delta_row[4 * q + 2]);
+                value[c].w += to_float(delta_row[4 * q + 3]);
+            }
+            if (write_h) reinterpret_cast<float4*>(h_row)[q] = value[c];
+            partial += value[c].x * value[c].x + value[c].y * value[c].y + value[c].z * value[c].z + value[c].w * value[c].w;
+        }
+    }
+    const float total = block_sum(partial, scratch);
+    const float inverse_rms = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int q = threadIdx.x + c * blockDim.x;
+        if (q < quads) {
+            const float4 w = reinterpret_cast<const float4*>(weight)[q];
+            out_row[4 * q + 0] = from_float<T>(value[c].x * inverse_rms * w.x);
+            out_row[4 * q + 1] = from_float<T>(value[c].y * inverse_rms * w.y);
+            out_row[4 * q + 2] = from_float<T>(value[c].z * inverse_rms * w.z);
+            out_row[4 * q + 3] = from_float<T>(value[c].w * inverse_rms * w.w);
+        }
+    }
+}
+
+template <typename T, typename D>
+static void launch_rms_norm(float* h, const D* delta, int n_partials, int64_t partial_stride, const int32_t* rows,
+                            const float* weight, float eps, T* out, int n_rows, int width, int write_h,
+                            hipStream_t stream) {
+    const bool aligned = width % 4 == 0 && n_partials == 1 &&
+                         reinterpret_cast<uintptr_t>(h) % 16 == 0 && reinterpret_cast<uintptr_t>(weight) % 16 == 0;
+    const int quads = width / 4;
+    if (aligned && quads <= 1024) {
+        const int threads = max(64, (quads + 63) / 64 * 64);
+        rms_norm_vec4_kernel<T, D, 1><<<n_rows, threads, 0, stream>>>(h, delta, rows, weight, eps, out, width, write_h);
+    } else if (aligned && quads <= 4096) {
+        rms_norm_vec4_kernel<T, D, 4><<<n_rows, 1024, 0, stream>>>(h, delta, rows, weight, eps, out, width, write_h);
+    } else {
+        const int threads = width >= 2048 ? 512 : 256;
+        rms_norm_kernel<T, D><<<n_rows, threads, 0, stream>>>(h, delta, n_partials, partial_stride, rows, weight, eps,
+                                                              out, width, write_h);
     }
 }
 
@@ -70,7 +146,8 @@ __global__ void residual_add_kernel(float* __restrict__ h, const T* __restrict__
 constexpr int kMaxHeadDim = 512;
 
 template <typename In, typename T>
-__global__ void qkv_rope_store_kernel(const In* __restrict__ qkv, const float* __restrict__ bias,
+__global__ void qkv_rope_store_kernel(const In* __restrict__ qkv, int n_partials, int64_t partial_stride,
+                                      const float* __restrict__ bias,
                                       const int32_t* __restrict__ positions,
                                       const int32_t* __restrict__ slot_mapping,
                                       const double* __restrict__ inv_freq, int n_freq,
@@ -80,6 +157,8 @@ __global__ void qkv_rope_store_kernel(const In* __restrict__ qkv, const float* _
     __shared__ float sin_table[kMaxHeadDim / 2];
     const int token = blockIdx.x;
     const int position = positions[token];
+    const int heads_per_block = gridDim.y == 1 ? heads + 2 * kv_heads : max(1, static_cast<int>(blockDim.x) / (head_dim / 2));
+    const int first_head = blockIdx.y * heads_per_block;
     for (int index = threadIdx.x; index < n_freq; index += blockDim.x) {
         const double angle = static_cast<double>(position) * inv_freq[index];
         cos_table[index] = static_cast<float>(cos(angle));
@@ -93,9 +172,11 @@ __global__ void qkv_rope_store_kernel(const In* __restrict__ qkv, const float* _
     const int slot = slot_mapping ? slot_mapping[token] : -1;
     const int64_t page = slot >= 0 ? slot / page_size : 0;
     const int offset = slot >= 0 ? slot % page_size : 0;
+    const CacheLayout layout(kv_heads, page_size, head_dim);
 
-    for (int item = threadIdx.x; item < total_heads * half; item += blockDim.x) {
-        const int head = item / half;
+    const int block_heads = min(heads_per_block, total_heads - first_head);
+    for (int item = threadIdx.x; item < block_heads * half; item += blockDim.x) {
+        const int head = first_head + item / half;
         const int pair = item % half;
         const bool is_value = head >= heads + kv_heads;
         int first, second;
@@ -112,6 +193,10 @@ __global__ void qkv_rope_store_kernel(const In* __restrict__ qkv, const float* _
         const int column = head * head_dim;
         float x1 = to_float(qkv[in_row + column + first]);
         float x2 = to_float(qkv[in_row + column + second]);
+        for (int part = 1; part < n_partials; ++part) {
+            x1 += to_float(qkv[part * partial_stride + in_row + column + first]);
+            x2 += to_float(qkv[part * partial_stride + in_row + column + second]);
+        }
         if (bias) {
             x1 += bias[column + first];
             x2 += bias[column + second];
@@ -128,14 +213,12 @@ __global__ void qkv_rope_store_kernel(const In* __restrict__ qkv, const float* _
             q_row[second] = from_float<T>(y2);
         } else if (slot >= 0 && !is_value) {
             const int kv_head = head - heads;
-            T* row = k_cache + ((page * kv_heads + kv_head) * page_size + offset) * head_dim;
-            row[first] = from_float<T>(y1);
-            row[second] = from_float<T>(y2);
-        } else if (slot >= 0) {  // value pages are transposed: [page, kv_head, dim, offset]
+            k_cache[layout.k_at(page, kv_head, offset, first)] = from_float<T>(y1);
+            k_cache[layout.k_at(page, kv_head, offset, second)] = from_float<T>(y2);
+        } else if (slot >= 0) {
             const int kv_head = head - heads - kv_heads;
-            T* column = v_cache + (page * kv_heads + kv_head) * head_dim * page_size + offset;
-            column[static_cast<int64_t>(first) * page_size] = from_float<T>(y1);
-            column[static_cast<int64_t>(second) * page_size] = from_float<T>(y2);
+            v_cache[layout.v_at(page, kv_head, offset, first)] = from_float<T>(y1);
+            v_cache[layout.v_at(page, kv_head, offset, second)] = from_float<T>(y2);
         }
     }
 }
@@ -181,22 +264,23 @@ int mll_embedding(const void* table, int table_dtype, const int32_t* ids, float*
     return check_launch("embedding");
 }
 
-int mll_rms_norm(float* h, const void* delta, int delta_dtype, const int32_t* rows, const float* weight, float eps,
+int mll_rms_norm(float* h, const void* delta, int delta_dtype, int n_partials, int64_t partial_stride,
+                 const int32_t* rows, const float* weight, float eps,
                  void* out, int dtype, int n_rows, int width, int write_h, hipStream_t stream) {
+    MLL_REQUIRE(n_partials >= 1, "rms_norm: the delta needs at least one part");
     MLL_REQUIRE(n_rows >= 0 && width > 0, "rms_norm: sizes must be positive");
     MLL_REQUIRE(eps > 0.0f, "rms_norm: eps must be positive");
     MLL_REQUIRE(!(write_h && rows), "rms_norm: cannot write h through a row selection");
     if (n_rows == 0) return 0;
-    const int threads = width >= 2048 ? 512 : 256;
     if (dtype == kF32 && delta_dtype == kF32) {
-        rms_norm_kernel<float, float><<<n_rows, threads, 0, stream>>>(
-            h, static_cast<const float*>(delta), rows, weight, eps, static_cast<float*>(out), width, write_h);
+        launch_rms_norm<float, float>(h, static_cast<const float*>(delta), n_partials, partial_stride, rows, weight, eps,
+                                      static_cast<float*>(out), n_rows, width, write_h, stream);
     } else if (dtype == kBF16 && delta_dtype == kF32) {
-        rms_norm_kernel<bf16, float><<<n_rows, threads, 0, stream>>>(
-            h, static_cast<const float*>(delta), rows, weight, eps, static_cast<bf16*>(out), width, write_h);
+        launch_rms_norm<bf16, float>(h, static_cast<const float*>(delta), n_partials, partial_stride, rows, weight, eps,
+                                     static_cast<bf16*>(out), n_rows, width, write_h, stream);
     } else if (dtype == kBF16 && delta_dtype == kBF16) {
-        rms_norm_kernel<bf16, bf16><<<n_rows, threads, 0, stream>>>(
-            h, static_cast<const bf16*>(delta), rows, weight, eps, static_cast<bf16*>(out), width, write_h);
+        launch_rms_norm<bf16, bf16>(h, static_cast<const bf16*>(delta), n_partials, partial_stride, rows, weight, eps,
+                                    static_cast<bf16*>(out), n_rows, width, write_h, stream);
     } else {
         return fail("rms_norm: unsupported combination of output and delta dtypes");
     }
@@ -217,31 +301,36 @@ int mll_residual_add(float* h, const void* delta, int dtype, int n_rows, int wid
     return check_launch("residual_add");
 }
 
-int mll_qkv_rope_store(const void* qkv, int in_dtype, int dtype, const float* bias, const int32_t* positions,
+int mll_qkv_rope_store(const void* qkv, int in_dtype, int n_partials, int64_t partial_stride, int dtype,
+                       const float* bias, const int32_t* positions,
                        const int32_t* slot_mapping, const double* inv_freq, int n_freq,
                        void* q_out, void* k_cache, void* v_cache,
                        int n_tokens, int heads, int kv_heads, int head_dim, int page_size,
                        hipStream_t stream) {
     MLL_REQUIRE(heads > 0 && kv_heads >= 0 && head_dim > 0, "qkv_rope_store: sizes must be positive");
+    MLL_REQUIRE(n_partials >= 1, "qkv_rope_store: the input needs at least one part");
     MLL_REQUIRE(head_dim % 2 == 0 && head_dim <= kMaxHeadDim, "qkv_rope_store: head_dim must be even and at most 512");
     MLL_REQUIRE(n_freq >= 0 && 2 * n_freq <= head_dim, "qkv_rope_store: rotary part exceeds head_dim");
     MLL_REQUIRE(inv_freq != nullptr || n_freq == 0, "qkv_rope_store: n_freq without a frequency table");
-    MLL_REQUIRE(slot_mapping == nullptr || (k_cache && v_cache && page_size > 0),
-                "qkv_rope_store: slot_mapping needs both caches and a page size");
+    MLL_REQUIRE(slot_mapping == nullptr || (k_cache && v_cache && page_size > 0 && page_size % 16 == 0),
+                "qkv_rope_store: slot_mapping needs both caches and a page size that is a multiple of 16");
     if (n_tokens == 0) return 0;
+    // A block takes as many heads of one token as give its 256 threads one pair each.
+    const int heads_per_block = max(1, 256 / (head_dim / 2));
+    const dim3 grid(n_tokens, (heads + 2 * kv_heads + heads_per_block - 1) / heads_per_block);
     if (dtype == kF32 && in_dtype == kF32) {
-        qkv_rope_store_kernel<float, float><<<n_tokens, 256, 0, stream>>>(
-            static_cast<const float*>(qkv), bias, positions, slot_mapping, inv_freq, n_freq,
+        qkv_rope_store_kernel<float, float><<<grid, 256, 0, stream>>>(
+            static_cast<const float*>(qkv), n_partials, partial_stride, bias, positions, slot_mapping, inv_freq, n_freq,
             static_cast<float*>(q_out), static_cast<float*>(k_cache), static_cast<float*>(v_cache),
             heads, kv_heads, head_dim, page_size);
     } else if (dtype == kBF16 && in_dtype == kF32) {
-        qkv_rope_store_kernel<float, bf16><<<n_tokens, 256, 0, stream>>>(
-            static_cast<const float*>(qkv), bias, positions, slot_mapping, inv_freq, n_freq,
+        qkv_rope_store_kernel<float, bf16><<<grid, 256, 0, stream>>>(
+            static_cast<const float*>(qkv), n_partials, partial_stride, bias, positions, slot_mapping, inv_freq, n_freq,
             static_cast<bf16*>(q_out), static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache),
             heads, kv_heads, head_dim, page_size);
     } else if (dtype == kBF16 && in_dtype == kBF16) {
-        qkv_rope_store_kernel<bf16, bf16><<<n_tokens, 256, 0, stream>>>(
-            static_cast<const bf16*>(qkv), bias, positions, slot_mapping, inv_freq, n_freq,
+        qkv_rope_store_kernel<bf16, bf16><<<grid, 256, 0, stream>>>(
+            static_cast<const bf16*>(qkv), n_partials, partial_stride, bias, positions, slot_mapping, inv_freq, n_freq,
             static_cast<bf16*>(q_out), static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache),
             heads, kv_heads, head_dim, page_size);
     } else {

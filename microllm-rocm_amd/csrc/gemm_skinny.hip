@@ -1,0 +1,207 @@
+// Matrix products with few rows (decoding): C = A . W^T for bfloat16 A [M <= 64, K] and a weight that was
+// packed once, at load time, into the order the MFMA consumes it, so that a wave streams its 16 rows of W as
+// consecutive 1 KB pieces. The kernel is bound by reading W once from HBM.
+//
+// Packed layout: [N/16][K/32][quad 0..3][row 0..15][8 elements]; lane (row + 16 * quad) of a wave reads its
+// 16 bytes of piece (n_tile, k_step) at byte offset lane * 16: the A operand of v_mfma_f32_16x16x32_bf16.
+// The product is computed transposed (C^T = W . A^T): the activations are the B operand, 16 rows per tile.
+// A workgroup owns NT tiles of W; its waves (1 to 16, more when W has few rows, so that the GPU is filled)
+// take the k steps in turn and their sums are added in wave order through LDS: the result is the same in
+// every run and, for up to 16 rows, does not depend on the other rows of A.
+#include "common.h"
+#include "microllm_hip.h"
+
+namespace mll {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
+
+
+union Piece {
+    bf16x8 v;
+    uintx4 raw;
+};
+
+__device__ inline float silu_f(float value) {
+    return value / (1.0f + __expf(-value));
+}
+
+// EPILOGUE: 0 = float32 [M, N]; 1 = bfloat16 [M, N]; 2 = bfloat16 [M, N / 2] = silu(even rows of W) * (odd rows).
+template <int MT, int NT, int EPILOGUE>
+__global__ __launch_bounds__(1024) void gemm_skinny_kernel(
+    const bf16* __restrict__ a, const bf16* __restrict__ w_packed, void* __restrict__ out,
+    int m, int n, int k, int n_tiles, int k_steps) {
+    extern __shared__ float reduce_shared[];   // [waves][NT * MT][64 lanes][4]
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int waves = blockDim.x / kWave;
+    const int col = lane % 16, quad = lane / 16;
+    const int tile0 = blockIdx.x * NT;
+
+    floatx4 acc[NT][MT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    const bf16* w_ptr[NT];
+    bool w_live[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        w_live[nt] = tile0 + nt < n_tiles;
+        w_ptr[nt] = w_packed + static_cast<int64_t>(w_live[nt] ? tile0 + nt : tile0) * k_steps * 512 + lane * 8;
+    }
+    const bf16* a_ptr[MT];
+    bool a_live[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int row = mt * 16 + col;
+        a_live[mt] = row < m;
+        a_ptr[mt] = a + static_cast<int64_t>(a_live[mt] ? row : 0) * k + quad * 8;
+    }
+
+    // A wave takes DEPTH consecutive k steps at a time, then skips what the other waves take. All loads of
+    // the DEPTH steps are issued before the first product, so that a wave keeps several KB of W in flight.
+    constexpr int DEPTH = (MT + NT <= 2) ? 8 : ((MT + NT <= 4) ? 4 : 2);
+    for (int ks = wave * DEPTH; ks < k_steps; ks += waves * DEPTH) {
+        Piece w_piece[DEPTH][NT];
+        Piece a_piece[DEPTH][MT];
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) {
+            const bool live = ks + u < k_steps;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                w_piece[u][nt].raw = uintx4{0u, 0u, 0u, 0u};
+                if (live && w_live[nt])
+                    w_piece[u][nt].raw = __builtin_nontemporal_load(
+                        reinterpret_cast<const uintx4*>(w_ptr[nt] + static_cast<int64_t>(ks + u) * 512));
+            }
+            const int k_offset = (ks + u) * 32;
+            const bool in_k = live && k_offset + quad * 8 < k;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                a_piece[u][mt].raw = uintx4{0u, 0u, 0u, 0u};
+                if (a_live[mt] && in_k) a_piece[u][mt].raw = *reinterpret_cast<const uintx4*>(a_ptr[mt] + k_offset);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_piece[u][nt].v, a_piece[u][mt].v, acc[nt][mt], 0, 0, 0);
+    }
+
+    // The waves' sums, added in wave order by wave 0.
+    if (waves > 1) {
+        floatx4* slots = reinterpret_cast<floatx4*>(reduce_shared);
+        if (wave > 0) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) slots[((wave - 1) * NT * MT + nt * MT + mt) * kWave + lane] = acc[nt][mt];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+        for (int other = 0; other < waves - 1; ++other)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[nt][mt] += slots[(other * NT * MT + nt * MT + mt) * kWave + lane];
+    }
+
+    // acc[nt][mt][i] = C[row mt*16 + col][column (tile0 + nt)*16 + quad*4 + i]
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int n_tile = tile0 + nt;
+        if (n_tile >= n_tiles) continue;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int row = mt * 16 + col;
+            if (row >= m) continue;
+            if (EPILOGUE == 0) {
+                float* target = static_cast<float*>(out) + static_cast<int64_t>(row) * n;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int column = n_tile * 16 + quad * 4 + i;
+                    if (column < n) target[column] = acc[nt][mt][i];
+                }
+            } else if (EPILOGUE == 1) {
+                bf16* target = static_cast<bf16*>(out) + static_cast<int64_t>(row) * n;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int column = n_tile * 16 + quad * 4 + i;
+                    if (column < n) target[column] = from_float<bf16>(acc[nt][mt][i]);
+                }
+            } else {
+                bf16* target = static_cast<bf16*>(out) + static_cast<int64_t>(row) * (n / 2);
+#pragma unroll
+                for (int i = 0; i < 4; i += 2) {
+                    const int column = n_tile * 8 + quad * 2 + i / 2;
+                    if (column < n / 2) target[column] = from_float<bf16>(silu_f(acc[nt][mt][i]) * acc[nt][mt][i + 1]);
+                }
+            }
+        }
+    }
+}
+
+template <int MT, int NT, int EPILOGUE>
+static void launch_one(const bf16* a, const bf16* w, void* out, int m, int n, int k, int n_tiles, int k_steps,
+                       hipStream_t stream) {
+    const int groups = (n_tiles + NT - 1) / NT;
+    // Waves per workgroup: enough that about eight thousand waves stream W, at most 16, and no more than
+    // there are pieces of k for them.
+    constexpr int DEPTH = (MT + NT <= 2) ? 8 : ((MT + NT <= 4) ? 4 : 2);
+    int waves = 1;
+    while (waves < 16 && groups * waves * 2 <= 8192 && waves * 2 * DEPTH <= k_steps) waves *= 2;
+    const size_t lds = waves > 1 ? static_cast<size_t>(waves - 1) * NT * MT * kWave * sizeof(floatx4) : 0;
+    gemm_skinny_kernel<MT, NT, EPILOGUE><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps);
+}
+
+template <int EPILOGUE>
+static int launch_skinny(const void* a, const void* w_packed, void* out, int m, int n, int k, hipStream_t stream) {
+    const int n_tiles = (n + 15) / 16;
+    const int k_steps = (k + 31) / 32;
+    const bf16* a_ = static_cast<const bf16*>(a);
+    const bf16* w_ = static_cast<const bf16*>(w_packed);
+    const int m_tiles = (m + 15) / 16;
+    // Few tiles of W: one per workgroup, so that the GPU is filled. Many: up to four, as many as A has.
+    const bool wide = n_tiles >= 2048;
+    switch (m_tiles) {
+        case 1: launch_one<1, 1, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream); break;
+        case 2:
+            if (wide) launch_one<2, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream);
+            else launch_one<2, 1, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream);
+            break;
+        case 3:
+            if (wide) launch_one<3, 4, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream);
+            else launch_one<3, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream);
+            break;
+        case 4:
+            if (wide) launch_one<4, 4, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream);
+            else launch_one<4, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream);
+            break;
+        default: return fail("gemm_skinny: more than 64 rows");
+    }
+    return check_launch("gemm_skinny");
+}
+
+}  // namespace mll
+
+using namespace mll;
+
+extern "C" int mll_gemm_skinny(const void* a, const void* w_packed, void* out, int epilogue, int m, int n, int k,
+                               hipStream_t stream) {
+    MLL_REQUIRE(m >= 0 && m <= 64, "gemm_skinny: takes at most 64 rows");
+    MLL_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_skinny: k must be a positive multiple of 8");
+    MLL_REQUIRE(epilogue != 2 || n % 2 == 0, "gemm_skinny: the gated epilogue needs an even number of weight rows");
+    if (m == 0) return 0;
+    switch (epilogue) {
+        case 0: return launch_skinny<0>(a, w_packed, out, m, n, k, stream);
+        case 1: return launch_skinny<1>(a, w_packed, out, m, n, k, stream);
+        case 2: return launch_skinny<2>(a, w_packed, out, m, n, k, stream);
+        default: return fail("gemm_skinny: unknown epilogue");
+    }
+}

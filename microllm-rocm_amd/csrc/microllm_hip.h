@@ -20,8 +20,10 @@ int mll_embedding(const void* table, int table_dtype, const int32_t* ids, float*
 // For i < n_rows, r = rows ? rows[i] : i:  v = h[r] + (delta ? delta[r] : 0);
 // if write_h, h[r] = v;  out[i] = v * rsqrt(mean(v^2) + eps) * weight.
 // h is the float32 residual stream; out has element type `dtype`, delta `delta_dtype`
-// (float32, or the same as out).
-int mll_rms_norm(float* h, const void* delta, int delta_dtype, const int32_t* rows, const float* weight, float eps,
+// (float32, or the same as out). delta may come in n_partials parts, partial_stride elements apart, which
+// are added in order (the partial sums of a matrix product that was split over k).
+int mll_rms_norm(float* h, const void* delta, int delta_dtype, int n_partials, int64_t partial_stride,
+                 const int32_t* rows, const float* weight, float eps,
                  void* out, int dtype, int n_rows, int width, int write_h, hipStream_t stream);
 
 // Adds a pending delta into the residual stream: h[r] += delta[r] for all rows.
@@ -33,8 +35,10 @@ int mll_residual_add(float* h, const void* delta, int dtype, int n_rows, int wid
 // slot = slot_mapping[t] (negative: not stored) addresses key pages [page, kv_head, offset, dim] and
 // value pages [page, kv_head, dim, offset] (transposed, so that a dim's keys are contiguous) with
 // page = slot / page_size, offset = slot % page_size.  k_cache / v_cache nullable together with slot_mapping. qkv has element type
-// `in_dtype` (float32, or the same as `dtype`); q_out and the pages have `dtype`.
-int mll_qkv_rope_store(const void* qkv, int in_dtype, int dtype, const float* bias, const int32_t* positions,
+// `in_dtype` (float32, or the same as `dtype`) and may come in n_partials parts, partial_stride elements
+// apart, which are added in order; q_out and the pages have `dtype`.
+int mll_qkv_rope_store(const void* qkv, int in_dtype, int n_partials, int64_t partial_stride, int dtype,
+                       const float* bias, const int32_t* positions,
                        const int32_t* slot_mapping, const double* inv_freq, int n_freq,
                        void* q_out, void* k_cache, void* v_cache,
                        int n_tokens, int heads, int kv_heads, int head_dim, int page_size,
@@ -69,6 +73,14 @@ int mll_silu_mul(const void* gate, const void* up, int64_t in_stride, void* out,
 // thread per output element, so a row's result does not depend on the other rows.
 int mll_gemm_f32(const float* a, const float* w, const float* bias, float* c,
                  int m, int n, int k, hipStream_t stream);
+
+// C = A . W^T for bfloat16 A [m <= 64, k] and a weight packed as [n/16][k/32][4][16][8] (zero padded):
+// element (row, col) of W sits at piece (row / 16, col / 32), position ((col % 32) / 8, row % 16, col % 8).
+// epilogue 0: float32 [m, n]; 1: bfloat16 [m, n]; 2: bfloat16 [m, n / 2] = silu(even weight rows' results) *
+// (odd rows' results). The order of additions is fixed by (n, k) and the number of 16-row tiles of A: the
+// same in every run, and for up to 16 rows independent of the other rows.
+int mll_gemm_skinny(const void* a, const void* w_packed, void* out, int epilogue, int m, int n, int k,
+                    hipStream_t stream);
 
 // Index of the first maximum of each row; a row that holds a non-finite value gives -1.
 int mll_argmax(const float* logits, int32_t* out, int n_rows, int vocab, hipStream_t stream);

@@ -52,10 +52,16 @@ class StepContext:
     host_slots: List[int] = field(default_factory=list)
     max_count: int = 0
     max_total: int = 0
+    planned_total: int = 0      # the longest request this step's launch shapes are planned for (>= max_total)
 
 
 class BatchBuilder:
-    """Packs a step's metadata and moves it to the device through one pinned staging buffer."""
+    """Packs a step's metadata and moves it to the device through one pinned staging buffer.
+
+    With ``fixed_width`` every block table is padded to that many columns, so that the layout of the packed
+    buffer depends on the numbers of tokens and requests alone: a step that is replayed from a HIP graph
+    finds every array at the address it had when the graph was captured.
+    """
 
     def __init__(self, cache: CacheManager, device: torch.device):
         self.cache = cache
@@ -75,7 +81,7 @@ class BatchBuilder:
         return self._staging, self._device_buffer
 
     def build(self, requests: Sequence[RequestCache], token_lists: Sequence[Sequence[int]],
-              wants: Sequence[Sequence[int]]) -> StepContext:
+              wants: Sequence[Sequence[int]], fixed_width: Optional[int] = None) -> StepContext:
         page_size = self.cache.page_size
         counts = [len(tokens) for tokens in token_lists]
         starts = [request.num_tokens for request in requests]
@@ -93,6 +99,10 @@ class BatchBuilder:
         tables, mappings, widths = [], [], []
         for group in self.cache.groups:
             width = max(1, max(len(request.pages[group.index]) for request in requests))
+            if fixed_width is not None:
+                if width > fixed_width:
+                    raise ValueError("a block table is wider than the fixed width")
+                width = fixed_width
             table = np.full((n_seqs, width), RELEASED, dtype=np.int32)
             for row, request in enumerate(requests):
                 pages = request.pages[group.index]
@@ -126,9 +136,11 @@ class BatchBuilder:
         for g, group in enumerate(self.cache.groups):
             paged.append(PagedView(piece_at(8 + 2 * g, (n_seqs, widths[g])), piece_at(9 + 2 * g),
                                    page_size, widths[g]))
+        longest = max(totals) if totals else 0
         return StepContext(
             n_tokens=n_tokens, n_seqs=n_seqs, tokens=piece_at(0), positions=piece_at(1), seq_of_token=piece_at(2),
             cu_tokens=piece_at(3), seq_start=piece_at(4), seq_total=piece_at(5), slots=piece_at(6),
             want_rows=piece_at(7) if want_rows.size else None, paged=paged,
             starts=list(starts), counts=counts, host_slots=[request.slot for request in requests],
-            max_count=max(counts) if counts else 0, max_total=max(totals) if totals else 0)
+            max_count=max(counts) if counts else 0, max_total=longest,
+            planned_total=longest if fixed_width is None else fixed_width * page_size)

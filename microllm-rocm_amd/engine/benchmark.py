@@ -13,6 +13,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import PagedBinding
+from ..parts.linear import Weight
 from ..sampling import Sampler, SamplingParams
 from .batch import StepEntry
 from .engine import Engine
@@ -83,12 +84,13 @@ def weight_bytes(engine: Engine) -> int:
     seen, total = set(), 0
     embedding_only = None
     model = engine.model
-    if model.embedding.table.data_ptr() != model.head.weight.data_ptr():
+    if model.embedding.table.data_ptr() != model.head.weight.tensor.data_ptr():
         embedding_only = model.embedding.table.data_ptr()
-    tensors = [model.final_norm.weight, model.head.weight]
+    tensors = [model.final_norm.weight, model.head.weight.tensor]
     for block in model.blocks:
         for part in block.parts():
             tensors += [value for value in vars(part).values() if isinstance(value, torch.Tensor)]
+            tensors += [value.tensor for value in vars(part).values() if isinstance(value, Weight)]
             position = getattr(part, "position", None)
             if position is not None:
                 tensors += [value for value in vars(position).values() if isinstance(value, torch.Tensor)]
@@ -118,12 +120,12 @@ def step_flops(engine: Engine, tokens: int) -> float:
     for block in engine.model.blocks:
         for part in block.parts():
             for name, value in vars(part).items():
-                if isinstance(value, torch.Tensor) and value.dim() == 2:
-                    flops += 2.0 * value.numel() * tokens
+                if isinstance(value, Weight):
+                    flops += 2.0 * value.tensor.numel() * tokens
         mixer = block.mixer
         if hasattr(mixer, "heads"):
             window = mixer.window or tokens
             pairs = sum(min(position + 1, window) for position in range(tokens))
             flops += 4.0 * mixer.heads * mixer.head_dim * pairs
-    flops += 2.0 * engine.model.head.weight.numel()
+    flops += 2.0 * engine.model.head.weight.tensor.numel()
     return flops

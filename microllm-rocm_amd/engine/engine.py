@@ -35,11 +35,25 @@ def parse_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
     return _DTYPES[dtype]
 
 
+MAX_GRAPH_REQUESTS = 256
+MIN_GRAPH_WIDTH = 16
+
+
+class _DecodeGraph:
+    """One captured decode step: its own metadata buffers, the graph and the logits it writes."""
+
+    def __init__(self, engine: "Engine", width: int):
+        self.builder = BatchBuilder(engine.cache, engine.device)
+        self.width = width
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.logits: Optional[torch.Tensor] = None
+
+
 class Engine:
     def __init__(self, spec: ModelSpec, tensors: Mapping[str, torch.Tensor], dtype: Union[str, torch.dtype] = "bfloat16",
                  device: Union[str, torch.device] = "cuda:0", page_size: int = 16,
                  max_tokens: Optional[int] = None, num_pages: Optional[int] = None, max_requests: int = 64,
-                 tensors_placed: bool = False):
+                 tensors_placed: bool = False, use_graphs: bool = True):
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU is visible; this engine has no CPU path")
         library.load()  # fail now, and loudly, if the kernels are missing and cannot be built
@@ -64,6 +78,11 @@ class Engine:
         self._bindings = self.cache.bindings()
         self._builder = BatchBuilder(self.cache, self.device)
         self.steps_run = 0
+        # Steps in which every request brings one token are replayed from HIP graphs, one per (number of
+        # requests, block-table width): the launches of a decode step cost more host time than GPU time.
+        self.use_graphs = use_graphs
+        self._graphs: Dict[tuple, "_DecodeGraph"] = {}
+        self.graph_replays = 0
 
     # ---- construction --------------------------------------------------------------------
     @classmethod
@@ -101,6 +120,36 @@ class Engine:
 
     def is_open(self, request_id: Hashable) -> bool:
         return request_id in self.cache.requests
+
+    # ---- decode steps from graphs ---------------------------------------------------------
+    def _graph_step(self, requests: List[RequestCache], entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        n = len(entries)
+        widest = max(len(pages) for request in requests for pages in request.pages) if self.cache.groups else 1
+        width = max(MIN_GRAPH_WIDTH, 1 << (max(widest, 1) - 1).bit_length())
+        key = (n, width)
+        state = self._graphs.get(key)
+        if state is None:
+            state = self._graphs[key] = _DecodeGraph(self, width)
+        tokens = [entry.tokens for entry in entries]
+        every_row = [[0]] * n   # the graph computes the logits of every row; the wanted ones are picked after
+        ctx = state.builder.build(requests, tokens, every_row, fixed_width=width)
+        if state.graph is None:
+            # Once eagerly (libraries create their handles and workspaces), then the capture. The step writes
+            # the same keys and values to the same slots each time, so running it twice changes nothing.
+            self.model.forward(ctx, self._bindings, ctx.want_rows)
+            torch.cuda.synchronize(self.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                state.logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
+            state.graph = graph
+        state.graph.replay()
+        self.graph_replays += 1
+        wanted = [index for index, entry in enumerate(entries) if len(entry.want) > 0]
+        if not wanted:
+            return None
+        if len(wanted) == n:
+            return state.logits
+        return state.logits[torch.tensor(wanted, device=self.device)]
 
     # ---- the step ------------------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry], reserved: bool = False) -> Optional[torch.Tensor]:
@@ -144,8 +193,11 @@ class Engine:
                 for request in taken:
                     self.cache.cancel_reservation(request)
                 raise
-        ctx = self._builder.build(requests, [entry.tokens for entry in entries], [entry.want for entry in entries])
-        logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
+        if self.use_graphs and len(entries) <= MAX_GRAPH_REQUESTS and all(len(entry.tokens) == 1 for entry in entries):
+            logits = self._graph_step(requests, entries)
+        else:
+            ctx = self._builder.build(requests, [entry.tokens for entry in entries], [entry.want for entry in entries])
+            logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
         for request, entry in zip(requests, entries):
             self.cache.commit(request, len(entry.tokens))
         self.steps_run += 1

@@ -74,11 +74,15 @@ def rms_norm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch
     _need(h.dim() == 2 and weight.dim() == 1 and weight.shape[0] == h.shape[1],
           "rms_norm weight must match the last dimension")
     width = h.shape[1]
-    delta_code = F32
+    delta_code, n_partials = F32, 1
     if delta is not None:
         _device_tensor(delta, "delta")
         _need(delta.dtype in (torch.float32, out_dtype), "delta must be float32 or have the output's dtype")
-        _need(tuple(delta.shape) == tuple(h.shape), "delta must have the residual stream's shape")
+        if delta.dim() == 3:   # partial sums [parts, rows, width], added in order
+            n_partials = delta.shape[0]
+            _need(n_partials >= 1 and tuple(delta.shape[1:]) == tuple(h.shape), "delta parts must have the residual stream's shape")
+        else:
+            _need(tuple(delta.shape) == tuple(h.shape), "delta must have the residual stream's shape")
         delta_code = _code(delta.dtype)
     if rows is not None:
         _device_tensor(rows, "row selection", torch.int32)
@@ -90,7 +94,8 @@ def rms_norm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch
         out = torch.empty((n_rows, width), dtype=out_dtype, device=h.device)
     _device_tensor(out, "norm output", out_dtype)
     _need(tuple(out.shape) == (n_rows, width), "norm output has the wrong shape")
-    _check(lib.mll_rms_norm(_ptr(h), _ptr(delta), delta_code, _ptr(rows), _ptr(weight), ctypes.c_float(eps), _ptr(out),
+    _check(lib.mll_rms_norm(_ptr(h), _ptr(delta), delta_code, n_partials, ctypes.c_int64(h.numel()), _ptr(rows),
+                            _ptr(weight), ctypes.c_float(eps), _ptr(out),
                             _code(out_dtype), n_rows, width, int(write_h), _stream()), lib)
     return out
 
@@ -115,9 +120,13 @@ def qkv_rope_store(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: t
     lib = library.load()
     _device_tensor(qkv, "qkv")
     _need(qkv.dtype in (torch.float32, out_dtype), "qkv must be float32 or have the output's dtype")
-    n_tokens = qkv.shape[0]
     total = (heads + 2 * kv_heads) * head_dim
-    _need(qkv.dim() == 2 and qkv.shape[1] == total, f"qkv must be [tokens, {total}]")
+    n_partials = 1
+    if qkv.dim() == 3:   # partial sums [parts, tokens, total], added in order
+        n_partials = qkv.shape[0]
+        _need(n_partials >= 1, "qkv needs at least one part")
+    n_tokens = qkv.shape[-2]
+    _need(qkv.dim() in (2, 3) and qkv.shape[-1] == total, f"qkv must be [tokens, {total}]")
     if bias is not None:
         _device_tensor(bias, "qkv bias", torch.float32)
         _need(tuple(bias.shape) == (total,), "qkv bias has the wrong size")
@@ -131,34 +140,39 @@ def qkv_rope_store(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: t
         _device_tensor(slot_mapping, "slot mapping", torch.int32)
         _need(tuple(slot_mapping.shape) == (n_tokens,), "slot mapping must hold one entry per token")
         _need(k_cache is not None and v_cache is not None, "slot mapping needs both caches")
-        _device_tensor(k_cache, "key pages", out_dtype)
-        _device_tensor(v_cache, "value pages", out_dtype)
-        _need(k_cache.dim() == 4 and tuple(k_cache.shape[1:]) == (kv_heads, page_size, head_dim),
-              "key pages must be [pages, kv_heads, page_size, head_dim]")
-        _need(v_cache.dim() == 4 and tuple(v_cache.shape) == (k_cache.shape[0], kv_heads, head_dim, page_size),
-              "value pages must be [pages, kv_heads, head_dim, page_size]")
+        _check_pages(k_cache, v_cache, out_dtype, kv_heads, head_dim, page_size)
     if q_out is None:
         q_out = torch.empty((n_tokens, heads * head_dim), dtype=out_dtype, device=qkv.device)
     _device_tensor(q_out, "q output", out_dtype)
     _need(tuple(q_out.shape) == (n_tokens, heads * head_dim), "q output has the wrong shape")
-    _check(lib.mll_qkv_rope_store(_ptr(qkv), _code(qkv.dtype), _code(out_dtype), _ptr(bias), _ptr(positions), _ptr(slot_mapping),
+    _check(lib.mll_qkv_rope_store(_ptr(qkv), _code(qkv.dtype), n_partials, ctypes.c_int64(n_tokens * total),
+                                  _code(out_dtype), _ptr(bias), _ptr(positions), _ptr(slot_mapping),
                                   _ptr(inv_freq), n_freq, _ptr(q_out), _ptr(k_cache), _ptr(v_cache),
                                   n_tokens, heads, kv_heads, head_dim, page_size, _stream()), lib)
     return q_out
 
 
+def _check_pages(k_cache, v_cache, dtype, kv_heads, head_dim, page_size=None) -> int:
+    """Key and value pages must have the tiled shapes of ``cache.layout``; returns the page size."""
+    from ..cache.layout import key_page_shape, value_page_shape
+    _device_tensor(k_cache, "key pages", dtype)
+    _device_tensor(v_cache, "value pages", dtype)
+    _need(k_cache.dim() == 6 and v_cache.dim() == 7, "key pages must have 6 dimensions and value pages 7 (tiled layout)")
+    found = k_cache.shape[2] * 16
+    _need(page_size is None or page_size == found, "the pages do not have the page size given")
+    pages = k_cache.shape[0]
+    _need(tuple(k_cache.shape) == key_page_shape(pages, kv_heads, found, head_dim), "key pages have the wrong shape")
+    _need(tuple(v_cache.shape) == value_page_shape(pages, kv_heads, found, head_dim), "value pages have the wrong shape")
+    return found
+
+
 def _check_paged(q, k_cache, v_cache, block_table, heads, kv_heads, head_dim) -> int:
     _device_tensor(q, "queries")
     _need(q.dim() == 2 and q.shape[1] == heads * head_dim, "queries must be [tokens, heads * head_dim]")
-    _device_tensor(k_cache, "key pages", q.dtype)
-    _device_tensor(v_cache, "value pages", q.dtype)
-    _need(k_cache.dim() == 4 and k_cache.shape[1] == kv_heads and k_cache.shape[3] == head_dim,
-          "key pages must be [pages, kv_heads, page_size, head_dim]")
-    _need(v_cache.dim() == 4 and tuple(v_cache.shape) == (k_cache.shape[0], kv_heads, head_dim, k_cache.shape[2]),
-          "value pages must be [pages, kv_heads, head_dim, page_size]")
+    page_size = _check_pages(k_cache, v_cache, q.dtype, kv_heads, head_dim)
     _device_tensor(block_table, "block table", torch.int32)
     _need(block_table.dim() == 2, "block table must be [requests, pages]")
-    return k_cache.shape[2]
+    return page_size
 
 
 def paged_attention_rowwise(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -307,12 +321,62 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, view, ctx,
                     scale: float, window: int, heads: int, kv_heads: int, head_dim: int) -> torch.Tensor:
     """Attention of the step's queries over their requests' pages; chooses the kernel for the batch's shape."""
-    page_size = k_cache.shape[2]
+    page_size = k_cache.shape[2] * 16
     mfma_fits = q.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256 and page_size % 16 == 0
     if mfma_fits and ctx.max_count == 1:
-        visible = min(ctx.max_total, window) if window > 0 else ctx.max_total
+        longest = max(ctx.planned_total, ctx.max_total)
+        visible = min(longest, window) if window > 0 else longest
         splits = decode_splits(ctx.n_tokens, kv_heads, visible)
         return paged_attention_decode(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
                                       scale, window, heads, kv_heads, head_dim, splits)
     return paged_attention_rowwise(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
                                    scale, window, heads, kv_heads, head_dim)
+
+
+def pack_weight(weight: torch.Tensor, interleave_halves: bool = False) -> torch.Tensor:
+    """The weight ``[n, k]`` in the order ``gemm_skinny`` streams it: ``[n/16, k/32, 4, 16, 8]``, zero padded.
+
+    With ``interleave_halves`` rows ``i`` and ``n/2 + i`` become neighbours first (gate and up of a gated
+    feed-forward), which is what the gated epilogue expects.
+    """
+    _need(weight.dim() == 2 and weight.dtype == torch.bfloat16, "pack_weight takes a bfloat16 matrix")
+    n, k = weight.shape
+    if interleave_halves:
+        _need(n % 2 == 0, "interleaving needs an even number of rows")
+        weight = torch.stack([weight[: n // 2], weight[n // 2:]], dim=1).reshape(n, k)
+    n_padded, k_padded = -(-n // 16) * 16, -(-k // 32) * 32
+    if (n_padded, k_padded) != (n, k):
+        padded = torch.zeros((n_padded, k_padded), dtype=weight.dtype, device=weight.device)
+        padded[:n, :k] = weight
+        weight = padded
+    packed = weight.view(n_padded // 16, 16, k_padded // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous()
+    return packed
+
+
+SKINNY_MAX_ROWS = 64
+
+
+def gemm_skinny(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f32") -> torch.Tensor:
+    """``x @ W.T`` for at most 64 bfloat16 rows and a packed weight.
+
+    ``f32``: float32 ``[m, n]``; ``bf16``: bfloat16 ``[m, n]``; ``gated``: bfloat16 ``[m, n / 2]`` of
+    silu(gate) * up for interleaved rows.
+    """
+    lib = library.load()
+    _device_tensor(x, "gemm input", torch.bfloat16)
+    _device_tensor(packed, "packed weight", torch.bfloat16)
+    _need(x.dim() == 2 and packed.dim() == 5 and tuple(packed.shape[2:]) == (4, 16, 8), "gemm_skinny takes [m, k] and a packed weight")
+    m, k = x.shape
+    _need(m <= SKINNY_MAX_ROWS, "gemm_skinny takes at most 64 rows")
+    _need(k % 8 == 0, "gemm_skinny needs k to be a multiple of 8")
+    _need(packed.shape[0] == -(-n // 16) and packed.shape[1] == -(-k // 32), "the packed weight does not fit n and k")
+    if epilogue == "f32":
+        code, out = 0, torch.empty((m, n), dtype=torch.float32, device=x.device)
+    elif epilogue == "bf16":
+        code, out = 1, torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    elif epilogue == "gated":
+        code, out = 2, torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
+    else:
+        raise KernelLibraryError(f"unknown epilogue {epilogue!r}")
+    _check(lib.mll_gemm_skinny(_ptr(x), _ptr(packed), _ptr(out), code, m, n, k, _stream()), lib)
+    return out

@@ -17,7 +17,7 @@ import torch
 
 from ..ops import kernels
 from .base import MATRIX, Mixer, PagedKVNeed, Runtime, TensorDecl, VECTOR
-from .linear import linear
+from .linear import Weight, linear
 from .registry import build_part, register_part
 from .spec import PartSpec
 
@@ -62,11 +62,11 @@ class PagedAttention(Mixer):
         weights = [tensors[self.name(f"{role}_proj.weight")] for role, _ in self._projections()]
         if len({w.dtype for w in weights}) != 1:
             raise TypeError("the q, k and v weights of one layer must share a dtype to be stacked")
-        self.qkv_weight = torch.cat(weights, dim=0).contiguous() if len(weights) > 1 else weights[0]
+        self.qkv_weight = Weight(torch.cat(weights, dim=0).contiguous() if len(weights) > 1 else weights[0])
         if self.qkv_bias:
             biases = [tensors[self.name(f"{role}_proj.bias")] for role, _ in self._projections()]
             self.qkv_bias_vector = torch.cat(biases, dim=0).contiguous() if len(biases) > 1 else biases[0]
-        self.o_weight = tensors[self.name("o_proj.weight")]
+        self.o_weight = Weight(tensors[self.name("o_proj.weight")])
 
     def cache_need(self):
         if not self.owns_kv:
@@ -97,7 +97,7 @@ class PagedAttention(Mixer):
         window = int(self.window) if self.window else 0
         o = kernels.paged_attention(q, cache.k, cache.v, view, ctx, self.scale, window,
                                     self.heads, kv_heads, self.head_dim)
-        return linear(o, self.o_weight, out_dtype=torch.float32)        # summed into the residual stream in float32
+        return linear(o, self.o_weight, out_dtype=torch.float32)   # summed into the residual stream in float32
 
 
 register_part("mixer", "paged_attention", PagedAttention)

@@ -12,7 +12,7 @@ import torch
 
 from ..ops import kernels
 from .base import FeedForward, MATRIX, Runtime, TensorDecl
-from .linear import linear
+from .linear import Weight, linear
 from .registry import register_part
 from .spec import PartSpec
 
@@ -37,12 +37,12 @@ class SwiGLU(FeedForward):
         up = tensors[self.name("up_proj.weight")]
         if gate.dtype != up.dtype:
             raise TypeError("the gate and up weights of one layer must share a dtype to be stacked")
-        self.gate_up_weight = torch.cat([gate, up], dim=0).contiguous()
-        self.down_weight = tensors[self.name("down_proj.weight")]
+        self.gate_up_weight = Weight(torch.cat([gate, up], dim=0).contiguous(), gated=True)
+        self.down_weight = Weight(tensors[self.name("down_proj.weight")])
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        gate_up = linear(x, self.gate_up_weight)
-        return linear(kernels.silu_mul(gate_up), self.down_weight, out_dtype=torch.float32)
+        z = linear(x, self.gate_up_weight, gated=True)
+        return linear(z, self.down_weight, out_dtype=torch.float32)
 
 
 register_part("ffn", "swiglu", SwiGLU)

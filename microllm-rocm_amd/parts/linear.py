@@ -2,7 +2,10 @@
 
 The reference stores ``[in, out]`` and transposes every linear at load
 (src/model/model.cpp:285, 1939-1973); keeping ``[out, in]`` removes that pass and
-lets several weights that share an input be stacked along ``out``.
+lets several weights that share an input be stacked along ``out``. A bfloat16
+weight is held twice on the GPU: as stored, for the library product that steps
+with many rows use, and packed in the order the MFMA consumes it, for the kernel
+that streams it once when a step has few rows (decoding).
 """
 from __future__ import annotations
 
@@ -13,14 +16,49 @@ import torch
 from ..ops import kernels
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """``x @ weight.T`` with float32 accumulation; the result has ``out_dtype`` (default: x's)."""
+class Weight:
+    """A linear's weight ``[out, in]`` and, for bfloat16, its packed copy."""
+
+    def __init__(self, tensor: torch.Tensor, gated: bool = False, pack: bool = True):
+        self.tensor = tensor
+        self.out_features, self.in_features = tensor.shape
+        self.gated = gated   # rows are [gate; up]: the packed copy interleaves them for the fused epilogue
+        self.packed: Optional[torch.Tensor] = None
+        if pack and tensor.is_cuda and tensor.dtype == torch.bfloat16 and self.in_features % 8 == 0:
+            self.packed = kernels.pack_weight(tensor, interleave_halves=gated)
+
+    @property
+    def dtype(self) -> torch.dtype:
+        return self.tensor.dtype
+
+
+SKINNY_ROWS = 16   # up to this many rows the streaming kernel beats the library on MI355X
+
+
+def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None, gated: bool = False) -> torch.Tensor:
+    """``x @ W.T`` with float32 accumulation; the result has ``out_dtype`` (default: x's).
+
+    With ``gated`` the weight's rows are [gate; up] and the result is ``silu(gate) * up`` of half the
+    width, in x's dtype.
+    """
+    if isinstance(weight, torch.Tensor):
+        weight = Weight(weight, pack=False)
     out_dtype = out_dtype or x.dtype
-    if weight.dtype == torch.float32:
+    w = weight.tensor
+    if w.dtype == torch.float32:
         # True 32-bit product, also for a 32-bit weight inside a bfloat16 engine.
         a = x if x.dtype == torch.float32 else x.to(torch.float32)
-        y = kernels.gemm_f32(a, weight)
+        y = kernels.gemm_f32(a, w)
+        if gated:
+            return kernels.silu_mul(y if x.dtype == torch.float32 else y.to(x.dtype))
         return y if out_dtype == torch.float32 else y.to(out_dtype)
-    if x.dtype != weight.dtype:
-        raise TypeError(f"cannot multiply {x.dtype} activations with a {weight.dtype} weight")
-    return kernels.gemm_bf16(x, weight, out_dtype)
+    if x.dtype != w.dtype:
+        raise TypeError(f"cannot multiply {x.dtype} activations with a {w.dtype} weight")
+    rows = x.shape[0]
+    if weight.packed is not None and rows <= SKINNY_ROWS:
+        if gated:
+            return kernels.gemm_skinny(x, weight.packed, weight.out_features, "gated")
+        return kernels.gemm_skinny(x, weight.packed, weight.out_features, "bf16" if out_dtype == torch.bfloat16 else "f32")
+    if gated:
+        return kernels.silu_mul(kernels.gemm_bf16(x, w, torch.bfloat16))
+    return kernels.gemm_bf16(x, w, out_dtype)

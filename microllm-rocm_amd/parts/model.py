@@ -14,7 +14,7 @@ import torch
 from ..ops import kernels
 from .base import CacheNeed, MATRIX, Part, Runtime, TensorDecl
 from .block import Block, build_block
-from .linear import linear
+from .linear import Weight, linear
 from .registry import build_part, register_part
 from .spec import ModelSpec, PartSpec
 
@@ -54,7 +54,7 @@ class LMHead(Part):
         return {self.name("weight"): TensorDecl((self.vocab, self.width), MATRIX)}
 
     def bind(self, tensors):
-        self.weight = tensors[self.name("weight")]
+        self.weight = Weight(tensors[self.name("weight")])
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return linear(x, self.weight, out_dtype=torch.float32)

@@ -9,6 +9,9 @@ import torch
 
 import plain_qwen2 as plain
 
+from microllm_rocm_amd.cache.layout import (key_page_shape, key_rows, value_page_shape, value_rows, write_key_rows,
+                                            write_value_rows)
+
 pytestmark = pytest.mark.gpu
 
 DEVICE = "cuda:0"
@@ -105,7 +108,7 @@ def reference_qkv(qkv, bias, positions, theta, heads, kv_heads, hd, rotary):
 @pytest.mark.parametrize("in_dtype,out_dtype", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
                                                 (torch.bfloat16, torch.bfloat16)])
 @pytest.mark.parametrize("heads,kv_heads,hd,rotary,page_size,use_bias", [
-    (5, 5, 48, 48, 16, True), (6, 2, 16, 16, 8, False), (7, 1, 80, 32, 32, True), (3, 3, 24, 0, 16, True)])
+    (5, 5, 48, 48, 16, True), (6, 2, 16, 16, 48, False), (7, 1, 80, 32, 32, True), (3, 3, 24, 0, 16, True)])
 def test_qkv_rope_store(in_dtype, out_dtype, heads, kv_heads, hd, rotary, page_size, use_bias):
     rng = np.random.default_rng(heads * 100 + hd)
     tokens, pages = 11, 9
@@ -118,8 +121,8 @@ def test_qkv_rope_store(in_dtype, out_dtype, heads, kv_heads, hd, rotary, page_s
     inv_freq = None
     if rotary:
         inv_freq = torch.tensor(theta ** (-np.arange(0, rotary, 2, dtype=np.float64) / rotary), dtype=torch.float64, device=DEVICE)
-    k_pages = torch.full((pages, kv_heads, page_size, hd), 7.0, dtype=out_dtype, device=DEVICE)
-    v_pages = torch.full((pages, kv_heads, hd, page_size), 7.0, dtype=out_dtype, device=DEVICE)
+    k_pages = torch.full(key_page_shape(pages, kv_heads, page_size, hd), 7.0, dtype=out_dtype, device=DEVICE)
+    v_pages = torch.full(value_page_shape(pages, kv_heads, page_size, hd), 7.0, dtype=out_dtype, device=DEVICE)
     q = kernels().qkv_rope_store(qkv, torch.from_numpy(bias_ref).to(DEVICE) if use_bias else None,
                                  torch.from_numpy(positions).to(DEVICE), torch.from_numpy(slots).to(DEVICE), inv_freq,
                                  k_pages, v_pages, heads, kv_heads, hd, page_size, out_dtype)
@@ -127,7 +130,8 @@ def test_qkv_rope_store(in_dtype, out_dtype, heads, kv_heads, hd, rotary, page_s
                                         theta, heads, kv_heads, hd, rotary)
     tol = tolerance(out_dtype)
     np.testing.assert_allclose(q.float().cpu().numpy().reshape(tokens, heads, hd), q_ref, **tol)
-    k_host, v_host = k_pages.float().cpu().numpy(), v_pages.float().cpu().numpy()
+    k_host = key_rows(k_pages, hd).float().cpu().numpy()        # [page, kv_head, position, dim]
+    v_host = value_rows(v_pages, hd).float().cpu().numpy()
     written = np.zeros((pages, page_size), dtype=bool)
     for token, slot in enumerate(slots):
         if slot < 0:
@@ -135,8 +139,8 @@ def test_qkv_rope_store(in_dtype, out_dtype, heads, kv_heads, hd, rotary, page_s
         page, offset = divmod(int(slot), page_size)
         written[page, offset] = True
         np.testing.assert_allclose(k_host[page, :, offset, :], k_ref[token], **tol)
-        np.testing.assert_allclose(v_host[page, :, :, offset], v_ref[token], **tol)
-    assert np.all(k_host.transpose(0, 2, 1, 3)[~written] == 7.0) and np.all(v_host.transpose(0, 3, 1, 2)[~written] == 7.0)
+        np.testing.assert_allclose(v_host[page, :, offset, :], v_ref[token], **tol)
+    assert np.all(k_host.transpose(0, 2, 1, 3)[~written] == 7.0) and np.all(v_host.transpose(0, 2, 1, 3)[~written] == 7.0)
 
 
 def test_rope_vector_of_the_reference_and_large_positions():
@@ -170,8 +174,8 @@ def build_paged_case(rng, dtype, seq_lengths, counts, heads, kv_heads, hd, page_
         cursor += count
     k_ref = [rng.normal(size=(length, kv_heads, hd)) for length in seq_lengths]
     v_ref = [rng.normal(size=(length, kv_heads, hd)) for length in seq_lengths]
-    k_pages = np.full((total_pages, kv_heads, page_size, hd), 1e4, dtype=np.float32)
-    v_pages = np.full((total_pages, kv_heads, hd, page_size), -1e4, dtype=np.float32)
+    k_rows = np.full((total_pages, kv_heads, page_size, hd), 1e4, dtype=np.float32)    # [page, kv_head, position, dim]
+    v_rows = np.full((total_pages, kv_heads, page_size, hd), -1e4, dtype=np.float32)
     exact_k, exact_v = [], []
     for s, length in enumerate(seq_lengths):
         k_exact, _ = prepare(k_ref[s], dtype)
@@ -180,12 +184,16 @@ def build_paged_case(rng, dtype, seq_lengths, counts, heads, kv_heads, hd, page_
         exact_v.append(v_exact)
         for position in range(length):
             page, offset = table[s, position // page_size], position % page_size
-            k_pages[page, :, offset, :] = k_exact[position]
-            v_pages[page, :, :, offset] = v_exact[position]
+            k_rows[page, :, offset, :] = k_exact[position]
+            v_rows[page, :, offset, :] = v_exact[position]
+    k_pages = torch.zeros(key_page_shape(total_pages, kv_heads, page_size, hd), dtype=dtype, device=DEVICE)
+    v_pages = torch.zeros(value_page_shape(total_pages, kv_heads, page_size, hd), dtype=dtype, device=DEVICE)
+    write_key_rows(k_pages, torch.from_numpy(k_rows).to(dtype).to(DEVICE))
+    write_value_rows(v_pages, torch.from_numpy(v_rows).to(dtype).to(DEVICE))
     seq_of_token = np.repeat(np.arange(n_seqs), counts).astype(np.int32)
     positions = np.concatenate([np.arange(length - count, length) for length, count in zip(seq_lengths, counts)]).astype(np.int32)
     q_exact, q = prepare(rng.normal(size=(len(positions), heads * hd)), dtype)
-    tensors = dict(q=q, k=torch.from_numpy(k_pages).to(dtype).to(DEVICE), v=torch.from_numpy(v_pages).to(dtype).to(DEVICE),
+    tensors = dict(q=q, k=k_pages, v=v_pages,
                    table=torch.from_numpy(table).to(DEVICE), seq=torch.from_numpy(seq_of_token).to(DEVICE),
                    pos=torch.from_numpy(positions).to(DEVICE))
     return tensors, q_exact, exact_k, exact_v, seq_of_token, positions
@@ -206,7 +214,7 @@ def reference_attention(q_exact, exact_k, exact_v, seq_of_token, positions, head
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kv_heads,hd,page_size,window", [
-    (4, 2, 16, 16, 0), (3, 1, 32, 16, 24), (5, 5, 48, 16, 100), (6, 3, 24, 8, 0), (2, 1, 128, 32, 70), (8, 1, 200, 4, 0)])
+    (4, 2, 16, 16, 0), (3, 1, 32, 16, 24), (5, 5, 48, 16, 100), (6, 3, 24, 48, 0), (2, 1, 128, 32, 70), (8, 1, 200, 16, 0)])
 def test_rowwise_attention(dtype, heads, kv_heads, hd, page_size, window):
     rng = np.random.default_rng(hd + window)
     lengths, counts = [150, 1, 64, 97], [40, 1, 64, 1]
@@ -248,10 +256,10 @@ def test_a_far_key_among_hundreds_and_the_window_edge(kernel):
         direction /= np.linalg.norm(direction)
         q = np.tile(direction * 16.0, heads)[None, :]
         table = t["table"].cpu().numpy()
-        k_pages = t["k"].float().cpu().numpy()
+        k_rows = key_rows(t["k"], hd).float()
         page, offset = table[0, target // page_size], target % page_size
-        k_pages[page, :, offset, :] = direction * 16.0          # score 256 * scale against |others| ~ 16 * scale
-        t["k"] = torch.from_numpy(k_pages).to(dtype).to(DEVICE)
+        k_rows[page, :, offset, :] = torch.from_numpy(direction * 16.0).float()    # score 256 * scale against |others| ~ 16 * scale
+        write_key_rows(t["k"], k_rows.to(dtype))
         _, t["q"] = prepare(q, dtype)
         scale = 1.0 / math.sqrt(hd)
         if kernel == "decode":
@@ -364,3 +372,60 @@ def test_sampling_frequencies():
     chosen = kernels().sample(logits, torch.full((4000,), 0.8, device=DEVICE), None, uniform).cpu().numpy()
     expected = np.exp(np.array([1.0, 0.0, -1.0, 0.5, -30.0]) / 0.8)
     np.testing.assert_allclose(np.bincount(chosen, minlength=5) / 4000, expected / expected.sum(), atol=0.025)
+
+
+# ---- the streaming product for few rows -------------------------------------------------------------------------
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 40, 64])
+@pytest.mark.parametrize("n,k", [(331, 120), (96, 64), (1000, 200), (4608, 3584), (176, 24), (3584, 18944), (40000, 256)])
+def test_gemm_skinny(m, n, k):
+    rng = np.random.default_rng(m * 7 + n)
+    a_ref, a = to_bf16_exact(rng.normal(size=(m, k)))
+    w_ref, w = to_bf16_exact(rng.normal(size=(n, k)) * 0.1)
+    ka = kernels()
+    packed = ka.pack_weight(w)
+    assert packed.shape == (-(-n // 16), -(-k // 32), 4, 16, 8)
+    expected = a_ref @ w_ref.T
+    scale = np.abs(expected).max()
+    full = ka.gemm_skinny(a, packed, n, "f32")
+    assert full.dtype == torch.float32 and full.shape == (m, n)
+    assert np.abs(full.double().cpu().numpy() - expected).max() <= 1e-5 * scale
+    out = ka.gemm_skinny(a, packed, n, "bf16")
+    assert out.dtype == torch.bfloat16 and np.abs(out.float().cpu().numpy() - expected).max() <= 5e-3 * scale
+    # the same in every run; and among calls of up to 16 rows a row's result does not depend on the other rows
+    assert torch.equal(ka.gemm_skinny(a, packed, n, "f32"), full)
+    if m <= 16:
+        alone = ka.gemm_skinny(a[m - 1:m].contiguous(), packed, n, "f32")
+        assert torch.equal(alone[0], full[m - 1])
+
+
+@pytest.mark.parametrize("m,width,k", [(3, 203, 96), (16, 176, 64), (33, 1000, 120)])
+def test_gemm_skinny_gated_epilogue(m, width, k):
+    rng = np.random.default_rng(width)
+    a_ref, a = to_bf16_exact(rng.normal(size=(m, k)))
+    w_ref, w = to_bf16_exact(rng.normal(size=(2 * width, k)) * 0.2)      # rows: [gate; up]
+    packed = kernels().pack_weight(w, interleave_halves=True)
+    out = kernels().gemm_skinny(a, packed, 2 * width, "gated")
+    expected = plain.silu(a_ref @ w_ref[:width].T) * (a_ref @ w_ref[width:].T)
+    assert out.shape == (m, width)
+    np.testing.assert_allclose(out.float().cpu().numpy(), expected, rtol=1.2e-2, atol=1.2e-2 * np.abs(expected).max())
+
+
+def test_consumers_add_partial_sums_in_order():
+    rng = np.random.default_rng(3)
+    k = kernels()
+    h_ref = rng.normal(size=(5, 120)).astype(np.float32)
+    parts = rng.normal(size=(4, 5, 120)).astype(np.float32)
+    weight = np.ones(120, dtype=np.float32)
+    h = torch.from_numpy(h_ref.copy()).to(DEVICE)
+    out = k.rms_norm(h, torch.from_numpy(weight).to(DEVICE), 1e-5, torch.float32, delta=torch.from_numpy(parts).to(DEVICE), write_h=True)
+    total = h_ref.astype(np.float64) + parts.astype(np.float64).sum(axis=0)
+    np.testing.assert_allclose(h.cpu().numpy(), total, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(out.cpu().numpy(), plain.rms_norm(total, weight, 1e-5), rtol=1e-5, atol=1e-5)
+    heads, kv_heads, hd = 3, 1, 16
+    qkv_parts = rng.normal(size=(3, 6, (heads + 2 * kv_heads) * hd)).astype(np.float32)
+    positions = torch.arange(6, dtype=torch.int32, device=DEVICE)
+    q_parts = k.qkv_rope_store(torch.from_numpy(qkv_parts).to(DEVICE), None, positions, None, None, None, None,
+                               heads, kv_heads, hd, 16, torch.float32)
+    q_sum = k.qkv_rope_store(torch.from_numpy(qkv_parts.sum(axis=0)).to(DEVICE), None, positions, None, None, None, None,
+                             heads, kv_heads, hd, 16, torch.float32)
+    np.testing.assert_allclose(q_parts.cpu().numpy(), q_sum.cpu().numpy(), rtol=1e-6, atol=1e-6)
