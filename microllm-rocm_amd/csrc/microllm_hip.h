@@ -54,6 +54,16 @@ int mll_paged_attention_rowwise(const void* q, int dtype, const void* k_cache, c
                                 float scale, int window, int n_tokens, int heads, int kv_heads,
                                 int head_dim, int page_size, hipStream_t stream);
 
+// The same attention for bfloat16 portions of prompts with MFMA: one workgroup per (tile of up to
+// mll_paged_attention_prefill_tile() consecutive tokens of one request, query head). `tiles` holds, for each
+// tile, (request index, first token in the flat list, number of tokens); a tile never spans two requests and
+// its tokens have consecutive positions.
+int mll_paged_attention_prefill(const void* q, const void* k_cache, const void* v_cache,
+                                const int32_t* block_table, int table_width, const int32_t* tiles,
+                                int n_tiles, const int32_t* positions, void* out, float scale, int window,
+                                int heads, int kv_heads, int head_dim, int page_size, hipStream_t stream);
+int mll_paged_attention_prefill_tile();
+
 // out[t, c] = silu(gate[t, c]) * up[t, c]; gate and up rows are `in_stride` elements apart.
 // The same attention for bfloat16 with MFMA, one workgroup per (token, kv head, split of the keys): meant
 // for steps whose requests bring one token each, right for any. head_dim a multiple of 16 up to 256,

@@ -16,6 +16,9 @@ import torch
 from ..cache.manager import CacheManager, RELEASED, RequestCache
 
 
+QUERY_TILE = 64   # tokens of one request that one workgroup of the prefill attention kernel takes
+
+
 @dataclass
 class StepEntry:
     """One request's next tokens and the places among them whose logits are wanted."""
@@ -45,6 +48,7 @@ class StepContext:
     seq_total: torch.Tensor     # int32 [requests]: positions in the cache once this step is done
     slots: torch.Tensor         # int32 [requests]: state slot of every request
     want_rows: Optional[torch.Tensor]  # int32 [wanted]: rows of the flat list whose logits are wanted
+    query_tiles: torch.Tensor   # int32 [tiles, 3]: (request, first token in the flat list, tokens) per tile of <= 64 tokens
     paged: List[PagedView]
     # the same on the host, for parts written in Python and for choosing kernels
     starts: List[int] = field(default_factory=list)
@@ -112,8 +116,11 @@ class BatchBuilder:
             mappings.append(mapping.astype(np.int32))
             widths.append(width)
         slots = np.asarray([request.slot for request in requests], dtype=np.int32)
+        query_tiles = np.asarray([(index, cu[index] + offset, min(QUERY_TILE, count - offset))
+                                  for index, count in enumerate(counts) for offset in range(0, count, QUERY_TILE)],
+                                 dtype=np.int32).reshape(-1, 3)
         pieces = [tokens, positions, seq_of_token, cu, np.asarray(starts, np.int32), np.asarray(totals, np.int32),
-                  slots, want_rows]
+                  slots, want_rows, query_tiles.reshape(-1)]
         for table, mapping in zip(tables, mappings):
             pieces += [table.reshape(-1), mapping]
         offsets, cursor = [], 0
@@ -134,13 +141,13 @@ class BatchBuilder:
 
         paged = []
         for g, group in enumerate(self.cache.groups):
-            paged.append(PagedView(piece_at(8 + 2 * g, (n_seqs, widths[g])), piece_at(9 + 2 * g),
+            paged.append(PagedView(piece_at(9 + 2 * g, (n_seqs, widths[g])), piece_at(10 + 2 * g),
                                    page_size, widths[g]))
         longest = max(totals) if totals else 0
         return StepContext(
             n_tokens=n_tokens, n_seqs=n_seqs, tokens=piece_at(0), positions=piece_at(1), seq_of_token=piece_at(2),
             cu_tokens=piece_at(3), seq_start=piece_at(4), seq_total=piece_at(5), slots=piece_at(6),
-            want_rows=piece_at(7) if want_rows.size else None, paged=paged,
+            want_rows=piece_at(7) if want_rows.size else None, query_tiles=piece_at(8, (-1, 3)), paged=paged,
             starts=list(starts), counts=counts, host_slots=[request.slot for request in requests],
             max_count=max(counts) if counts else 0, max_total=longest,
             planned_total=longest if fixed_width is None else fixed_width * page_size)

@@ -285,9 +285,10 @@ def gemm_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = to
 
 
 def decode_splits(n_tokens: int, kv_heads: int, longest: int) -> int:
-    """How many splits of the keys fill the GPU: about a thousand workgroups, at least 128 keys each."""
-    wanted = -(-1024 // max(1, n_tokens * kv_heads))
-    return max(1, min(wanted, -(-longest // 128), 256))
+    """How many splits of the keys: about one workgroup per compute unit, at least 256 keys each (measured on
+    MI355X: more splits cost more in joining them than they gain)."""
+    wanted = -(-256 // max(1, n_tokens * kv_heads))
+    return max(1, min(wanted, longest // 256, 256))
 
 
 def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
@@ -318,17 +319,44 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     return out
 
 
+def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                            query_tiles: torch.Tensor, positions: torch.Tensor, scale: float, window: int,
+                            heads: int, kv_heads: int, head_dim: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The MFMA kernel for bfloat16 portions of prompts; ``query_tiles`` rows are (request, first token, tokens)."""
+    lib = library.load()
+    page_size = _check_paged(q, k_cache, v_cache, block_table, heads, kv_heads, head_dim)
+    _need(q.dtype == torch.bfloat16, "the prefill kernel takes bfloat16")
+    _need(head_dim % 16 == 0 and 16 <= head_dim <= 256, "the prefill kernel takes head sizes in steps of 16 up to 256")
+    _device_tensor(query_tiles, "query tiles", torch.int32)
+    _need(query_tiles.dim() == 2 and query_tiles.shape[1] == 3, "query tiles must be [tiles, 3]")
+    _device_tensor(positions, "positions", torch.int32)
+    _need(positions.shape[0] == q.shape[0], "positions must hold one entry per token")
+    if out is None:
+        out = torch.empty_like(q)
+    _check(lib.mll_paged_attention_prefill(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
+                                           _ptr(query_tiles), query_tiles.shape[0], _ptr(positions), _ptr(out),
+                                           ctypes.c_float(scale), int(window), heads, kv_heads, head_dim, page_size,
+                                           _stream()), lib)
+    return out
+
+
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, view, ctx,
                     scale: float, window: int, heads: int, kv_heads: int, head_dim: int) -> torch.Tensor:
-    """Attention of the step's queries over their requests' pages; chooses the kernel for the batch's shape."""
-    page_size = k_cache.shape[2] * 16
-    mfma_fits = q.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256 and page_size % 16 == 0
+    """Attention of the step's queries over their requests' pages; chooses the kernel for the batch's shape.
+
+    bfloat16 with a head size in steps of 16: the MFMA kernels, split over the keys when every request brings
+    one token, tiled over the queries otherwise. Everything else (float32, other head sizes): the plain kernel.
+    """
+    mfma_fits = q.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256
     if mfma_fits and ctx.max_count == 1:
         longest = max(ctx.planned_total, ctx.max_total)
         visible = min(longest, window) if window > 0 else longest
         splits = decode_splits(ctx.n_tokens, kv_heads, visible)
         return paged_attention_decode(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
                                       scale, window, heads, kv_heads, head_dim, splits)
+    if mfma_fits:
+        return paged_attention_prefill(q, k_cache, v_cache, view.block_table, ctx.query_tiles, ctx.positions,
+                                       scale, window, heads, kv_heads, head_dim)
     return paged_attention_rowwise(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
                                    scale, window, heads, kv_heads, head_dim)
 

@@ -240,7 +240,26 @@ def test_decode_attention(heads, kv_heads, hd, page_size, window, splits):
     np.testing.assert_allclose(out.float().cpu().numpy(), reference, **tolerance(torch.bfloat16))
 
 
-@pytest.mark.parametrize("kernel", ["rowwise_f32", "rowwise_bf16", "decode"])
+@pytest.mark.parametrize("heads,kv_heads,hd,page_size,window", [
+    (4, 2, 16, 16, 0), (3, 1, 32, 16, 24), (5, 5, 48, 16, 100), (28, 4, 128, 16, 0), (14, 2, 64, 32, 40),
+    (2, 1, 80, 16, 300), (3, 3, 256, 16, 0), (7, 7, 112, 64, 129), (6, 3, 96, 48, 17)])
+def test_prefill_attention(heads, kv_heads, hd, page_size, window):
+    rng = np.random.default_rng(heads + hd + window)
+    lengths, counts = [517, 1, 200, 97, 64, 131, 40], [130, 1, 200, 17, 64, 2, 33]
+    t, q_exact, ek, ev, seq, pos = build_paged_case(rng, torch.bfloat16, lengths, counts, heads, kv_heads, hd, page_size)
+    scale = 1.0 / math.sqrt(hd)
+    tiles, start = [], 0
+    for index, count in enumerate(counts):
+        tiles += [(index, start + offset, min(64, count - offset)) for offset in range(0, count, 64)]
+        start += count
+    query_tiles = torch.tensor(tiles, dtype=torch.int32, device=DEVICE)
+    out = kernels().paged_attention_prefill(t["q"], t["k"], t["v"], t["table"], query_tiles, t["pos"], scale, window,
+                                            heads, kv_heads, hd)
+    reference = reference_attention(q_exact, ek, ev, seq, pos, heads, kv_heads, hd, scale, window)
+    np.testing.assert_allclose(out.float().cpu().numpy(), reference, **tolerance(torch.bfloat16))
+
+
+@pytest.mark.parametrize("kernel", ["rowwise_f32", "rowwise_bf16", "decode", "prefill"])
 def test_a_far_key_among_hundreds_and_the_window_edge(kernel):
     """One key is made to dominate the softmax; the output must be that key's value. With random keys a wrong
     page or an off-by-one at the window's edge would change the result too little to see."""
@@ -265,6 +284,10 @@ def test_a_far_key_among_hundreds_and_the_window_edge(kernel):
         if kernel == "decode":
             out = k.paged_attention_decode(t["q"], t["k"], t["v"], t["table"], t["seq"], t["pos"], scale, window,
                                            heads, kv_heads, hd, 6)
+        elif kernel == "prefill":
+            out = k.paged_attention_prefill(t["q"], t["k"], t["v"], t["table"],
+                                            torch.tensor([[0, 0, 1]], dtype=torch.int32, device=DEVICE), t["pos"],
+                                            scale, window, heads, kv_heads, hd)
         else:
             out = k.paged_attention_rowwise(t["q"], t["k"], t["v"], t["table"], t["seq"], t["pos"], scale, window,
                                             heads, kv_heads, hd)
