@@ -1,0 +1,244 @@
+"""The command line, in the manner of the reference's ``microllm_hf_infer`` (apps/hf_infer.cpp:32-73, 75-286):
+``--name value`` pairs, booleans as ``true|false``, an unknown option is an error, one JSON object on
+standard output. Options the reference has keep their names and meanings; what this engine adds
+(``--model``, ``--dtype``, sampling, pages, the token budget) follows the same style.
+
+    microllm_hf_infer --config DIR/config.json --weights DIR/model.safetensors --tokens 1,2,3 \\
+                      --device hip --new-tokens 16
+
+Workloads (``--workload``): ``prefill`` times the prompt alone, ``decode`` times steady decoding after it,
+``both`` (default) generates ``--new-tokens`` tokens after the prompt, ``continuous`` serves several requests
+whose prompts are cyclic slices of the given token ids (apps/hf_infer.cpp:845-861), arriving at given steps.
+"""
+from __future__ import annotations
+
+import json
+import os
+import sys
+import time
+from typing import Dict, List, Optional
+
+OPTIONS: Dict[str, object] = {
+    # the reference's options
+    "config": None, "weights": None, "tokens": "", "device": "hip", "top-k": 10, "logits-output": None,
+    "new-tokens": 0, "warmup": 0, "steps": 1, "prefill-warmup": 0, "prefill-steps": 1, "workload": "both",
+    "batch": 1, "decode-mode": "generation", "kv-cache-dtype": None, "cache-capacity": 0,
+    "continuous-slots": 0, "continuous-prompt-lengths": "", "continuous-new-token-lengths": "",
+    "continuous-prompt-offsets": "", "continuous-arrival-steps": "",
+    # this engine's own
+    "model": None, "dtype": "bfloat16", "temperature": 0.0, "sample-top-k": 0, "seed": 1, "stop-tokens": "",
+    "block-size": 16, "num-blocks": 0, "max-batched-tokens": 2048, "prefill-chunk": 512, "max-requests": 64,
+    "random-config": None, "prompt-lengths": "", "prompt-seed": 0, "use-graphs": "true",
+}
+
+
+class UsageError(Exception):
+    pass
+
+
+def parse(argv: List[str]) -> Dict[str, object]:
+    options = dict(OPTIONS)
+    index = 0
+    while index < len(argv):
+        name = argv[index]
+        if not name.startswith("--") or name[2:] not in OPTIONS:
+            raise UsageError(f"unknown option {name}")
+        if index + 1 >= len(argv):
+            raise UsageError(f"option {name} needs a value")
+        key, text = name[2:], argv[index + 1]
+        default = OPTIONS[key]
+        try:
+            if isinstance(default, bool) or isinstance(default, str) or default is None:
+                options[key] = text
+            elif isinstance(default, int):
+                options[key] = int(text)
+            elif isinstance(default, float):
+                options[key] = float(text)
+        except ValueError:
+            raise UsageError(f"option {name} needs a number, got {text!r}") from None
+        index += 2
+    return options
+
+
+def integers(text: str, what: str) -> List[int]:
+    if not text:
+        return []
+    try:
+        values = [int(piece) for piece in text.split(",")]
+    except ValueError:
+        raise UsageError(f"{what} must be comma-separated integers") from None
+    if any(value < 0 for value in values):
+        raise UsageError(f"{what} must be non-negative")
+    return values
+
+
+def boolean(text: str, what: str) -> bool:
+    if text not in ("true", "false"):
+        raise UsageError(f"{what} must be true or false")
+    return text == "true"
+
+
+def main(argv: Optional[List[str]] = None) -> int:
+    argv = list(sys.argv[1:] if argv is None else argv)
+    if argv and argv[0] in ("-h", "--help"):
+        print(__doc__)
+        print("options: " + " ".join(f"--{name}" for name in OPTIONS))
+        return 0
+    try:
+        options = parse(argv)
+        return run(options)
+    except UsageError as error:
+        print(f"microllm_hf_infer: {error}", file=sys.stderr)
+        return 2
+
+
+def run(options: Dict[str, object]) -> int:
+    if options["device"] != "hip":
+        raise UsageError("this engine runs on --device hip only")
+    if options["workload"] not in ("both", "prefill", "decode", "continuous"):
+        raise UsageError("--workload must be both, prefill, decode or continuous")
+    model_dir = options["model"]
+    if model_dir is None and options["config"] is not None:
+        model_dir = os.path.dirname(os.path.abspath(str(options["config"])))
+        if options["weights"] is not None and os.path.dirname(os.path.abspath(str(options["weights"]))) != model_dir:
+            raise UsageError("--config and --weights must lie in one model folder")
+    if model_dir is None and options["random-config"] is None:
+        raise UsageError("give --model DIR, --config and --weights, or --random-config FILE")
+    dtype = str(options["dtype"])
+    if options["kv-cache-dtype"] is not None and options["kv-cache-dtype"] not in ("fp32", "bf16"):
+        raise UsageError("--kv-cache-dtype must be fp32 or bf16")
+    if dtype in ("fp32",):
+        dtype = "float32"
+    if dtype in ("bf16",):
+        dtype = "bfloat16"
+    if options["kv-cache-dtype"] is not None and {"fp32": "float32", "bf16": "bfloat16"}[str(options["kv-cache-dtype"])] != dtype:
+        raise UsageError("the cache has the engine's dtype: --kv-cache-dtype must agree with --dtype")
+
+    import numpy as np
+    import torch
+    from .. import Engine, GenerationConfig, Scheduler, generate
+    from ..config import load_config
+    from ..engine.benchmark import decode_throughput, prefill_throughput
+    from ..engine.batch import StepEntry
+
+    tokens = integers(str(options["tokens"]), "--tokens")
+    prompt_lengths = integers(str(options["prompt-lengths"]), "--prompt-lengths")
+    batch = int(options["batch"])
+    new_tokens = int(options["new-tokens"])
+    block_size = int(options["block-size"])
+    started = time.perf_counter()
+
+    continuous = options["workload"] == "continuous"
+    if continuous:
+        lengths = integers(str(options["continuous-prompt-lengths"]), "--continuous-prompt-lengths")
+        new_lengths = integers(str(options["continuous-new-token-lengths"]), "--continuous-new-token-lengths")
+        arrivals = integers(str(options["continuous-arrival-steps"]), "--continuous-arrival-steps") or [0] * len(lengths)
+        offsets = integers(str(options["continuous-prompt-offsets"]), "--continuous-prompt-offsets") or [0] * len(lengths)
+        if not lengths or not (len(lengths) == len(new_lengths) == len(arrivals) == len(offsets)):
+            raise UsageError("continuous lengths, new-token lengths, arrival steps and offsets must match in count")
+        needed = sum(-(-(a + b) // block_size) * block_size for a, b in zip(lengths, new_lengths))
+    else:
+        needed = batch * (-(-(max(len(tokens), max(prompt_lengths, default=0)) + new_tokens + int(options["steps"])
+                               + int(options["warmup"])) // block_size) + 1) * block_size
+    capacity = int(options["cache-capacity"])
+    num_blocks = int(options["num-blocks"]) or None
+    max_tokens = None if num_blocks else max(needed, capacity * batch, block_size)
+    engine_options = dict(dtype=dtype, device="cuda:0", page_size=block_size, max_tokens=max_tokens, num_pages=num_blocks,
+                          max_requests=max(int(options["max-requests"]), batch),
+                          use_graphs=boolean(str(options["use-graphs"]), "--use-graphs"))
+    if model_dir is not None:
+        engine = Engine.from_folder(str(model_dir), **engine_options)
+    else:
+        architecture, config = load_config(str(options["random-config"]))
+        engine = Engine.from_random(config, seed=int(options["seed"]), on_device=True, **engine_options)
+    load_ms = (time.perf_counter() - started) * 1e3
+    vocab = engine.spec.vocab_size
+    if not tokens and prompt_lengths:
+        rng = np.random.default_rng(int(options["prompt-seed"]))
+        tokens = rng.integers(0, vocab, size=prompt_lengths[0]).tolist()
+    if not tokens:
+        raise UsageError("give --tokens a,b,c or --prompt-lengths N with --prompt-seed")
+
+    report = {"schema_version": 1, "device": "hip", "device_name": torch.cuda.get_device_name(0),
+              "architecture": engine.spec.architecture, "compute_dtype": dtype, "workload": options["workload"],
+              "load_ms": round(load_ms, 3), "token_count": len(tokens), "batch": batch,
+              "kv_block_size": block_size, "kv_blocks": engine.cache.groups[0].pool.num_pages if engine.cache.groups else 0,
+              "allocated_cache_bytes": engine.cache.allocated_bytes()}
+    stop_tokens = tuple(integers(str(options["stop-tokens"]), "--stop-tokens"))
+    params = GenerationConfig(max_new_tokens=new_tokens, temperature=float(options["temperature"]),
+                              top_k=int(options["sample-top-k"]), seed=int(options["seed"]), stop_tokens=stop_tokens)
+
+    if continuous:
+        prompts = [[tokens[(index + offset) % len(tokens)] for index in range(length)]
+                   for length, offset in zip(lengths, offsets)]
+        per_request = [GenerationConfig(max_new_tokens=new, temperature=params.temperature, top_k=params.top_k,
+                                        seed=params.seed + index, stop_tokens=stop_tokens)
+                       for index, new in enumerate(new_lengths)]
+        slots = int(options["continuous-slots"]) or None
+        torch.cuda.synchronize()
+        begun = time.perf_counter()
+        outputs, scheduler = generate(engine, prompts, per_request, max_batched_tokens=int(options["max-batched-tokens"]),
+                                      prefill_chunk=int(options["prefill-chunk"]), max_requests=slots,
+                                      arrival_steps=arrivals, return_scheduler=True)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - begun
+        generated = [output[len(prompt):] for output, prompt in zip(outputs, prompts)]
+        metrics = scheduler.metrics
+        requests = [scheduler.request(index) for index in range(len(prompts))]
+        report.update({
+            "request_count": len(prompts), "continuous_slots": slots or engine.cache.max_requests,
+            "prompt_lengths": lengths, "new_token_lengths": new_lengths, "arrival_steps": arrivals, "prompt_offsets": offsets,
+            "measured_ms": round(elapsed * 1e3, 3), "measured_tokens": sum(len(g) for g in generated),
+            "tokens_per_second": round(sum(len(g) for g in generated) / elapsed, 3),
+            "scheduler_steps": metrics.scheduler_steps, "slot_admissions": metrics.admissions,
+            "preemptions": metrics.preemptions, "prefill_tokens": metrics.prefill_tokens, "decode_tokens": metrics.decode_tokens,
+            "completed_requests": metrics.completed_requests, "peak_active_requests": metrics.peak_active_requests,
+            "peak_active_cache_bytes": metrics.peak_held_pages * (engine.cache.allocated_bytes() // max(1, report["kv_blocks"])),
+            "request_ttft_ms": [round((r.first_token_time - r.submit_time) * 1e3, 3) for r in requests],
+            "request_completion_ms": [round((r.completion_time - r.submit_time) * 1e3, 3) for r in requests],
+            "generated": generated, "token_checksum": int(sum((i + 1) * t for g in generated for i, t in enumerate(g)) % (1 << 31)),
+        })
+        print(json.dumps(report), flush=True)
+        return 0
+
+    prompts = [list(tokens) for _ in range(batch)]
+    if options["workload"] in ("prefill", "both"):
+        timings = []
+        logits = None
+        for iteration in range(int(options["prefill-warmup"]) + int(options["prefill-steps"])):
+            ids = [("prefill", iteration, row) for row in range(batch)]
+            for request_id in ids:
+                engine.open(request_id)
+            torch.cuda.synchronize()
+            begun = time.perf_counter()
+            logits = engine.step([StepEntry(request_id, prompt, [len(prompt) - 1]) for request_id, prompt in zip(ids, prompts)])
+            torch.cuda.synchronize()
+            if iteration >= int(options["prefill-warmup"]):
+                timings.append(time.perf_counter() - begun)
+            for request_id in ids:
+                engine.close(request_id)
+        report["prefill_ms"] = round(min(timings) * 1e3, 3)
+        report["prefill_tokens_per_second"] = round(batch * len(tokens) / min(timings), 3)
+        last = logits[0].cpu().numpy()
+        top = np.argsort(-last, kind="stable")[:int(options["top-k"])]
+        report["top_logits"] = [[int(index), float(last[index])] for index in top]
+        if options["logits-output"]:
+            last.astype("<f4").tofile(str(options["logits-output"]))       # apps/hf_infer.cpp:1175-1181
+    if options["workload"] == "decode" or (options["workload"] == "both" and options["decode-mode"] == "steady"):
+        steady = decode_throughput(engine, batch, max(len(tokens), capacity and capacity - int(options["steps"]) - int(options["warmup"]) or len(tokens)),
+                                   max(1, int(options["steps"])), int(options["warmup"]))
+        report["decode_tokens_per_second"] = round(steady["tokens_per_second"], 3)
+        report["decode_ms_per_step"] = round(steady["ms_per_step"], 4)
+    if options["workload"] == "both" and new_tokens > 0:
+        torch.cuda.synchronize()
+        begun = time.perf_counter()
+        outputs = generate(engine, prompts, params, max_batched_tokens=int(options["max-batched-tokens"]),
+                           prefill_chunk=int(options["prefill-chunk"]))
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - begun
+        report["generated_tokens"] = outputs[0][len(tokens):]
+        report["generation_ms"] = round(elapsed * 1e3, 3)
+        report["generation_tokens_per_second"] = round(sum(len(o) - len(tokens) for o in outputs) / elapsed, 3)
+    report["prompt_tokens"] = len(tokens)
+    print(json.dumps(report), flush=True)
+    return 0

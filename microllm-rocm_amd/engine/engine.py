@@ -80,7 +80,7 @@ class Engine:
         self.steps_run = 0
         # Steps in which every request brings one token are replayed from HIP graphs, one per (number of
         # requests, block-table width): the launches of a decode step cost more host time than GPU time.
-        self.use_graphs = use_graphs
+        self.use_graphs = use_graphs and all(part.graph_safe for part in self.model.parts())
         self._graphs: Dict[tuple, "_DecodeGraph"] = {}
         self.graph_replays = 0
 

@@ -23,6 +23,7 @@ from .spec import PartSpec
 
 
 class PagedAttention(Mixer):
+    graph_safe = True
     def __init__(self, spec: PartSpec, runtime: Runtime):
         super().__init__(spec, runtime)
         p = spec.params

@@ -52,6 +52,10 @@ CacheNeed = Union[PagedKVNeed, StateNeed, None]
 
 class Part:
     category = "part"
+    # True for a part whose forward launches the same kernels on the same addresses whatever the step's
+    # contents, reads the step's metadata on the device only, and may run twice without changing the
+    # result: the engine replays decode steps from HIP graphs only if every part of the model says so.
+    graph_safe = False
 
     def __init__(self, spec: PartSpec, runtime: Runtime):
         self.spec = spec

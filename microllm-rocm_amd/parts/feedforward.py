@@ -18,6 +18,7 @@ from .spec import PartSpec
 
 
 class SwiGLU(FeedForward):
+    graph_safe = True
     def __init__(self, spec: PartSpec, runtime: Runtime):
         super().__init__(spec, runtime)
         self.hidden = int(spec.params["hidden_size"])

@@ -22,6 +22,7 @@ from .spec import ModelSpec, PartSpec
 class TokenEmbedding(Part):
     """``h0[t] = E[id_t]`` widened to float32 (src/model/model.cpp:1111)."""
     category = "embedding"
+    graph_safe = True
 
     def __init__(self, spec: PartSpec, runtime: Runtime):
         super().__init__(spec, runtime)
@@ -43,6 +44,7 @@ class LMHead(Part):
     """``logits = x W^T`` in float32; a tied head names the embedding's table as its weight
     (src/model/model.cpp:1121-1128)."""
     category = "head"
+    graph_safe = True
 
     def __init__(self, spec: PartSpec, runtime: Runtime):
         super().__init__(spec, runtime)
@@ -97,6 +99,15 @@ class Model:
             block.bind(tensors)
         self.final_norm.bind(tensors)
         self.head.bind(tensors)
+
+    def parts(self) -> List[Part]:
+        found: List[Part] = [self.embedding, self.final_norm, self.head]
+        for block in self.blocks:
+            found += list(block.parts())
+            position = getattr(block.mixer, "position", None)
+            if position is not None:
+                found.append(position)
+        return found
 
     def cache_needs(self) -> List[CacheNeed]:
         """The cache need of every run entry; None for an entry that owns none."""

@@ -17,6 +17,7 @@ from .spec import PartSpec
 
 
 class RMSNorm(Norm):
+    graph_safe = True
     def __init__(self, spec: PartSpec, runtime: Runtime):
         super().__init__(spec, runtime)
         self.size = int(spec.params["size"])

@@ -16,6 +16,7 @@ from .spec import PartSpec
 
 
 class RopeSplitHalf(PositionEncoding):
+    graph_safe = True
     fused_split_half = True
 
     def __init__(self, spec: PartSpec, runtime: Runtime):

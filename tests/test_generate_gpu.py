@@ -1,0 +1,127 @@
+"""Generation through the entry point, the scheduler on the real engine, and the command line."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import plain_qwen2 as plain
+from replay_tools import PlainModel
+from tiny import CONFIGS, make_folder, random_tokens
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SHARP = {"std": 0.12, "norm_std": 0.1}
+
+
+def engine_for(folder, dtype="float32", **options):
+    from microllm_rocm_amd import Engine
+    options.setdefault("max_tokens", 1024)
+    return Engine.from_folder(folder, dtype=dtype, **options)
+
+
+@pytest.mark.parametrize("which,lengths,new_tokens", [("A", (7, 13), 8), ("B", (5, 17, 40, 64), 16)])
+def test_greedy_generation_matches_the_plain_implementation(tmp_path, which, lengths, new_tokens):
+    from microllm_rocm_amd import GenerationConfig, generate, generate_serial
+    folder = make_folder(tmp_path, which, SHARP)
+    model = PlainModel(folder)
+    config = CONFIGS[which]
+    prompts = [random_tokens(1 + index, length, config.vocab_size) for index, length in enumerate(lengths)]
+    expected = [prompt + plain.generate_greedy(model.config, model.weights, prompt, new_tokens) for prompt in prompts]
+    engine = engine_for(folder)
+    params = GenerationConfig(max_new_tokens=new_tokens, temperature=0.0)
+    assert generate(engine, prompts, params, prefill_chunk=16, max_batched_tokens=24,
+                    arrival_steps=[0, 1, 3, 4][:len(prompts)]) == expected
+    assert [generate_serial(engine, prompt, params) for prompt in prompts] == expected
+    assert generate(engine, prompts[0], params) == expected[0]          # one prompt in, one sequence out
+    engine.cache.check()
+    assert not engine.cache.requests
+    bf16 = generate(engine_for(folder, "bfloat16"), prompts, params, prefill_chunk=16)
+    same = sum(a == b for got, want in zip(bf16, expected) for a, b in zip(got, want))
+    assert same >= 0.9 * sum(len(want) for want in expected)            # rounding may flip a near tie
+
+
+def test_sampling_in_batches_equals_requests_run_alone_and_follows_the_plain_rule(tmp_path):
+    from microllm_rocm_amd import GenerationConfig, generate, generate_serial
+    folder = make_folder(tmp_path, "B", SHARP)
+    model = PlainModel(folder)
+    config = CONFIGS["B"]
+    prompts = [random_tokens(30 + index, length, config.vocab_size) for index, length in enumerate((5, 17, 40, 64))]
+    params = [GenerationConfig(max_new_tokens=16, temperature=0.8, seed=index, top_k=(0, 20)[index % 2]) for index in range(4)]
+    engine = engine_for(folder)
+    batched = generate(engine, prompts, params, prefill_chunk=16, max_batched_tokens=32, arrival_steps=[0, 2, 2, 5])
+    alone = [generate_serial(engine, prompt, p) for prompt, p in zip(prompts, params)]
+    assert batched == alone
+    # every drawn token is the one the plain rule draws from the plain logits of the same prefix
+    for sequence, prompt, p in zip(batched, prompts, params):
+        for draw in range(16):
+            prefix = sequence[:len(prompt) + draw]
+            expected = plain.sample(model.logits(prefix)[-1], p.temperature, p.top_k, plain.uniform_for(p.seed, draw))
+            if expected != sequence[len(prompt) + draw]:
+                # float32 against float64 logits: only a draw that falls on an interval's edge may differ
+                weights = plain.sampling_weights(model.logits(prefix)[-1], p.temperature, p.top_k)
+                cumulative = np.cumsum(weights) / weights.sum()
+                target = plain.uniform_for(p.seed, draw)
+                assert min(abs(cumulative - target)) < 1e-4
+                break
+
+
+def test_few_pages_preempt_and_recompute_to_the_same_tokens(tmp_path):
+    from microllm_rocm_amd import GenerationConfig, generate
+    folder = make_folder(tmp_path, "A", SHARP)
+    config = CONFIGS["A"]
+    prompts = [random_tokens(50 + index, 30, config.vocab_size) for index in range(3)]
+    params = GenerationConfig(max_new_tokens=40, temperature=0.0)
+    roomy = generate(engine_for(folder, max_tokens=1024), prompts, params)
+    tight_engine = engine_for(folder, num_pages=9, max_tokens=None)           # 9 pages of 16: three requests of 70 do not fit
+    tight, scheduler = generate(tight_engine, prompts, params, return_scheduler=True)
+    assert scheduler.metrics.preemptions >= 1
+    assert tight == roomy
+    assert tight_engine.cache.free_pages() == [9]
+
+
+def test_stop_tokens_and_limits(tmp_path):
+    from microllm_rocm_amd import GenerationConfig, Scheduler, generate
+    folder = make_folder(tmp_path, "A", SHARP)
+    engine = engine_for(folder)
+    prompt = random_tokens(9, 11, CONFIGS["A"].vocab_size)
+    free_run = generate(engine, prompt, GenerationConfig(max_new_tokens=12, temperature=0.0))[len(prompt):]
+    stopped = generate(engine, prompt, GenerationConfig(max_new_tokens=12, temperature=0.0, stop_tokens=(free_run[3],)))
+    assert stopped[len(prompt):] == free_run[:free_run.index(free_run[3]) + 1]
+    with pytest.raises(ValueError, match="max positions"):
+        Scheduler(engine).submit(prompt, GenerationConfig(max_new_tokens=200))
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        generate(engine, [[999]], GenerationConfig(max_new_tokens=1))
+
+
+def test_command_line(tmp_path):
+    folder = make_folder(tmp_path, "B", SHARP)
+    model = PlainModel(folder)
+    prompt = random_tokens(3, 9, CONFIGS["B"].vocab_size)
+    expected = plain.generate_greedy(model.config, model.weights, prompt, 6)
+    logits_path = tmp_path / "last.f32"
+    command = [sys.executable, os.path.join(ROOT, "bin", "microllm_hf_infer"), "--config", os.path.join(folder, "config.json"),
+               "--weights", os.path.join(folder, "model.safetensors"), "--tokens", ",".join(map(str, prompt)),
+               "--device", "hip", "--dtype", "float32", "--new-tokens", "6", "--logits-output", str(logits_path)]
+    result = subprocess.run(command, capture_output=True, text=True, timeout=300)
+    assert result.returncode == 0, result.stderr
+    report = json.loads(result.stdout.strip().splitlines()[-1])
+    assert report["generated_tokens"] == expected and report["prompt_tokens"] == len(prompt)
+    last = np.fromfile(logits_path, dtype="<f4")
+    reference = model.logits(prompt)[-1]
+    assert np.abs(last - reference).max() <= 2e-5 * np.abs(reference).max()
+    bad = subprocess.run(command + ["--bogus", "1"], capture_output=True, text=True, timeout=120)
+    assert bad.returncode != 0 and "bogus" in bad.stderr
+    continuous = subprocess.run(command[:6] + ["--tokens", ",".join(map(str, prompt)), "--device", "hip", "--dtype", "float32",
+                                               "--workload", "continuous", "--continuous-prompt-lengths", "5,9,7",
+                                               "--continuous-new-token-lengths", "4,6,3", "--continuous-arrival-steps", "0,1,1",
+                                               "--continuous-slots", "2"], capture_output=True, text=True, timeout=300)
+    assert continuous.returncode == 0, continuous.stderr
+    report = json.loads(continuous.stdout.strip().splitlines()[-1])
+    assert report["completed_requests"] == 3 and [len(r) for r in report["generated"]] == [4, 6, 3]
+    for generated, length, new in zip(report["generated"], (5, 9, 7), (4, 6, 3)):
+        cyclic = [prompt[i % len(prompt)] for i in range(length)]
+        assert generated == plain.generate_greedy(model.config, model.weights, cyclic, new)
