@@ -384,7 +384,8 @@ def pack_weight(weight: torch.Tensor, interleave_halves: bool = False) -> torch.
 SKINNY_MAX_ROWS = 64
 
 
-def gemm_skinny(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f32") -> torch.Tensor:
+def gemm_skinny(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f32",
+                rows: Optional[int] = None) -> torch.Tensor:
     """``x @ W.T`` for at most 64 bfloat16 rows and a packed weight.
 
     ``f32``: float32 ``[m, n]``; ``bf16``: bfloat16 ``[m, n]``; ``gated``: bfloat16 ``[m, n / 2]`` of
@@ -393,8 +394,15 @@ def gemm_skinny(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "
     lib = library.load()
     _device_tensor(x, "gemm input", torch.bfloat16)
     _device_tensor(packed, "packed weight", torch.bfloat16)
-    _need(x.dim() == 2 and packed.dim() == 5 and tuple(packed.shape[2:]) == (4, 16, 8), "gemm_skinny takes [m, k] and a packed weight")
-    m, k = x.shape
+    _need(packed.dim() == 5 and tuple(packed.shape[2:]) == (4, 16, 8), "gemm_skinny takes a packed weight")
+    a_packed = x.dim() == 5       # activations in piece order [m/16, k/32, 4, 16, 8]; `rows` says how many are real
+    if a_packed:
+        _need(tuple(x.shape[2:]) == (4, 16, 8) and rows is not None and rows <= x.shape[0] * 16, "bad packed activations")
+        m, k = rows, packed.shape[1] * 32
+        _need(x.shape[1] == packed.shape[1], "packed activations and weight differ in k")
+    else:
+        _need(x.dim() == 2, "gemm_skinny takes [m, k] activations")
+        m, k = x.shape
     _need(m <= SKINNY_MAX_ROWS, "gemm_skinny takes at most 64 rows")
     _need(k % 8 == 0, "gemm_skinny needs k to be a multiple of 8")
     _need(packed.shape[0] == -(-n // 16) and packed.shape[1] == -(-k // 32), "the packed weight does not fit n and k")
@@ -406,5 +414,5 @@ def gemm_skinny(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "
         code, out = 2, torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
     else:
         raise KernelLibraryError(f"unknown epilogue {epilogue!r}")
-    _check(lib.mll_gemm_skinny(_ptr(x), _ptr(packed), _ptr(out), code, m, n, k, _stream()), lib)
+    _check(lib.mll_gemm_skinny(_ptr(x), int(a_packed), _ptr(packed), _ptr(out), code, m, n, k, _stream()), lib)
     return out

@@ -306,11 +306,12 @@ def test_a_far_key_among_hundreds_and_the_window_edge(kernel):
 
 # ---- feed-forward activation -------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_silu_mul(dtype):
+@pytest.mark.parametrize("width", [203, 208, 4864])
+def test_silu_mul(dtype, width):
     rng = np.random.default_rng(1)
-    reference, gate_up = prepare(np.concatenate([rng.normal(size=(9, 2 * 203)) * 4, [[-90.0] * 203 + [1.0] * 203]]), dtype)
+    reference, gate_up = prepare(np.concatenate([rng.normal(size=(9, 2 * width)) * 4, [[-90.0] * width + [1.0] * width]]), dtype)
     out = kernels().silu_mul(gate_up)
-    expected = plain.silu(reference[:, :203]) * reference[:, 203:]
+    expected = plain.silu(reference[:, :width]) * reference[:, width:]
     np.testing.assert_allclose(out.float().cpu().numpy(), expected, **tolerance(dtype))
     vector = kernels().silu_mul(torch.tensor([[-1.0, 0.0, 1.0, 2.0, 2.0, 2.0]], device=DEVICE)).cpu().numpy()[0]
     np.testing.assert_allclose(vector, [-2 / (1 + math.e), 0.0, 2 / (1 + math.exp(-1))], rtol=1e-6)   # ops_test.cpp:487-495
@@ -414,6 +415,8 @@ def test_gemm_skinny(m, n, k):
     assert np.abs(full.double().cpu().numpy() - expected).max() <= 1e-5 * scale
     out = ka.gemm_skinny(a, packed, n, "bf16")
     assert out.dtype == torch.bfloat16 and np.abs(out.float().cpu().numpy() - expected).max() <= 5e-3 * scale
+    # activations given in the weight's piece order give the same numbers
+    assert torch.equal(ka.gemm_skinny(ka.pack_weight(a), packed, n, "f32", rows=m), full)
     # the same in every run; and among calls of up to 16 rows a row's result does not depend on the other rows
     assert torch.equal(ka.gemm_skinny(a, packed, n, "f32"), full)
     if m <= 16:
