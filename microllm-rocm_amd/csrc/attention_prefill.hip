@@ -1,12 +1,13 @@
 // Paged attention for portions of prompts in bfloat16: MFMA for both products, online softmax in float32.
 //
-// A workgroup (4 waves) takes 64 consecutive tokens of one request's portion and one query head; a wave
-// takes 16 of those tokens. As in the decode kernel, scores are computed transposed, S^T = K . Q^T, with the
-// 16 columns now being 16 query positions, and O^T = V^T . P^T follows from registers alone. A wave walks the
-// keys of its request from the first one any of its queries can see to its last query's own position, in
-// pairs of 16-key tiles read straight from the pages (which are laid out in MFMA order, cache_layout.h);
-// only pairs that touch the causal diagonal or the window's edge pay for the mask.
-// The list of 64-token tiles (request, first token in the flat list, tokens in the tile) is built on the host.
+// A workgroup (4 waves) takes up to 128 consecutive tokens of one request's portion and one query head; a wave
+// takes 32 of them as two blocks of 16 columns. The workgroup walks the keys its tokens can see in blocks of
+// 64 (32 for head sizes above 128): the block's key and value tiles are copied from the pages into LDS as they
+// lie there (the pages are in MFMA order, cache_layout.h), the next block's being fetched from memory while
+// this one is used. As in the decode kernel, scores are computed transposed, S^T = K . Q^T, the 16 columns
+// being query positions, and O^T = V^T . P^T follows from registers; every fragment of K and V read from LDS
+// serves both column blocks. Only pairs of tiles that touch the causal diagonal or the window's edge pay
+// for the mask. The list of tiles (request, first token in the flat list, tokens) is built on the host.
 #include "cache_layout.h"
 #include "common.h"
 #include "microllm_hip.h"
@@ -19,7 +20,8 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kPrefillWaves = 4;
 constexpr int kPrefillThreads = kPrefillWaves * kWave;
-constexpr int kPrefillTile = 16 * kPrefillWaves;   // tokens per workgroup
+constexpr int kPrefillWaveTokens = 32;
+constexpr int kPrefillTile = kPrefillWaveTokens * kPrefillWaves;   // tokens per workgroup
 
 union PFrag8 {
     bf16x8 v;
@@ -28,7 +30,7 @@ union PFrag8 {
 };
 
 template <int HD_TILES>
-__global__ __launch_bounds__(kPrefillThreads) void paged_attention_prefill_kernel(
+__global__ __launch_bounds__(kPrefillThreads, 2) void paged_attention_prefill_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles,
     const int32_t* __restrict__ positions, bf16* __restrict__ out, float scale, int window, int heads,
@@ -36,6 +38,12 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_attention_prefill_kerne
     constexpr int HD = HD_TILES * 16;
     constexpr int K_STEPS = (HD + 31) / 32;
     constexpr int K_CHUNKS = HD / 8;
+    constexpr int BLOCK_KEYS = HD <= 128 ? 64 : 32;
+    constexpr int BLOCK_TILES = BLOCK_KEYS / 16;
+    constexpr int TILE_ELEMENTS = HD * 16;                       // of keys and of values alike
+    constexpr int TILE_PASSES = (TILE_ELEMENTS * 2 + kPrefillThreads * 16 - 1) / (kPrefillThreads * 16);
+    extern __shared__ __align__(16) bf16 lds[];                  // [2 stages][K | V][BLOCK_TILES][TILE_ELEMENTS]
+    constexpr int STAGE_ELEMENTS = 2 * BLOCK_TILES * TILE_ELEMENTS;
 
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
@@ -47,129 +55,200 @@ __global__ __launch_bounds__(kPrefillThreads) void paged_attention_prefill_kerne
     const int tile_count = tiles[3 * blockIdx.x + 2];
     const int head = blockIdx.y;
     const int kv_head = head / (heads / kv_heads);
-    const int first = wave * 16;              // this wave's first token inside the tile
-    if (first >= tile_count) return;
-    const int valid = min(16, tile_count - first);
-    const int token0 = tile_token + first;
-    const int position0 = positions[token0];  // tokens of a portion have consecutive positions
-    const int my_position = position0 + min(col, valid - 1);   // columns past the end repeat the last token
-    const int last_position = position0 + valid - 1;
-    const int my_low = window > 0 ? max(0, my_position - window + 1) : 0;
-    const int first_low = window > 0 ? max(0, position0 - window + 1) : 0;
-    const int last_low = window > 0 ? max(0, last_position - window + 1) : 0;
     const int32_t* table = block_table + static_cast<int64_t>(seq) * table_width;
     const CacheLayout layout(kv_heads, page_size, HD);
+    const float scale_log2 = scale * 1.4426950408889634f;      // scores are kept in units of log 2: p = 2^(s - max)
 
-    PFrag8 q_frag[K_STEPS];
+    // The workgroup's tokens and the keys any of them can see.
+    const int tile_position = positions[tile_token];             // tokens of a portion have consecutive positions
+    const int group_last = tile_position + tile_count - 1;
+    const int group_low = window > 0 ? max(0, tile_position - window + 1) : 0;
+    // This wave's tokens.
+    const int wave_first = wave * kPrefillWaveTokens;
+    const int wave_valid = min(kPrefillWaveTokens, max(0, tile_count - wave_first));
+    const int column_blocks = (wave_valid + 15) / 16;
+    const int wave_position = tile_position + wave_first;
+    const int wave_last = wave_position + wave_valid - 1;
+    const int wave_low = window > 0 ? max(0, wave_position - window + 1) : 0;
+    const int wave_last_low = window > 0 ? max(0, wave_last - window + 1) : 0;
+
+    PFrag8 q_frag[2][K_STEPS];
+    int my_position[2], my_low[2];
 #pragma unroll
-    for (int ks = 0; ks < K_STEPS; ++ks) {
-        const int dim = ks * 32 + quad * 8;
-        q_frag[ks].raw = make_uint4(0, 0, 0, 0);
-        if (dim < HD)
-            q_frag[ks].raw = *reinterpret_cast<const uint4*>(
-                q + (static_cast<int64_t>(token0 + min(col, valid - 1)) * heads + head) * HD + dim);
+    for (int c = 0; c < 2; ++c) {
+        const int valid = min(16, max(0, wave_valid - 16 * c));
+        const int index = wave_first + 16 * c + min(col, max(valid - 1, 0));      // columns past the end repeat the last token
+        my_position[c] = tile_position + index;
+        my_low[c] = window > 0 ? max(0, my_position[c] - window + 1) : 0;
+#pragma unroll
+        for (int ks = 0; ks < K_STEPS; ++ks) {
+            const int dim = ks * 32 + quad * 8;
+            q_frag[c][ks].raw = make_uint4(0, 0, 0, 0);
+            if (valid > 0 && dim < HD)
+                q_frag[c][ks].raw = *reinterpret_cast<const uint4*>(
+                    q + (static_cast<int64_t>(tile_token + index) * heads + head) * HD + dim);
+        }
     }
 
-    floatx4 o_acc[HD_TILES];
+    floatx4 o_acc[2][HD_TILES];
+    float running_max[2] = {-INFINITY, -INFINITY}, running_sum[2] = {0.0f, 0.0f};
 #pragma unroll
-    for (int d = 0; d < HD_TILES; ++d) o_acc[d] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-    float running_max = -INFINITY, running_sum = 0.0f;
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int d = 0; d < HD_TILES; ++d) o_acc[c][d] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    auto page_of = [&](int tile_key) -> int {
-        return (tile_key <= last_position && tile_key + 15 >= first_low) ? table[tile_key / page_size] : -1;
-    };
-    const int pair_end = last_position / 32 + 1;
-    int pair = first_low / 32;
-    int next_page[2] = {page_of(pair * 32), page_of(pair * 32 + 16)};
-    for (; pair < pair_end; ++pair) {
-        const int key0 = pair * 32;
-        const int page[2] = {next_page[0], next_page[1]};
-        if (pair + 1 < pair_end) {
-            next_page[0] = page_of((pair + 1) * 32);
-            next_page[1] = page_of((pair + 1) * 32 + 16);
-        }
-        PFrag8 k_frag[2][K_STEPS];
-        PFrag8 v_frag[HD_TILES];
+    // Copy of one block's tiles: thread i moves bytes [16 i, 16 i + 16) of every pass of every tile.
+    uint4 staged[BLOCK_TILES][2][TILE_PASSES];
+    auto fetch = [&](int block) {
 #pragma unroll
-        for (int d = 0; d < HD_TILES; ++d) v_frag[d].raw = make_uint4(0, 0, 0, 0);
+        for (int t = 0; t < BLOCK_TILES; ++t) {
+            const int tile_key = block * BLOCK_KEYS + 16 * t;
+            const bool live = tile_key <= group_last && tile_key + 15 >= group_low;
+            const int64_t page = live ? table[tile_key / page_size] : 0;
+            const int offset = tile_key % page_size;
+            const bf16* k_tile = k_cache + layout.k_tile(page, kv_head, offset / 16);
+            const bf16* v_tile = v_cache + layout.v_tile(page, kv_head, offset / 16);
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const int offset = (key0 + 16 * t) % page_size;
-            const bf16* k_tile = k_cache + layout.k_tile(max(page[t], 0), kv_head, offset / 16) + col * 8;
-            const bf16* v_tile = v_cache + layout.v_tile(max(page[t], 0), kv_head, offset / 16) + (quad * 16 + col) * 4;
-#pragma unroll
-            for (int ks = 0; ks < K_STEPS; ++ks) {
-                const int piece = ks * 4 + quad;
-                k_frag[t][ks].raw = make_uint4(0, 0, 0, 0);
-                if (page[t] >= 0 && piece < K_CHUNKS)
-                    k_frag[t][ks].raw = *reinterpret_cast<const uint4*>(k_tile + piece * 128);
-            }
-            if (page[t] >= 0) {
-#pragma unroll
-                for (int d = 0; d < HD_TILES; ++d)
-                    v_frag[d].h[t] = *reinterpret_cast<const bf16x4*>(v_tile + d * 256);
-            }
-        }
-
-        float score[8];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            floatx4 s = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-            for (int ks = 0; ks < K_STEPS; ++ks)
-                s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_frag[t][ks].v, q_frag[ks].v, s, 0, 0, 0);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) score[4 * t + i] = s[i] * scale;
-        }
-        // Pairs every query of the wave sees whole need no mask.
-        if (key0 + 31 > position0 || key0 < last_low) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int key = key0 + 16 * (j / 4) + 4 * quad + (j % 4);
-                if (key > my_position || key < my_low) score[j] = -INFINITY;
-                // Keys no query of the wave can see may be stale memory: keep them out of the product.
-                if (key > last_position || key < first_low) {
-#pragma unroll
-                    for (int d = 0; d < HD_TILES; ++d) v_frag[d].v[j] = static_cast<__bf16>(0.0f);
+            for (int pass = 0; pass < TILE_PASSES; ++pass) {
+                const int element = (pass * kPrefillThreads + threadIdx.x) * 8;
+                staged[t][0][pass] = make_uint4(0, 0, 0, 0);
+                staged[t][1][pass] = make_uint4(0, 0, 0, 0);
+                if (live && element < TILE_ELEMENTS) {
+                    staged[t][0][pass] = *reinterpret_cast<const uint4*>(k_tile + element);
+                    staged[t][1][pass] = *reinterpret_cast<const uint4*>(v_tile + element);
                 }
             }
         }
+    };
+    auto stash = [&](int stage) {
+        bf16* base = lds + stage * STAGE_ELEMENTS;
+#pragma unroll
+        for (int t = 0; t < BLOCK_TILES; ++t)
+#pragma unroll
+            for (int pass = 0; pass < TILE_PASSES; ++pass) {
+                const int element = (pass * kPrefillThreads + threadIdx.x) * 8;
+                if (element < TILE_ELEMENTS) {
+                    *reinterpret_cast<uint4*>(base + t * TILE_ELEMENTS + element) = staged[t][0][pass];
+                    *reinterpret_cast<uint4*>(base + (BLOCK_TILES + t) * TILE_ELEMENTS + element) = staged[t][1][pass];
+                }
+            }
+    };
 
-        float tile_max = score[0];
+    const int first_block = group_low / BLOCK_KEYS;
+    const int last_block = group_last / BLOCK_KEYS;
+    fetch(first_block);
+    stash(0);
+    __syncthreads();
+    for (int block = first_block; block <= last_block; ++block) {
+        const int stage = (block - first_block) & 1;
+        if (block < last_block) fetch(block + 1);
+        const bf16* k_lds = lds + stage * STAGE_ELEMENTS;
+        const bf16* v_lds = k_lds + BLOCK_TILES * TILE_ELEMENTS;
+
+        if (wave_valid > 0) {
 #pragma unroll
-        for (int j = 1; j < 8; ++j) tile_max = fmaxf(tile_max, score[j]);
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
-        const float new_max = fmaxf(running_max, tile_max);
-        // A query may see nothing of a pair that others see (the window's edge): its maximum stays -inf.
-        const float safe_max = new_max == -INFINITY ? 0.0f : new_max;
-        const float rescale = __expf(running_max - safe_max);
-        PFrag8 p_frag;
-        float tile_sum = 0.0f;
+            for (int pair = 0; pair < BLOCK_TILES / 2; ++pair) {
+                const int key0 = block * BLOCK_KEYS + 32 * pair;
+                if (key0 > wave_last || key0 + 31 < wave_low) continue;   // nothing of this pair is visible to the wave
+                PFrag8 k_frag[2][K_STEPS];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const float p = __expf(score[j] - safe_max);
-            tile_sum += p;
-            p_frag.v[j] = static_cast<__bf16>(p);
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int ks = 0; ks < K_STEPS; ++ks) {
+                        const int piece = ks * 4 + quad;
+                        k_frag[t][ks].raw = make_uint4(0, 0, 0, 0);
+                        if (piece < K_CHUNKS)
+                            k_frag[t][ks].raw = *reinterpret_cast<const uint4*>(
+                                k_lds + (2 * pair + t) * TILE_ELEMENTS + piece * 128 + col * 8);
+                    }
+                const bool needs_mask = key0 + 31 > wave_position || key0 < wave_last_low;
+                PFrag8 p_frag[2];
+                float rescale[2];
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    if (c >= column_blocks) {
+                        p_frag[c].raw = make_uint4(0, 0, 0, 0);
+                        rescale[c] = 1.0f;
+                        continue;
+                    }
+                    float score[8];
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        floatx4 s = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                        for (int ks = 0; ks < K_STEPS; ++ks)
+                            s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_frag[t][ks].v, q_frag[c][ks].v, s, 0, 0, 0);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) score[4 * t + i] = s[i] * scale_log2;
+                    }
+                    if (needs_mask) {
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const int key = key0 + 16 * (j / 4) + 4 * quad + (j % 4);
+                            if (key > my_position[c] || key < my_low[c]) score[j] = -INFINITY;
+                        }
+                    }
+                    float tile_max = score[0];
+#pragma unroll
+                    for (int j = 1; j < 8; ++j) tile_max = fmaxf(tile_max, score[j]);
+                    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
+                    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+                    const float new_max = fmaxf(running_max[c], tile_max);
+                    // A query may see nothing of a pair that others see (the window's edge): its maximum stays -inf.
+                    const float safe_max = new_max == -INFINITY ? 0.0f : new_max;
+                    rescale[c] = __builtin_amdgcn_exp2f(running_max[c] - safe_max);
+                    float tile_sum = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float p = __builtin_amdgcn_exp2f(score[j] - safe_max);
+                        tile_sum += p;
+                        p_frag[c].v[j] = static_cast<__bf16>(p);
+                    }
+                    tile_sum += __shfl_xor(tile_sum, 16, kWave);
+                    tile_sum += __shfl_xor(tile_sum, 32, kWave);
+                    running_sum[c] = running_sum[c] * rescale[c] + tile_sum;
+                    running_max[c] = new_max;
+                }
+                // Once the running maxima have settled, no column's sum needs rescaling: skip the multiplications.
+                const bool any_rescale = __any(rescale[0] != 1.0f || rescale[1] != 1.0f);
+#pragma unroll
+                for (int d = 0; d < HD_TILES; ++d) {
+                    PFrag8 v_frag;
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+                        v_frag.h[t] = *reinterpret_cast<const bf16x4*>(
+                            v_lds + (2 * pair + t) * TILE_ELEMENTS + d * 256 + (quad * 16 + col) * 4);
+                    if (needs_mask) {
+                        // Keys no token of the workgroup can see may be stale memory: 0 * NaN must not reach the sum.
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const int key = key0 + 16 * (j / 4) + 4 * quad + (j % 4);
+                            if (key > group_last || key < group_low) v_frag.v[j] = static_cast<__bf16>(0.0f);
+                        }
+                    }
+#pragma unroll
+                    for (int c = 0; c < 2; ++c) {
+                        if (any_rescale) o_acc[c][d] *= rescale[c];
+                        o_acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_frag.v, p_frag[c].v, o_acc[c][d], 0, 0, 0);
+                    }
+                }
+            }
         }
-        tile_sum += __shfl_xor(tile_sum, 16, kWave);
-        tile_sum += __shfl_xor(tile_sum, 32, kWave);
-        running_sum = running_sum * rescale + tile_sum;
-        running_max = new_max;
-#pragma unroll
-        for (int d = 0; d < HD_TILES; ++d) {
-            o_acc[d] *= rescale;
-            o_acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_frag[d].v, p_frag.v, o_acc[d], 0, 0, 0);
-        }
+        if (block < last_block) stash(stage ^ 1);
+        __syncthreads();
     }
 
-    if (col < valid) {
-        const float inverse = 1.0f / running_sum;
-        bf16* out_row = out + (static_cast<int64_t>(token0 + col) * heads + head) * HD;
 #pragma unroll
-        for (int d = 0; d < HD_TILES; ++d)
+    for (int c = 0; c < 2; ++c) {
+        const int valid = min(16, max(0, wave_valid - 16 * c));
+        if (col < valid) {
+            const float inverse = 1.0f / running_sum[c];
+            bf16* out_row = out + (static_cast<int64_t>(tile_token + wave_first + 16 * c + col) * heads + head) * HD;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) out_row[d * 16 + quad * 4 + i] = from_float<bf16>(o_acc[d][i] * inverse);
+            for (int d = 0; d < HD_TILES; ++d)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) out_row[d * 16 + quad * 4 + i] = from_float<bf16>(o_acc[c][d][i] * inverse);
+        }
     }
 }
 
@@ -177,8 +256,11 @@ template <int HD_TILES>
 static int launch_prefill(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
                           int table_width, const int32_t* tiles, int n_tiles, const int32_t* positions, void* out,
                           float scale, int window, int heads, int kv_heads, int page_size, hipStream_t stream) {
+    constexpr int HD = HD_TILES * 16;
+    constexpr int BLOCK_KEYS = HD <= 128 ? 64 : 32;
+    const size_t lds_bytes = 2 * 2 * (BLOCK_KEYS / 16) * HD * 16 * sizeof(bf16);   // at most 64 KB
     const dim3 grid(n_tiles, heads);
-    paged_attention_prefill_kernel<HD_TILES><<<grid, kPrefillThreads, 0, stream>>>(
+    paged_attention_prefill_kernel<HD_TILES><<<grid, kPrefillThreads, lds_bytes, stream>>>(
         static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), block_table,
         table_width, tiles, positions, static_cast<bf16*>(out), scale, window, heads, kv_heads, page_size);
     return check_launch("paged_attention_prefill");

@@ -16,7 +16,7 @@ import torch
 from ..cache.manager import CacheManager, RELEASED, RequestCache
 
 
-QUERY_TILE = 64   # tokens of one request that one workgroup of the prefill attention kernel takes
+QUERY_TILE = 128   # tokens of one request that one workgroup of the prefill attention kernel takes
 
 
 @dataclass
@@ -48,7 +48,7 @@ class StepContext:
     seq_total: torch.Tensor     # int32 [requests]: positions in the cache once this step is done
     slots: torch.Tensor         # int32 [requests]: state slot of every request
     want_rows: Optional[torch.Tensor]  # int32 [wanted]: rows of the flat list whose logits are wanted
-    query_tiles: torch.Tensor   # int32 [tiles, 3]: (request, first token in the flat list, tokens) per tile of <= 64 tokens
+    query_tiles: torch.Tensor   # int32 [tiles, 3]: (request, first token in the flat list, tokens) per tile of <= 128 tokens
     paged: List[PagedView]
     # the same on the host, for parts written in Python and for choosing kernels
     starts: List[int] = field(default_factory=list)
@@ -116,9 +116,11 @@ class BatchBuilder:
             mappings.append(mapping.astype(np.int32))
             widths.append(width)
         slots = np.asarray([request.slot for request in requests], dtype=np.int32)
-        query_tiles = np.asarray([(index, cu[index] + offset, min(QUERY_TILE, count - offset))
-                                  for index, count in enumerate(counts) for offset in range(0, count, QUERY_TILE)],
-                                 dtype=np.int32).reshape(-1, 3)
+        # Tiles with the most keys to walk come first, so that the longest workgroups start first.
+        tile_list = sorted(((index, cu[index] + offset, min(QUERY_TILE, count - offset))
+                            for index, count in enumerate(counts) for offset in range(0, count, QUERY_TILE)),
+                           key=lambda tile: -(starts[tile[0]] + tile[1] - cu[tile[0]] + tile[2]))
+        query_tiles = np.asarray(tile_list, dtype=np.int32).reshape(-1, 3)
         pieces = [tokens, positions, seq_of_token, cu, np.asarray(starts, np.int32), np.asarray(totals, np.int32),
                   slots, want_rows, query_tiles.reshape(-1)]
         for table, mapping in zip(tables, mappings):

@@ -245,12 +245,12 @@ def test_decode_attention(heads, kv_heads, hd, page_size, window, splits):
     (2, 1, 80, 16, 300), (3, 3, 256, 16, 0), (7, 7, 112, 64, 129), (6, 3, 96, 48, 17)])
 def test_prefill_attention(heads, kv_heads, hd, page_size, window):
     rng = np.random.default_rng(heads + hd + window)
-    lengths, counts = [517, 1, 200, 97, 64, 131, 40], [130, 1, 200, 17, 64, 2, 33]
+    lengths, counts = [517, 1, 300, 97, 64, 131, 40], [130, 1, 300, 17, 64, 2, 33]
     t, q_exact, ek, ev, seq, pos = build_paged_case(rng, torch.bfloat16, lengths, counts, heads, kv_heads, hd, page_size)
     scale = 1.0 / math.sqrt(hd)
     tiles, start = [], 0
     for index, count in enumerate(counts):
-        tiles += [(index, start + offset, min(64, count - offset)) for offset in range(0, count, 64)]
+        tiles += [(index, start + offset, min(128, count - offset)) for offset in range(0, count, 128)]
         start += count
     query_tiles = torch.tensor(tiles, dtype=torch.int32, device=DEVICE)
     out = kernels().paged_attention_prefill(t["q"], t["k"], t["v"], t["table"], query_tiles, t["pos"], scale, window,
