@@ -30,8 +30,9 @@ template <int HD_TILES>
 __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ seq_of_token,
-    const int32_t* __restrict__ positions, bf16* __restrict__ out, float* __restrict__ part_o,
-    float* __restrict__ part_ml, float scale, int window, int heads, int kv_heads, int page_size, int n_splits) {
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ token_ids, bf16* __restrict__ out,
+    float* __restrict__ part_o, float* __restrict__ part_ml, float scale, int window, int heads, int kv_heads,
+    int page_size, int n_splits) {
     constexpr int HD = HD_TILES * 16;
     constexpr int K_STEPS = (HD + 31) / 32;
     constexpr int K_CHUNKS = HD / 8;
@@ -42,7 +43,7 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
     __shared__ float m_shared[kSlots][16];
     __shared__ float l_shared[kSlots][16];
 
-    const int token = blockIdx.x;
+    const int token = token_ids ? token_ids[blockIdx.x] : blockIdx.x;   // a step may give the kernel some of its tokens only
     const int group = heads / kv_heads;
     const int chunks = (group + 15) / 16;
     const int kv_head = blockIdx.y / chunks;
@@ -228,13 +229,14 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
             sum += weight * l_shared[w][h];
         }
         const int64_t row = static_cast<int64_t>(token) * heads + head0 + h;
+        const int64_t part_row = static_cast<int64_t>(blockIdx.x) * heads + head0 + h;   // partial results are kept densely
         if (n_splits == 1) {
             out[row * HD + dim] = from_float<bf16>(total / sum);
         } else {
-            part_o[(row * n_splits + split) * HD + dim] = total;
+            part_o[(part_row * n_splits + split) * HD + dim] = total;
             if (dim == 0) {
-                part_ml[(row * n_splits + split) * 2 + 0] = top;
-                part_ml[(row * n_splits + split) * 2 + 1] = sum;
+                part_ml[(part_row * n_splits + split) * 2 + 0] = top;
+                part_ml[(part_row * n_splits + split) * 2 + 1] = sum;
             }
         }
     }
@@ -242,9 +244,12 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
 
 // Joins the splits of one (token, head): out = sum_s w_s O_s / sum_s w_s l_s with w_s = exp(m_s - max m).
 __global__ void paged_attention_join_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                            bf16* __restrict__ out, int head_dim, int n_splits) {
-    const int64_t row = blockIdx.x;
-    const float* ml = part_ml + row * n_splits * 2;
+                                            const int32_t* __restrict__ token_ids, bf16* __restrict__ out, int heads,
+                                            int head_dim, int n_splits) {
+    const int token = token_ids ? token_ids[blockIdx.x / heads] : blockIdx.x / heads;
+    const int64_t row = static_cast<int64_t>(token) * heads + blockIdx.x % heads;
+    const int64_t part_row = blockIdx.x;
+    const float* ml = part_ml + part_row * n_splits * 2;
     float top = -INFINITY;
     for (int s = 0; s < n_splits; ++s) top = fmaxf(top, ml[2 * s]);
     for (int dim = threadIdx.x; dim < head_dim; dim += blockDim.x) {
@@ -253,7 +258,7 @@ __global__ void paged_attention_join_kernel(const float* __restrict__ part_o, co
             const float m = ml[2 * s];
             if (m == -INFINITY) continue;   // a split without keys
             const float weight = __expf(m - top);
-            total += weight * part_o[(row * n_splits + s) * head_dim + dim];
+            total += weight * part_o[(part_row * n_splits + s) * head_dim + dim];
             weight_sum += weight * ml[2 * s + 1];
         }
         out[row * head_dim + dim] = from_float<bf16>(total / weight_sum);
@@ -262,15 +267,15 @@ __global__ void paged_attention_join_kernel(const float* __restrict__ part_o, co
 
 template <int HD_TILES>
 static int launch_decode(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
-                         int table_width, const int32_t* seq_of_token, const int32_t* positions, void* out,
-                         float* part_o, float* part_ml, float scale, int window, int n_tokens, int heads, int kv_heads,
-                         int page_size, int n_splits, hipStream_t stream) {
+                         int table_width, const int32_t* seq_of_token, const int32_t* positions,
+                         const int32_t* token_ids, void* out, float* part_o, float* part_ml, float scale, int window,
+                         int n_tokens, int heads, int kv_heads, int page_size, int n_splits, hipStream_t stream) {
     const int group = heads / kv_heads;
     const dim3 grid(n_tokens, kv_heads * ((group + 15) / 16), n_splits);
     paged_attention_decode_kernel<HD_TILES><<<grid, kDecodeThreads, 0, stream>>>(
         static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), block_table,
-        table_width, seq_of_token, positions, static_cast<bf16*>(out), part_o, part_ml, scale, window, heads, kv_heads,
-        page_size, n_splits);
+        table_width, seq_of_token, positions, token_ids, static_cast<bf16*>(out), part_o, part_ml, scale, window, heads,
+        kv_heads, page_size, n_splits);
     return check_launch("paged_attention_decode");
 }
 
@@ -280,9 +285,9 @@ using namespace mll;
 
 extern "C" int mll_paged_attention_decode(const void* q, const void* k_cache, const void* v_cache,
                                           const int32_t* block_table, int table_width, const int32_t* seq_of_token,
-                                          const int32_t* positions, void* out, float* part_o, float* part_ml,
-                                          float scale, int window, int n_tokens, int heads, int kv_heads, int head_dim,
-                                          int page_size, int n_splits, hipStream_t stream) {
+                                          const int32_t* positions, const int32_t* token_ids, void* out, float* part_o,
+                                          float* part_ml, float scale, int window, int n_tokens, int heads, int kv_heads,
+                                          int head_dim, int page_size, int n_splits, hipStream_t stream) {
     MLL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "paged_attention_decode: heads must divide into kv_heads groups");
     MLL_REQUIRE(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256,
                 "paged_attention_decode: head_dim must be a multiple of 16 in [16, 256]");
@@ -294,9 +299,9 @@ extern "C" int mll_paged_attention_decode(const void* q, const void* k_cache, co
     int status = 0;
 #define MLL_DECODE_CASE(TILES)                                                                                        \
     case TILES:                                                                                                       \
-        status = launch_decode<TILES>(q, k_cache, v_cache, block_table, table_width, seq_of_token, positions, out,    \
-                                      part_o, part_ml, scale, window, n_tokens, heads, kv_heads, page_size, n_splits, \
-                                      stream);                                                                        \
+        status = launch_decode<TILES>(q, k_cache, v_cache, block_table, table_width, seq_of_token, positions,         \
+                                      token_ids, out, part_o, part_ml, scale, window, n_tokens, heads, kv_heads,      \
+                                      page_size, n_splits, stream);                                                   \
         break;
     switch (head_dim / 16) {
         MLL_DECODE_CASE(1) MLL_DECODE_CASE(2) MLL_DECODE_CASE(3) MLL_DECODE_CASE(4) MLL_DECODE_CASE(5)
@@ -309,8 +314,8 @@ extern "C" int mll_paged_attention_decode(const void* q, const void* k_cache, co
     if (status != 0) return status;
     if (n_splits > 1) {
         const int threads = head_dim <= 64 ? 64 : (head_dim <= 128 ? 128 : 256);
-        paged_attention_join_kernel<<<n_tokens * heads, threads, 0, stream>>>(part_o, part_ml, static_cast<bf16*>(out),
-                                                                             head_dim, n_splits);
+        paged_attention_join_kernel<<<n_tokens * heads, threads, 0, stream>>>(part_o, part_ml, token_ids,
+                                                                             static_cast<bf16*>(out), heads, head_dim, n_splits);
         return check_launch("paged_attention_join");
     }
     return 0;

@@ -69,11 +69,12 @@ int mll_paged_attention_prefill_tile();
 // for steps whose requests bring one token each, right for any. head_dim a multiple of 16 up to 256,
 // page_size a multiple of 16. n_splits > 1 needs part_o [tokens, heads, n_splits, head_dim] and
 // part_ml [tokens, heads, n_splits, 2] (float32 device scratch, contents need not be cleared).
+// token_ids (nullable) lists the n_tokens rows of q / out to work on; without it all rows 0 .. n_tokens-1.
 int mll_paged_attention_decode(const void* q, const void* k_cache, const void* v_cache,
                                const int32_t* block_table, int table_width, const int32_t* seq_of_token,
-                               const int32_t* positions, void* out, float* part_o, float* part_ml,
-                               float scale, int window, int n_tokens, int heads, int kv_heads, int head_dim,
-                               int page_size, int n_splits, hipStream_t stream);
+                               const int32_t* positions, const int32_t* token_ids, void* out, float* part_o,
+                               float* part_ml, float scale, int window, int n_tokens, int heads, int kv_heads,
+                               int head_dim, int page_size, int n_splits, hipStream_t stream);
 
 // out[t, c] = silu(gate[t, c]) * up[t, c]; gate and up rows are `in_stride` elements apart.
 int mll_silu_mul(const void* gate, const void* up, int64_t in_stride, void* out, int dtype,

@@ -48,7 +48,9 @@ class StepContext:
     seq_total: torch.Tensor     # int32 [requests]: positions in the cache once this step is done
     slots: torch.Tensor         # int32 [requests]: state slot of every request
     want_rows: Optional[torch.Tensor]  # int32 [wanted]: rows of the flat list whose logits are wanted
-    query_tiles: torch.Tensor   # int32 [tiles, 3]: (request, first token in the flat list, tokens) per tile of <= 128 tokens
+    query_tiles: torch.Tensor   # int32 [tiles, 3]: (request, first token in the flat list, tokens) per tile of <= 128
+                                # tokens, for the requests that bring more than one token (all, if none brings just one)
+    single_tokens: Optional[torch.Tensor]  # int32: rows of the requests that bring one token, when others bring more
     paged: List[PagedView]
     # the same on the host, for parts written in Python and for choosing kernels
     starts: List[int] = field(default_factory=list)
@@ -57,6 +59,7 @@ class StepContext:
     max_count: int = 0
     max_total: int = 0
     planned_total: int = 0      # the longest request this step's launch shapes are planned for (>= max_total)
+    max_single_total: int = 0   # the longest of the requests listed in single_tokens
 
 
 class BatchBuilder:
@@ -117,12 +120,16 @@ class BatchBuilder:
             widths.append(width)
         slots = np.asarray([request.slot for request in requests], dtype=np.int32)
         # Tiles with the most keys to walk come first, so that the longest workgroups start first.
+        mixed = any(count == 1 for count in counts) and any(count > 1 for count in counts)
         tile_list = sorted(((index, cu[index] + offset, min(QUERY_TILE, count - offset))
-                            for index, count in enumerate(counts) for offset in range(0, count, QUERY_TILE)),
+                            for index, count in enumerate(counts) if not (mixed and count == 1)
+                            for offset in range(0, count, QUERY_TILE)),
                            key=lambda tile: -(starts[tile[0]] + tile[1] - cu[tile[0]] + tile[2]))
         query_tiles = np.asarray(tile_list, dtype=np.int32).reshape(-1, 3)
+        single_tokens = np.asarray([cu[index] for index, count in enumerate(counts) if mixed and count == 1], dtype=np.int32)
+        max_single_total = max((totals[index] for index, count in enumerate(counts) if mixed and count == 1), default=0)
         pieces = [tokens, positions, seq_of_token, cu, np.asarray(starts, np.int32), np.asarray(totals, np.int32),
-                  slots, want_rows, query_tiles.reshape(-1)]
+                  slots, want_rows, query_tiles.reshape(-1), single_tokens]
         for table, mapping in zip(tables, mappings):
             pieces += [table.reshape(-1), mapping]
         offsets, cursor = [], 0
@@ -143,13 +150,14 @@ class BatchBuilder:
 
         paged = []
         for g, group in enumerate(self.cache.groups):
-            paged.append(PagedView(piece_at(9 + 2 * g, (n_seqs, widths[g])), piece_at(10 + 2 * g),
+            paged.append(PagedView(piece_at(10 + 2 * g, (n_seqs, widths[g])), piece_at(11 + 2 * g),
                                    page_size, widths[g]))
         longest = max(totals) if totals else 0
         return StepContext(
             n_tokens=n_tokens, n_seqs=n_seqs, tokens=piece_at(0), positions=piece_at(1), seq_of_token=piece_at(2),
             cu_tokens=piece_at(3), seq_start=piece_at(4), seq_total=piece_at(5), slots=piece_at(6),
-            want_rows=piece_at(7) if want_rows.size else None, query_tiles=piece_at(8, (-1, 3)), paged=paged,
+            want_rows=piece_at(7) if want_rows.size else None, query_tiles=piece_at(8, (-1, 3)),
+            single_tokens=piece_at(9) if single_tokens.size else None, max_single_total=max_single_total, paged=paged,
             starts=list(starts), counts=counts, host_slots=[request.slot for request in requests],
             max_count=max(counts) if counts else 0, max_total=longest,
             planned_total=longest if fixed_width is None else fixed_width * page_size)

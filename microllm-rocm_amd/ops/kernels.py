@@ -294,28 +294,37 @@ def decode_splits(n_tokens: int, kv_heads: int, longest: int) -> int:
 def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                            seq_of_token: torch.Tensor, positions: torch.Tensor, scale: float, window: int,
                            heads: int, kv_heads: int, head_dim: int, n_splits: int,
-                           out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The MFMA kernel for bfloat16 queries that each attend alone (one token per request)."""
+                           out: Optional[torch.Tensor] = None, token_ids: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The MFMA kernel for bfloat16 queries that each attend alone (one token per request).
+
+    ``token_ids`` restricts the work to those rows of ``q`` (the other rows of ``out`` are left alone)."""
     lib = library.load()
     page_size = _check_paged(q, k_cache, v_cache, block_table, heads, kv_heads, head_dim)
     _need(q.dtype == torch.bfloat16, "the decode kernel takes bfloat16")
     _need(head_dim % 16 == 0 and 16 <= head_dim <= 256, "the decode kernel takes head sizes in steps of 16 up to 256")
     _need(page_size % 16 == 0, "the decode kernel takes page sizes in steps of 16")
-    n_tokens = q.shape[0]
+    n_rows = q.shape[0]
     _device_tensor(seq_of_token, "request of token", torch.int32)
     _device_tensor(positions, "positions", torch.int32)
-    _need(seq_of_token.shape[0] == n_tokens and positions.shape[0] == n_tokens,
+    _need(seq_of_token.shape[0] == n_rows and positions.shape[0] == n_rows,
           "request-of-token and positions must hold one entry per token")
+    n_tokens = n_rows
+    if token_ids is not None:
+        _device_tensor(token_ids, "token ids", torch.int32)
+        _need(token_ids.dim() == 1 and token_ids.shape[0] <= n_rows, "token ids must list rows of q")
+        n_tokens = token_ids.shape[0]
     if out is None:
         out = torch.empty_like(q)
+    _device_tensor(out, "attention output", q.dtype)
+    _need(out.shape == q.shape, "attention output must have the queries' shape")
     part_o = part_ml = None
     if n_splits > 1:
         part_o = torch.empty((n_tokens, heads, n_splits, head_dim), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((n_tokens, heads, n_splits, 2), dtype=torch.float32, device=q.device)
     _check(lib.mll_paged_attention_decode(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
-                                          _ptr(seq_of_token), _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml),
-                                          ctypes.c_float(scale), int(window), n_tokens, heads, kv_heads, head_dim,
-                                          page_size, n_splits, _stream()), lib)
+                                          _ptr(seq_of_token), _ptr(positions), _ptr(token_ids), _ptr(out), _ptr(part_o),
+                                          _ptr(part_ml), ctypes.c_float(scale), int(window), n_tokens, heads, kv_heads,
+                                          head_dim, page_size, n_splits, _stream()), lib)
     return out
 
 
@@ -333,6 +342,8 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     _need(positions.shape[0] == q.shape[0], "positions must hold one entry per token")
     if out is None:
         out = torch.empty_like(q)
+    _device_tensor(out, "attention output", q.dtype)
+    _need(out.shape == q.shape, "attention output must have the queries' shape")
     _check(lib.mll_paged_attention_prefill(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
                                            _ptr(query_tiles), query_tiles.shape[0], _ptr(positions), _ptr(out),
                                            ctypes.c_float(scale), int(window), heads, kv_heads, head_dim, page_size,
@@ -355,8 +366,17 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         return paged_attention_decode(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
                                       scale, window, heads, kv_heads, head_dim, splits)
     if mfma_fits:
-        return paged_attention_prefill(q, k_cache, v_cache, view.block_table, ctx.query_tiles, ctx.positions,
-                                       scale, window, heads, kv_heads, head_dim)
+        # Portions go to the tiled kernel; requests that bring one token, if any, to the split kernel.
+        out = torch.empty_like(q)
+        if ctx.query_tiles.shape[0] > 0:
+            paged_attention_prefill(q, k_cache, v_cache, view.block_table, ctx.query_tiles, ctx.positions,
+                                    scale, window, heads, kv_heads, head_dim, out=out)
+        if ctx.single_tokens is not None:
+            visible = min(ctx.max_single_total, window) if window > 0 else ctx.max_single_total
+            splits = decode_splits(ctx.single_tokens.shape[0], kv_heads, visible)
+            paged_attention_decode(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
+                                   scale, window, heads, kv_heads, head_dim, splits, out=out, token_ids=ctx.single_tokens)
+        return out
     return paged_attention_rowwise(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
                                    scale, window, heads, kv_heads, head_dim)
 

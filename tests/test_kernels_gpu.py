@@ -238,6 +238,12 @@ def test_decode_attention(heads, kv_heads, hd, page_size, window, splits):
                                            heads, kv_heads, hd, splits)
     reference = reference_attention(q_exact, ek, ev, seq, pos, heads, kv_heads, hd, scale, window)
     np.testing.assert_allclose(out.float().cpu().numpy(), reference, **tolerance(torch.bfloat16))
+    # some rows only: the others are left as they were
+    some = torch.tensor([5, 0, 3], dtype=torch.int32, device=DEVICE)
+    partial = torch.full_like(out, 7.0)
+    kernels().paged_attention_decode(t["q"], t["k"], t["v"], t["table"], t["seq"], t["pos"], scale, window,
+                                     heads, kv_heads, hd, splits, out=partial, token_ids=some)
+    assert torch.equal(partial[[5, 0, 3]], out[[5, 0, 3]]) and bool((partial[[1, 2, 4, 6]] == 7.0).all())
 
 
 @pytest.mark.parametrize("heads,kv_heads,hd,page_size,window", [
