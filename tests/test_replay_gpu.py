@@ -155,3 +155,42 @@ def test_the_program_itself(tmp_path_factory, tmp_path, dtype):
     assert result.returncode == 0, result.stderr
     assert result.stdout.split() == [word for step in steps for word in ("done", str(step["step"]))]
     compare(collect(steps, out_dir, config.vocab_size), requests, plain_model, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page_size", [32, 64])
+def test_larger_pages(tmp_path_factory, tmp_path, dtype, page_size):
+    """Pages of 32 and 64 positions hold two and four 16-position tiles; the window's edge falls inside a page."""
+    from microllm_rocm_amd.engine import Engine
+    from microllm_rocm_amd.engine.replay import replay
+    config = CONFIGS["C"]
+    folder, plain_model = model_for(tmp_path_factory, "C", SHARP)
+    requests = requests_for(config, [150, 70, 129, 64, 200], seed=60)
+    steps, peak = mixed(requests, seed=9)
+    engine = Engine.from_folder(folder, dtype=dtype, page_size=page_size, max_tokens=round_up(peak, page_size) + 2 * page_size,
+                                max_requests=8)
+    replay(engine, io.StringIO(to_lines(steps)), str(tmp_path / "out"), io.StringIO())
+    engine.cache.check()
+    compare(collect(steps, tmp_path / "out", config.vocab_size), requests, plain_model, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_weights_stored_in_32_bit_stay_32_bit(tmp_path, dtype):
+    """A file of float32 tensors whose values bfloat16 cannot hold: they are not rounded, in either engine."""
+    import torch
+    from microllm_rocm_amd.engine import Engine
+    from microllm_rocm_amd.weights import write_model_folder
+    config = CONFIGS["B"]
+    folder = write_model_folder(str(tmp_path / "f32"), config, seed=11, dtype=torch.float32, stds=SHARP)
+    plain_model = PlainModel(folder)
+    assert np.abs(plain_model.weights["lm_head.weight"] - plain_model.weights["lm_head.weight"].astype(np.float32)
+                  .view(np.uint32).__and__(0xFFFF0000).view(np.float32)).max() > 0    # not bfloat16 values
+    requests = requests_for(config, [90, 40], seed=70)
+    steps = portions("r0", requests["r0"], [40, 2, 17, 1, 1, 1]) + [dict(step, step=step["step"] + 100) for step in whole({"r1": requests["r1"]})]
+    engine = run_trace(folder, dtype, steps, tmp_path / "out", max_tokens=192)
+    assert engine.model.head.weight.tensor.dtype == torch.float32
+    assert engine.model.blocks[0].mixer.qkv_weight.tensor.dtype == torch.float32
+    got = collect(steps, tmp_path / "out", config.vocab_size)
+    worst_max, _ = compare(got, requests, plain_model, dtype)
+    if dtype == "bfloat16":
+        assert worst_max > 1e-4      # activations are still bfloat16: this is not the 32-bit engine in disguise
