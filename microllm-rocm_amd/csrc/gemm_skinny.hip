@@ -30,7 +30,9 @@ __device__ inline float silu_f(float value) {
 // EPILOGUE: 0 = float32 [M, N]; 1 = bfloat16 [M, N]; 2 = bfloat16 [M, N / 2] = silu(even rows of W) * (odd rows).
 // A_PACKED: the activations come in the same piece order as the weight ([M/16][K/32][4][16][8], zero padded),
 // so a wave's load of a piece of A is one contiguous KB too; otherwise A is row-major [M, K].
-template <int MT, int NT, int EPILOGUE, bool A_PACKED>
+// TEMPORAL: W is read with ordinary loads instead of non-temporal ones (measured on MI355X: better for weights
+// of a few tens of MB, worse for the large ones).
+template <int MT, int NT, int EPILOGUE, bool A_PACKED, bool TEMPORAL>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w_packed, void* __restrict__ out,
     int m, int n, int k, int n_tiles, int k_steps) {
@@ -78,8 +80,10 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
             for (int nt = 0; nt < NT; ++nt) {
                 w_piece[u][nt].raw = uintx4{0u, 0u, 0u, 0u};
                 if (live && w_live[nt])
-                    w_piece[u][nt].raw = __builtin_nontemporal_load(
-                        reinterpret_cast<const uintx4*>(w_ptr[nt] + static_cast<int64_t>(ks) * 512));
+                    w_piece[u][nt].raw =
+                        TEMPORAL ? *reinterpret_cast<const uintx4*>(w_ptr[nt] + static_cast<int64_t>(ks) * 512)
+                                 : __builtin_nontemporal_load(
+                                       reinterpret_cast<const uintx4*>(w_ptr[nt] + static_cast<int64_t>(ks) * 512));
             }
             const int k_offset = ks * 32;
             const bool in_k = live && k_offset + quad * 8 < k;
@@ -166,10 +170,15 @@ static void launch_one(const bf16* a, int a_packed, const bf16* w, void* out, in
     int waves = 1;
     while (waves < 16 && groups * waves * 2 <= 8192 && waves * 2 * DEPTH <= k_steps) waves *= 2;
     const size_t lds = waves > 1 ? static_cast<size_t>(waves - 1) * NT * MT * kWave * sizeof(floatx4) : 0;
-    if (a_packed)
-        gemm_skinny_kernel<MT, NT, EPILOGUE, true><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps);
+    const bool temporal = static_cast<int64_t>(n_tiles) * k_steps * 1024 < (64ll << 20);   // bytes of the packed weight
+    if (a_packed && temporal)
+        gemm_skinny_kernel<MT, NT, EPILOGUE, true, true><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps);
+    else if (a_packed)
+        gemm_skinny_kernel<MT, NT, EPILOGUE, true, false><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps);
+    else if (temporal)
+        gemm_skinny_kernel<MT, NT, EPILOGUE, false, true><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps);
     else
-        gemm_skinny_kernel<MT, NT, EPILOGUE, false><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps);
+        gemm_skinny_kernel<MT, NT, EPILOGUE, false, false><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps);
 }
 
 template <int EPILOGUE>
@@ -180,11 +189,15 @@ static int launch_skinny(const void* a, int a_packed, const void* w_packed, void
     const bf16* a_ = static_cast<const bf16*>(a);
     const bf16* w_ = static_cast<const bf16*>(w_packed);
     const int m_tiles = (m + 15) / 16;
-    // Few tiles of W: one per workgroup, so that the GPU is filled. Many rows of A: two, so that every piece of
-    // A is used twice (four tiles a workgroup measured slower on MI355X).
+    // Few tiles of W: one per workgroup, so that the GPU is filled. Many tiles of W, or several rows of A and at
+    // least 128 workgroups left: two, so that every piece of A is used twice (all measured on MI355X; four tiles
+    // a workgroup were slower).
     const bool wide = n_tiles >= 2048;
     switch (m_tiles) {
-        case 1: launch_one<1, 1, EPILOGUE>(a_, a_packed, w_, out, m, n, k, n_tiles, k_steps, stream); break;
+        case 1:
+            if (wide || (m > 4 && n_tiles >= 256)) launch_one<1, 2, EPILOGUE>(a_, a_packed, w_, out, m, n, k, n_tiles, k_steps, stream);
+            else launch_one<1, 1, EPILOGUE>(a_, a_packed, w_, out, m, n, k, n_tiles, k_steps, stream);
+            break;
         case 2:
             if (wide) launch_one<2, 2, EPILOGUE>(a_, a_packed, w_, out, m, n, k, n_tiles, k_steps, stream);
             else launch_one<2, 1, EPILOGUE>(a_, a_packed, w_, out, m, n, k, n_tiles, k_steps, stream);

@@ -461,3 +461,29 @@ def test_consumers_add_partial_sums_in_order():
     q_sum = k.qkv_rope_store(torch.from_numpy(qkv_parts.sum(axis=0)).to(DEVICE), None, positions, None, None, None, None,
                              heads, kv_heads, hd, 16, torch.float32)
     np.testing.assert_allclose(q_parts.cpu().numpy(), q_sum.cpu().numpy(), rtol=1e-6, atol=1e-6)
+
+
+# ---- long contexts ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("window", [0, 5000])
+def test_attention_kernels_at_twenty_thousand_keys(window):
+    """Block tables hundreds of pages wide, positions beyond 2^14, many splits: all three kernels agree with the plain rule."""
+    heads, kv_heads, hd, page_size = 4, 2, 64, 16
+    rng = np.random.default_rng(99)
+    lengths, counts = [20011, 777, 12000], [150, 1, 40]
+    t, q_exact, ek, ev, seq, pos = build_paged_case(rng, torch.bfloat16, lengths, counts, heads, kv_heads, hd, page_size)
+    scale = 1.0 / math.sqrt(hd)
+    reference = reference_attention(q_exact, ek, ev, seq, pos, heads, kv_heads, hd, scale, window)
+    k = kernels()
+    tiles, start = [], 0
+    for index, count in enumerate(counts):
+        tiles += [(index, start + offset, min(128, count - offset)) for offset in range(0, count, 128)]
+        start += count
+    prefill = k.paged_attention_prefill(t["q"], t["k"], t["v"], t["table"], torch.tensor(tiles, dtype=torch.int32, device=DEVICE),
+                                        t["pos"], scale, window, heads, kv_heads, hd)
+    np.testing.assert_allclose(prefill.float().cpu().numpy(), reference, **tolerance(torch.bfloat16))
+    for splits in (1, 16, 200):
+        decode = k.paged_attention_decode(t["q"], t["k"], t["v"], t["table"], t["seq"], t["pos"], scale, window,
+                                          heads, kv_heads, hd, splits)
+        np.testing.assert_allclose(decode.float().cpu().numpy(), reference, **tolerance(torch.bfloat16))
+    rowwise = k.paged_attention_rowwise(t["q"], t["k"], t["v"], t["table"], t["seq"], t["pos"], scale, window, heads, kv_heads, hd)
+    np.testing.assert_allclose(rowwise.float().cpu().numpy(), reference, **tolerance(torch.bfloat16))
