@@ -16,6 +16,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..parts.base import CacheNeed, PagedKVNeed, StateNeed
@@ -54,12 +55,16 @@ class RequestCache:
 
 
 class CacheGroup:
-    def __init__(self, index: int, need: PagedKVNeed, num_pages: int, page_size: int):
+    def __init__(self, index: int, need: PagedKVNeed, num_pages: int, page_size: int, max_requests: int,
+                 max_blocks: int):
         self.index = index
         self.need = need
         self.page_size = page_size
         self.pool = PagePool(num_pages)
         self.entries: List[int] = []
+        # The block tables of all live requests, one row per state slot, kept up to date as pages come and go:
+        # a step gathers its rows from here instead of rebuilding them from lists.
+        self.tables = np.full((max_requests, max_blocks), RELEASED, dtype=np.int32)
 
     def first_needed_block(self, num_tokens: int) -> int:
         """Blocks below this index hold no key that a query at ``num_tokens`` or later can see."""
@@ -72,7 +77,7 @@ class CacheGroup:
 class CacheManager:
     def __init__(self, needs: Sequence[CacheNeed], reads: Sequence[Optional[int]], page_size: int,
                  num_pages: int, max_requests: int, dtype: torch.dtype = torch.float32,
-                 device: Optional[torch.device] = None):
+                 device: Optional[torch.device] = None, max_blocks: Optional[int] = None):
         if page_size <= 0:
             raise ValueError("page_size must be positive")
         if device is not None:
@@ -81,6 +86,7 @@ class CacheManager:
             raise ValueError("one need and one read source per run entry")
         self.page_size = page_size
         self.max_requests = max_requests
+        self.max_blocks = min(num_pages, max_blocks) if max_blocks else num_pages   # most blocks one request can hold
         self.dtype = dtype
         self.device = device
         self.groups: List[CacheGroup] = []
@@ -95,7 +101,7 @@ class CacheManager:
             if isinstance(need, PagedKVNeed):
                 group = by_need.get(need)
                 if group is None:
-                    group = CacheGroup(len(self.groups), need, num_pages, page_size)
+                    group = CacheGroup(len(self.groups), need, num_pages, page_size, max_requests, self.max_blocks)
                     self.groups.append(group)
                     by_need[need] = group
                 group.entries.append(entry)
@@ -169,7 +175,13 @@ class CacheManager:
                 raise OutOfPages(f"request {request.request_id!r} needs {need} pages in group {group.index}, "
                                  f"{group.pool.num_free} free of {group.pool.num_pages}")
         for need, group in zip(needed, self.groups):
-            request.pages[group.index].extend(group.pool.take(need))
+            if need:
+                pages = request.pages[group.index]
+                if len(pages) + need > self.max_blocks:
+                    raise OutOfPages(f"request {request.request_id!r} would hold more than {self.max_blocks} blocks")
+                taken = group.pool.take(need)
+                group.tables[request.slot, len(pages):len(pages) + need] = taken
+                pages.extend(taken)
         request.reserved += count
 
     def cancel_reservation(self, request: RequestCache) -> None:
@@ -179,6 +191,7 @@ class CacheManager:
             pages = request.pages[group.index]
             extra = [page for page in pages[keep:] if page != RELEASED]
             group.pool.give(extra)
+            group.tables[request.slot, keep:len(pages)] = RELEASED
             del pages[keep:]
         request.reserved = 0
 
@@ -189,6 +202,8 @@ class CacheManager:
         request.num_tokens += count
         request.reserved -= count
         for group in self.groups:
+            if group.need.window is None:
+                continue
             first = group.first_needed_block(request.num_tokens)
             pages = request.pages[group.index]
             passed = [index for index in range(min(first, len(pages))) if pages[index] != RELEASED]
@@ -196,6 +211,7 @@ class CacheManager:
                 group.pool.give(pages[index] for index in passed)
                 for index in passed:
                     pages[index] = RELEASED
+                    group.tables[request.slot, index] = RELEASED
 
     def close(self, request_id: Hashable) -> None:
         request = self.requests.pop(request_id, None)
@@ -203,6 +219,7 @@ class CacheManager:
             raise KeyError(f"request {request_id!r} is not open")
         for group in self.groups:
             group.pool.give(page for page in request.pages[group.index] if page != RELEASED)
+            group.tables[request.slot, :len(request.pages[group.index])] = RELEASED
             request.pages[group.index] = []
         self.slots.give([request.slot])
         request.closed = True
@@ -243,6 +260,12 @@ class CacheManager:
                 raise AssertionError(f"group {group.index}: a held page is on the free list")
             if len(free) + len(seen) != group.pool.num_pages:
                 raise AssertionError(f"group {group.index}: {group.pool.num_pages - len(free) - len(seen)} pages lost")
+            live_slots = {request.slot: request for request in self.requests.values()}
+            for slot in range(self.max_requests):
+                row = group.tables[slot]
+                pages = live_slots[slot].pages[group.index] if slot in live_slots else []
+                if list(row[:len(pages)]) != list(pages) or not np.all(row[len(pages):] == RELEASED):
+                    raise AssertionError(f"group {group.index}: the table row of slot {slot} differs from its request's pages")
         slots = [request.slot for request in self.requests.values()]
         if len(set(slots)) != len(slots):
             raise AssertionError("two requests share a state slot")

@@ -7,7 +7,7 @@
 // The product is computed transposed (C^T = W . A^T): the activations are the B operand, 16 rows per tile.
 // A workgroup owns NT tiles of W; its waves (1 to 16, more when W has few rows, so that the GPU is filled)
 // take the k steps in turn and their sums are added in wave order through LDS: the result is the same in
-// every run and, for up to 16 rows, does not depend on the other rows of A.
+// every run and does not depend on the other rows of A.
 #include "common.h"
 #include "microllm_hip.h"
 
@@ -17,6 +17,8 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 
+
+constexpr int kChunk = 8;   // k steps a wave takes in a row
 
 union Piece {
     bf16x8 v;
@@ -66,45 +68,49 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
                              : a + static_cast<int64_t>(a_live[mt] ? row : 0) * k + quad * 8;
     }
 
-    // A wave takes DEPTH consecutive k steps at a time, then skips what the other waves take. All loads of
-    // the DEPTH steps are issued before the first product, so that a wave keeps several KB of W in flight.
+    // A wave takes kChunk consecutive k steps at a time, then skips what the other waves take; which k steps a
+    // wave sums, and in which order, depends on (n, k) alone, not on the number of rows or tiles. The loads of
+    // DEPTH steps are issued before their products, so that a wave keeps several KB of W in flight.
     constexpr int DEPTH = (MT + NT <= 2) ? 8 : ((MT + NT <= 4) ? 4 : 2);
-    for (int base = wave * DEPTH; base < k_steps; base += waves * DEPTH) {
-        Piece w_piece[DEPTH][NT];
-        Piece a_piece[DEPTH][MT];
+    for (int chunk = wave * kChunk; chunk < k_steps; chunk += waves * kChunk) {
 #pragma unroll
-        for (int u = 0; u < DEPTH; ++u) {
-            const bool live = base + u < k_steps;
-            const int ks = base + u;
+        for (int base = chunk; base < chunk + kChunk; base += DEPTH) {
+            Piece w_piece[DEPTH][NT];
+            Piece a_piece[DEPTH][MT];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                w_piece[u][nt].raw = uintx4{0u, 0u, 0u, 0u};
-                if (live && w_live[nt])
-                    w_piece[u][nt].raw =
-                        TEMPORAL ? *reinterpret_cast<const uintx4*>(w_ptr[nt] + static_cast<int64_t>(ks) * 512)
-                                 : __builtin_nontemporal_load(
-                                       reinterpret_cast<const uintx4*>(w_ptr[nt] + static_cast<int64_t>(ks) * 512));
-            }
-            const int k_offset = ks * 32;
-            const bool in_k = live && k_offset + quad * 8 < k;
+            for (int u = 0; u < DEPTH; ++u) {
+                const int ks = base + u;
+                const bool live = ks < k_steps;
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                a_piece[u][mt].raw = uintx4{0u, 0u, 0u, 0u};
-                if (A_PACKED) {
-                    if (a_live[mt] && live)
-                        a_piece[u][mt].raw = *reinterpret_cast<const uintx4*>(a_ptr[mt] + static_cast<int64_t>(ks) * 512);
-                } else if (a_live[mt] && in_k) {
-                    a_piece[u][mt].raw = *reinterpret_cast<const uintx4*>(a_ptr[mt] + k_offset);
+                for (int nt = 0; nt < NT; ++nt) {
+                    w_piece[u][nt].raw = uintx4{0u, 0u, 0u, 0u};
+                    if (live && w_live[nt])
+                        w_piece[u][nt].raw =
+                            TEMPORAL ? *reinterpret_cast<const uintx4*>(w_ptr[nt] + static_cast<int64_t>(ks) * 512)
+                                     : __builtin_nontemporal_load(
+                                           reinterpret_cast<const uintx4*>(w_ptr[nt] + static_cast<int64_t>(ks) * 512));
+                }
+                const int k_offset = ks * 32;
+                const bool in_k = live && k_offset + quad * 8 < k;
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    a_piece[u][mt].raw = uintx4{0u, 0u, 0u, 0u};
+                    if (A_PACKED) {
+                        if (a_live[mt] && live)
+                            a_piece[u][mt].raw = *reinterpret_cast<const uintx4*>(a_ptr[mt] + static_cast<int64_t>(ks) * 512);
+                    } else if (a_live[mt] && in_k) {
+                        a_piece[u][mt].raw = *reinterpret_cast<const uintx4*>(a_ptr[mt] + k_offset);
+                    }
                 }
             }
+#pragma unroll
+            for (int u = 0; u < DEPTH; ++u)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_piece[u][nt].v, a_piece[u][mt].v, acc[nt][mt], 0, 0, 0);
         }
-#pragma unroll
-        for (int u = 0; u < DEPTH; ++u)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_piece[u][nt].v, a_piece[u][mt].v, acc[nt][mt], 0, 0, 0);
     }
 
     // The waves' sums, added in wave order by wave 0.
@@ -164,11 +170,10 @@ template <int MT, int NT, int EPILOGUE>
 static void launch_one(const bf16* a, int a_packed, const bf16* w, void* out, int m, int n, int k, int n_tiles,
                        int k_steps, hipStream_t stream) {
     const int groups = (n_tiles + NT - 1) / NT;
-    // Waves per workgroup: enough that about eight thousand waves stream W, at most 16, and no more than
-    // there are pieces of k for them.
-    constexpr int DEPTH = (MT + NT <= 2) ? 8 : ((MT + NT <= 4) ? 4 : 2);
+    // Waves per workgroup: enough that about eight thousand waves would stream W one tile each, at most 16, and
+    // no more than there are chunks of k for them. A function of (n, k) alone, like the split of k it implies.
     int waves = 1;
-    while (waves < 16 && groups * waves * 2 <= 8192 && waves * 2 * DEPTH <= k_steps) waves *= 2;
+    while (waves < 16 && n_tiles * waves * 2 <= 8192 && waves * 2 * kChunk <= k_steps) waves *= 2;
     const size_t lds = waves > 1 ? static_cast<size_t>(waves - 1) * NT * MT * kWave * sizeof(floatx4) : 0;
     const bool temporal = static_cast<int64_t>(n_tiles) * k_steps * 1024 < (64ll << 20);   // bytes of the packed weight
     if (a_packed && temporal)

@@ -88,8 +88,8 @@ int mll_gemm_f32(const float* a, const float* w, const float* bias, float* c,
 // C = A . W^T for bfloat16 A [m <= 64, k] and a weight packed as [n/16][k/32][4][16][8] (zero padded):
 // element (row, col) of W sits at piece (row / 16, col / 32), position ((col % 32) / 8, row % 16, col % 8).
 // epilogue 0: float32 [m, n]; 1: bfloat16 [m, n]; 2: bfloat16 [m, n / 2] = silu(even weight rows' results) *
-// (odd rows' results). The order of additions is fixed by (n, k) and the number of 16-row tiles of A: the
-// same in every run, and for up to 16 rows independent of the other rows. With a_packed the activations
+// (odd rows' results). The order of additions is fixed by (n, k): the same in every run and whatever the
+// other rows of A. With a_packed the activations
 // come in the weight's piece order too ([m/16][k/32][4][16][8], zero padded) instead of row-major [m, k].
 int mll_gemm_skinny(const void* a, int a_packed, const void* w_packed, void* out, int epilogue, int m, int n,
                     int k, hipStream_t stream);

@@ -90,46 +90,67 @@ class BatchBuilder:
     def build(self, requests: Sequence[RequestCache], token_lists: Sequence[Sequence[int]],
               wants: Sequence[Sequence[int]], fixed_width: Optional[int] = None) -> StepContext:
         page_size = self.cache.page_size
-        counts = [len(tokens) for tokens in token_lists]
-        starts = [request.num_tokens for request in requests]
         n_seqs = len(requests)
+        counts = [len(tokens) for tokens in token_lists]
         n_tokens = sum(counts)
-        totals = [start + count for start, count in zip(starts, counts)]
+        slots = np.fromiter((request.slot for request in requests), dtype=np.int32, count=n_seqs)
+        starts_array = np.fromiter((request.num_tokens for request in requests), dtype=np.int32, count=n_seqs)
+        starts = starts_array.tolist()
+        if n_tokens == n_seqs:      # every request brings one token: nothing to concatenate
+            counts_array = np.ones(n_seqs, dtype=np.int32)
+            tokens = np.fromiter((tokens[0] for tokens in token_lists), dtype=np.int32, count=n_seqs)
+            positions = starts_array
+            seq_of_token = np.arange(n_seqs, dtype=np.int32)
+        else:
+            counts_array = np.asarray(counts, dtype=np.int32)
+            tokens = np.concatenate([np.asarray(t, dtype=np.int32) for t in token_lists]) if n_tokens else np.zeros(0, np.int32)
+            positions = np.concatenate([np.arange(s, s + c, dtype=np.int32) for s, c in zip(starts, counts)]) \
+                if n_tokens else np.zeros(0, np.int32)
+            seq_of_token = np.repeat(np.arange(n_seqs, dtype=np.int32), counts)
+        totals_array = starts_array + counts_array
+        totals = totals_array.tolist()
         cu = np.zeros(n_seqs + 1, dtype=np.int32)
-        np.cumsum(counts, out=cu[1:])
-        tokens = np.concatenate([np.asarray(t, dtype=np.int32) for t in token_lists]) if n_tokens else np.zeros(0, np.int32)
-        positions = np.concatenate([np.arange(s, s + c, dtype=np.int32) for s, c in zip(starts, counts)]) \
-            if n_tokens else np.zeros(0, np.int32)
-        seq_of_token = np.repeat(np.arange(n_seqs, dtype=np.int32), counts)
-        want_rows = np.asarray([cu[index] + place for index, want in enumerate(wants) for place in want],
-                               dtype=np.int32)
+        np.cumsum(counts_array, out=cu[1:])
+        if all(len(want) == 1 and want[0] == 0 for want in wants) and n_tokens == n_seqs:
+            want_rows = np.arange(n_seqs, dtype=np.int32)
+        else:
+            want_rows = np.asarray([cu[index] + place for index, want in enumerate(wants) for place in want],
+                                   dtype=np.int32)
         tables, mappings, widths = [], [], []
+        blocks_needed = int((int(totals_array.max()) + page_size - 1) // page_size) if n_seqs else 1
         for group in self.cache.groups:
-            width = max(1, max(len(request.pages[group.index]) for request in requests))
+            width = max(1, blocks_needed)
             if fixed_width is not None:
                 if width > fixed_width:
                     raise ValueError("a block table is wider than the fixed width")
                 width = fixed_width
-            table = np.full((n_seqs, width), RELEASED, dtype=np.int32)
-            for row, request in enumerate(requests):
-                pages = request.pages[group.index]
-                table[row, :len(pages)] = pages
+            rows = group.tables[slots]                      # [requests, most blocks a request can hold]
+            if width <= rows.shape[1]:
+                table = np.ascontiguousarray(rows[:, :width])
+            else:
+                table = np.full((n_seqs, width), RELEASED, dtype=np.int32)
+                table[:, :rows.shape[1]] = rows
             mapping = table[seq_of_token, positions // page_size] * page_size + positions % page_size
             tables.append(table)
-            mappings.append(mapping.astype(np.int32))
+            mappings.append(mapping.astype(np.int32, copy=False))
             widths.append(width)
-        slots = np.asarray([request.slot for request in requests], dtype=np.int32)
-        # Tiles with the most keys to walk come first, so that the longest workgroups start first.
-        mixed = any(count == 1 for count in counts) and any(count > 1 for count in counts)
-        tile_list = sorted(((index, cu[index] + offset, min(QUERY_TILE, count - offset))
-                            for index, count in enumerate(counts) if not (mixed and count == 1)
-                            for offset in range(0, count, QUERY_TILE)),
-                           key=lambda tile: -(starts[tile[0]] + tile[1] - cu[tile[0]] + tile[2]))
-        query_tiles = np.asarray(tile_list, dtype=np.int32).reshape(-1, 3)
-        single_tokens = np.asarray([cu[index] for index, count in enumerate(counts) if mixed and count == 1], dtype=np.int32)
-        max_single_total = max((totals[index] for index, count in enumerate(counts) if mixed and count == 1), default=0)
-        pieces = [tokens, positions, seq_of_token, cu, np.asarray(starts, np.int32), np.asarray(totals, np.int32),
-                  slots, want_rows, query_tiles.reshape(-1), single_tokens]
+        if n_tokens == n_seqs:
+            index = np.arange(n_seqs, dtype=np.int32)
+            query_tiles = np.stack([index, index, np.ones(n_seqs, dtype=np.int32)], axis=1)
+            single_tokens = np.zeros(0, dtype=np.int32)
+            max_single_total = 0
+        else:
+            # Tiles with the most keys to walk come first, so that the longest workgroups start first.
+            mixed = any(count == 1 for count in counts)
+            tile_list = sorted(((index, cu[index] + offset, min(QUERY_TILE, count - offset))
+                                for index, count in enumerate(counts) if not (mixed and count == 1)
+                                for offset in range(0, count, QUERY_TILE)),
+                               key=lambda tile: -(starts[tile[0]] + tile[1] - cu[tile[0]] + tile[2]))
+            query_tiles = np.asarray(tile_list, dtype=np.int32).reshape(-1, 3)
+            single_tokens = np.asarray([cu[index] for index, count in enumerate(counts) if mixed and count == 1], dtype=np.int32)
+            max_single_total = max((totals[index] for index, count in enumerate(counts) if mixed and count == 1), default=0)
+        pieces = [tokens, positions, seq_of_token, cu, starts_array, totals_array, slots, want_rows,
+                  query_tiles.reshape(-1), single_tokens]
         for table, mapping in zip(tables, mappings):
             pieces += [table.reshape(-1), mapping]
         offsets, cursor = [], 0
@@ -158,6 +179,6 @@ class BatchBuilder:
             cu_tokens=piece_at(3), seq_start=piece_at(4), seq_total=piece_at(5), slots=piece_at(6),
             want_rows=piece_at(7) if want_rows.size else None, query_tiles=piece_at(8, (-1, 3)),
             single_tokens=piece_at(9) if single_tokens.size else None, max_single_total=max_single_total, paged=paged,
-            starts=list(starts), counts=counts, host_slots=[request.slot for request in requests],
+            starts=starts, counts=counts, host_slots=slots.tolist(),
             max_count=max(counts) if counts else 0, max_total=longest,
             planned_total=longest if fixed_width is None else fixed_width * page_size)

@@ -74,7 +74,8 @@ class Engine:
             num_pages = max(1, -(-max_tokens // page_size))
         reads = [entry.reads_cache_of for entry in spec.order]
         self.cache = CacheManager(self.model.cache_needs(), reads, page_size, num_pages, max_requests,
-                                  dtype=self.dtype, device=self.device)
+                                  dtype=self.dtype, device=self.device,
+                                  max_blocks=-(-spec.max_positions // page_size))
         self._bindings = self.cache.bindings()
         self._builder = BatchBuilder(self.cache, self.device)
         self.steps_run = 0
@@ -124,7 +125,7 @@ class Engine:
     # ---- decode steps from graphs ---------------------------------------------------------
     def _graph_step(self, requests: List[RequestCache], entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         n = len(entries)
-        widest = max(len(pages) for request in requests for pages in request.pages) if self.cache.groups else 1
+        widest = -(-(max(request.num_tokens for request in requests) + 1) // self.cache.page_size)
         width = max(MIN_GRAPH_WIDTH, 1 << (max(widest, 1) - 1).bit_length())
         key = (n, width)
         state = self._graphs.get(key)
