@@ -75,3 +75,30 @@ def write_model_folder(folder: str, config, seed: int, dtype: torch.dtype = torc
     config.save(folder)
     save_file(tensors, os.path.join(folder, "model.safetensors"), metadata={"format": "pt"})
     return folder
+
+
+def main(argv=None) -> int:
+    """``python -m microllm_rocm_amd.weights.random_init --config FILE --seed S --out DIR``: a model folder
+    (config.json, model.safetensors) with random weights for the architecture the configuration names."""
+    import argparse
+
+    from ..config.registry import load_config
+
+    parser = argparse.ArgumentParser(prog="microllm_make_model", description=main.__doc__)
+    parser.add_argument("--config", required=True, help="a config.json (or a folder that holds one)")
+    parser.add_argument("--seed", type=int, default=0)
+    parser.add_argument("--out", required=True, help="folder to write")
+    parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    parser.add_argument("--std", type=float, default=0.02, help="standard deviation of matrices, tables and biases")
+    parser.add_argument("--norm-std", type=float, default=0.0, help="norm weights are 1 + N(0, norm-std)")
+    args = parser.parse_args(argv)
+    _, config = load_config(args.config)
+    dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
+    write_model_folder(args.out, config, args.seed, dtype=dtype, stds={"std": args.std, "norm_std": args.norm_std})
+    print(args.out)
+    return 0
+
+
+if __name__ == "__main__":
+    import sys
+    sys.exit(main())

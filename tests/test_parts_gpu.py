@@ -242,3 +242,33 @@ def test_a_layer_reads_another_layers_cache(dtype):
     got += [engine.step([StepEntry("a", [token], [0])]).cpu() for token in tokens[22:]]
     tol = 2e-5 if dtype == "float32" else 4e-2
     assert np.abs(torch.cat(got).double().numpy() - expected).max() <= tol * np.abs(expected).max()
+
+
+def test_position_embedding_and_head_parts_alone():
+    rt = runtime(torch.bfloat16)
+    rope = build_part("position", PartSpec("rope_split_half", {"theta": 5e4, "head_dim": 48}), rt)
+    expected = 5e4 ** (-np.arange(0, 48, 2) / 48.0)
+    assert rope.fused_split_half and rope.inv_freq.dtype == torch.float64
+    np.testing.assert_allclose(rope.inv_freq.cpu().numpy(), expected, rtol=1e-15)
+    partial = build_part("position", PartSpec("rope_split_half", {"theta": 1e4, "head_dim": 64, "rotary_dim": 32}), rt)
+    assert partial.inv_freq.shape[0] == 16
+    with pytest.raises(ValueError):
+        build_part("position", PartSpec("rope_split_half", {"theta": 1e4, "head_dim": 64, "rotary_dim": 70}), rt)
+    rng = np.random.default_rng(5)
+    sizes = {"vocab_size": 331, "hidden_size": 72}
+    table = bf16_exact(rng.normal(size=(331, 72)))
+    embedding = build_part("embedding", PartSpec("token_embedding", sizes, {"weight": "e"}), rt)
+    head = build_part("head", PartSpec("lm_head", sizes, {"weight": "e"}), rt)       # tied: the same tensor name
+    assert embedding.tensors() == head.tensors()
+    tensors = {"e": table.to(DEVICE)}
+    embedding.bind(tensors)
+    head.bind(tensors)
+    ids = torch.tensor([3, 330, 0], dtype=torch.int32, device=DEVICE)
+    rows = embedding.forward(ids)
+    assert rows.dtype == torch.float32 and torch.equal(rows.cpu(), table[[3, 330, 0]].float())
+    x = bf16_exact(rng.normal(size=(5, 72)))
+    logits = head.forward(x.to(DEVICE))
+    assert logits.dtype == torch.float32 and logits.shape == (5, 331)
+    np.testing.assert_allclose(logits.cpu().numpy(), x.double().numpy() @ table.double().numpy().T, rtol=1e-4, atol=1e-4)
+    with pytest.raises(KeyError, match="unknown mixer kind 'nope'"):
+        build_part("mixer", PartSpec("nope"), rt)

@@ -194,3 +194,26 @@ def test_weights_stored_in_32_bit_stay_32_bit(tmp_path, dtype):
     worst_max, _ = compare(got, requests, plain_model, dtype)
     if dtype == "bfloat16":
         assert worst_max > 1e-4      # activations are still bfloat16: this is not the 32-bit engine in disguise
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_stale_pages_hold_anything(tmp_path_factory, tmp_path, dtype):
+    """Every page is filled with NaN before the trace: what a request has not written itself must never reach a
+    result, whether it lies beyond the request's length, before its window, or on a page used again."""
+    import torch
+    from microllm_rocm_amd.cache.manager import PagedBinding
+    from microllm_rocm_amd.engine import Engine
+    from microllm_rocm_amd.engine.replay import replay
+    config = CONFIGS["C"]
+    folder, plain_model = model_for(tmp_path_factory, "C", SHARP)
+    requests = requests_for(config, [170, 70, 129, 66, 210], seed=80)
+    steps, peak = mixed(requests, seed=11)
+    engine = Engine.from_folder(folder, dtype=dtype, max_tokens=peak, max_requests=8)
+    for binding in engine.cache.bindings():
+        if isinstance(binding, PagedBinding):
+            binding.k.fill_(float("nan"))
+            binding.v.fill_(float("nan"))
+    replay(engine, io.StringIO(to_lines(steps)), str(tmp_path / "out"), io.StringIO())
+    pool = engine.cache.groups[0].pool
+    assert pool.total_taken > pool.num_pages
+    compare(collect(steps, tmp_path / "out", config.vocab_size), requests, plain_model, dtype)

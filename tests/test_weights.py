@@ -161,3 +161,17 @@ def test_random_folder_is_seeded_and_follows_the_rules(tmp_path):
     assert plain_config["sliding_window"] == 24 and plain_config["max_window_layers"] == 1
     ones = plain.read_safetensors(os.path.join(write_model_folder(str(tmp_path / "a"), TINY_A, seed=0), "model.safetensors"))
     assert np.all(ones["model.norm.weight"] == 1.0)
+
+
+def test_model_folder_command(tmp_path):
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    TINY_A.save(str(tmp_path / "src"))
+    out = tmp_path / "made"
+    result = subprocess.run([sys.executable, os.path.join(root, "bin", "microllm_make_model"), "--config", str(tmp_path / "src"),
+                             "--seed", "4", "--out", str(out), "--std", "0.05"], capture_output=True, text=True)
+    assert result.returncode == 0, result.stderr
+    weights = plain.read_safetensors(str(out / "model.safetensors"))
+    assert set(weights) == set(_decls(TINY_A)) and abs(weights["model.embed_tokens.weight"].std() - 0.05) < 5e-3
+    assert plain.read_config(str(out))["hidden_size"] == 64
