@@ -241,9 +241,11 @@ __global__ void silu_mul_kernel(const T* __restrict__ gate, const T* __restrict_
     out[static_cast<int64_t>(token) * width + column] = from_float<T>(g * stable_sigmoid(g) * u);
 }
 
-// The same for bfloat16 rows whose width is a multiple of 8: 16 bytes of gate and of up per thread.
+// The same for bfloat16 rows whose width is a multiple of 8: 16 bytes of gate and of up per thread. With
+// `packed` the result is written in the piece order of the streaming matrix product
+// ([rows/16][width/32][4][16][8], rows padded with whatever the buffer holds) instead of row-major.
 __global__ void silu_mul_bf16x8_kernel(const bf16* __restrict__ gate, const bf16* __restrict__ up, int64_t in_stride,
-                                       bf16* __restrict__ out, int width) {
+                                       bf16* __restrict__ out, int width, int packed) {
     const int token = blockIdx.y;
     const int chunk = blockIdx.x * blockDim.x + threadIdx.x;
     if (chunk * 8 >= width) return;
@@ -255,7 +257,12 @@ __global__ void silu_mul_bf16x8_kernel(const bf16* __restrict__ gate, const bf16
         const float gv = to_float(g.v[i]);
         z.v[i] = from_float<bf16>(gv * stable_sigmoid(gv) * to_float(u.v[i]));
     }
-    *reinterpret_cast<uint4*>(out + static_cast<int64_t>(token) * width + chunk * 8) = z.raw;
+    int64_t target = static_cast<int64_t>(token) * width + chunk * 8;
+    if (packed) {
+        const int k_steps = (width + 31) / 32;
+        target = ((static_cast<int64_t>(token / 16) * k_steps + chunk / 4) * 64 + (chunk % 4) * 16 + token % 16) * 8;
+    }
+    *reinterpret_cast<uint4*>(out + target) = z.raw;
 }
 
 }  // namespace mll
@@ -357,8 +364,10 @@ int mll_qkv_rope_store(const void* qkv, int in_dtype, int n_partials, int64_t pa
 }
 
 int mll_silu_mul(const void* gate, const void* up, int64_t in_stride, void* out, int dtype,
-                 int n_tokens, int width, hipStream_t stream) {
+                 int n_tokens, int width, int packed, hipStream_t stream) {
     MLL_REQUIRE(n_tokens >= 0 && width > 0 && in_stride >= width, "silu_mul: bad sizes");
+    MLL_REQUIRE(!packed || (dtype == kBF16 && width % 32 == 0 && in_stride % 8 == 0),
+                "silu_mul: the packed output needs bfloat16 and a width that is a multiple of 32");
     if (n_tokens == 0) return 0;
     MLL_REQUIRE(n_tokens <= 65535, "silu_mul: more than 65535 tokens in one call");
     const dim3 grid((width + 255) / 256, n_tokens);
@@ -369,7 +378,9 @@ int mll_silu_mul(const void* gate, const void* up, int64_t in_stride, void* out,
                reinterpret_cast<uintptr_t>(up) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
         const dim3 wide_grid((width / 8 + 255) / 256, n_tokens);
         silu_mul_bf16x8_kernel<<<wide_grid, 256, 0, stream>>>(static_cast<const bf16*>(gate), static_cast<const bf16*>(up),
-                                                             in_stride, static_cast<bf16*>(out), width);
+                                                             in_stride, static_cast<bf16*>(out), width, packed);
+    } else if (packed) {
+        return fail("silu_mul: the packed output needs 16-byte aligned operands");
     } else if (dtype == kBF16) {
         silu_mul_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(gate), static_cast<const bf16*>(up),
                                                         in_stride, static_cast<bf16*>(out), width);

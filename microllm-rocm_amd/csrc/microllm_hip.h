@@ -76,9 +76,11 @@ int mll_paged_attention_decode(const void* q, const void* k_cache, const void* v
                                float* part_ml, float scale, int window, int n_tokens, int heads, int kv_heads,
                                int head_dim, int page_size, int n_splits, hipStream_t stream);
 
-// out[t, c] = silu(gate[t, c]) * up[t, c]; gate and up rows are `in_stride` elements apart.
+// out[t, c] = silu(gate[t, c]) * up[t, c]; gate and up rows are `in_stride` elements apart. With `packed`
+// (bfloat16, width a multiple of 32) out is written in the piece order mll_gemm_skinny reads activations in,
+// [tokens/16][width/32][4][16][8]; rows past n_tokens in the last group of 16 are not written.
 int mll_silu_mul(const void* gate, const void* up, int64_t in_stride, void* out, int dtype,
-                 int n_tokens, int width, hipStream_t stream);
+                 int n_tokens, int width, int packed, hipStream_t stream);
 
 // C[m, n] = sum_k A[m, k] * W[n, k] (+ bias[n]), all float32, k summed in ascending order by one
 // thread per output element, so a row's result does not depend on the other rows.

@@ -197,24 +197,32 @@ def paged_attention_rowwise(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     return out
 
 
-def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``silu(gate) * up`` of fused rows ``[tokens, 2 * width]`` (gate first)."""
+def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None, packed: bool = False) -> torch.Tensor:
+    """``silu(gate) * up`` of fused rows ``[tokens, 2 * width]`` (gate first).
+
+    With ``packed`` (bfloat16, width a multiple of 32, at most 64 tokens) the result comes in the piece order of
+    ``gemm_skinny``'s activations, ``[tokens/16, width/32, 4, 16, 8]``; padding rows are not written."""
     lib = library.load()
     _device_tensor(gate_up, "gate/up")
     _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "gate/up must be [tokens, 2 * width]")
     n_tokens, double = gate_up.shape
     width = double // 2
-    if out is None:
+    if packed:
+        _need(gate_up.dtype == torch.bfloat16 and width % 32 == 0 and n_tokens <= 65535, "packed silu_mul needs bfloat16 and width % 32 == 0")
+        _need(out is None, "packed silu_mul allocates its output")
+        # Rows past the last token are left as they are: a row of A only ever reaches its own row of the product.
+        out = torch.empty((-(-n_tokens // 16), width // 32, 4, 16, 8), dtype=gate_up.dtype, device=gate_up.device)
+    elif out is None:
         out = torch.empty((n_tokens, width), dtype=gate_up.dtype, device=gate_up.device)
     _device_tensor(out, "silu_mul output", gate_up.dtype)
-    _need(tuple(out.shape) == (n_tokens, width), "silu_mul output has the wrong shape")
+    _need(packed or tuple(out.shape) == (n_tokens, width), "silu_mul output has the wrong shape")
     element = gate_up.element_size()
     for start in range(0, n_tokens, 65535):
         count = min(65535, n_tokens - start)
         gate_ptr = gate_up.data_ptr() + start * double * element
         _check(lib.mll_silu_mul(ctypes.c_void_p(gate_ptr), ctypes.c_void_p(gate_ptr + width * element),
-                                ctypes.c_int64(double), ctypes.c_void_p(out.data_ptr() + start * width * element),
-                                _code(gate_up.dtype), count, width, _stream()), lib)
+                                ctypes.c_int64(double), ctypes.c_void_p(out.data_ptr() + (0 if packed else start * width * element)),
+                                _code(gate_up.dtype), count, width, int(packed), _stream()), lib)
     return out
 
 

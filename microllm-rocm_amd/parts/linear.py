@@ -32,14 +32,23 @@ class Weight:
         return self.tensor.dtype
 
 
-SKINNY_ROWS = 16   # up to this many rows the streaming kernel beats the library on MI355X
+SKINNY_ROWS = 16        # up to this many rows the streaming kernel beats the library on MI355X for every weight
+SKINNY_TALL_ROWS = 64   # and up to this many for a weight with a long reduction (in >= 4 * out), where the library
+                        # does not split k, if the activations come in the kernel's piece order
 
 
-def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None, gated: bool = False) -> torch.Tensor:
+def streams_tall(weight: "Weight", rows: int) -> bool:
+    """Whether ``linear`` wants packed activations for this weight and this many rows (see ``SKINNY_TALL_ROWS``)."""
+    return (weight.packed is not None and SKINNY_ROWS < rows <= SKINNY_TALL_ROWS
+            and weight.in_features >= 4 * weight.out_features and weight.in_features % 32 == 0)
+
+
+def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None, gated: bool = False,
+           rows: Optional[int] = None) -> torch.Tensor:
     """``x @ W.T`` with float32 accumulation; the result has ``out_dtype`` (default: x's).
 
     With ``gated`` the weight's rows are [gate; up] and the result is ``silu(gate) * up`` of half the
-    width, in x's dtype.
+    width, in x's dtype. ``x`` may come in the streaming kernel's piece order (5 dimensions) with ``rows`` real rows.
     """
     if isinstance(weight, torch.Tensor):
         weight = Weight(weight, pack=False)
@@ -54,6 +63,9 @@ def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None, gat
         return y if out_dtype == torch.float32 else y.to(out_dtype)
     if x.dtype != w.dtype:
         raise TypeError(f"cannot multiply {x.dtype} activations with a {w.dtype} weight")
+    if x.dim() == 5:      # activations in piece order, made for streams_tall(weight, rows)
+        return kernels.gemm_skinny(x, weight.packed, weight.out_features, "bf16" if out_dtype == torch.bfloat16 else "f32",
+                                   rows=rows)
     rows = x.shape[0]
     if weight.packed is not None and rows <= SKINNY_ROWS:
         if gated:

@@ -319,6 +319,10 @@ def test_silu_mul(dtype, width):
     out = kernels().silu_mul(gate_up)
     expected = plain.silu(reference[:, :width]) * reference[:, width:]
     np.testing.assert_allclose(out.float().cpu().numpy(), expected, **tolerance(dtype))
+    if dtype == torch.bfloat16 and width % 32 == 0:
+        packed = kernels().silu_mul(gate_up, packed=True)       # the same numbers in the streaming product's piece order
+        rows = packed.permute(0, 3, 1, 2, 4).reshape(-1, width)[:out.shape[0]]
+        assert torch.equal(rows, out)
     vector = kernels().silu_mul(torch.tensor([[-1.0, 0.0, 1.0, 2.0, 2.0, 2.0]], device=DEVICE)).cpu().numpy()[0]
     np.testing.assert_allclose(vector, [-2 / (1 + math.e), 0.0, 2 / (1 + math.exp(-1))], rtol=1e-6)   # ops_test.cpp:487-495
 

@@ -63,10 +63,11 @@ def test_rms_norm_part(dtype):
 def test_swiglu_part(dtype):
     rng = np.random.default_rng(1)
     names = {f"{r}_proj.weight": f"f.{r}" for r in ("gate", "up", "down")}
-    part = build_part("ffn", PartSpec("swiglu", {"hidden_size": 72, "intermediate_size": 136}, names), runtime(dtype))
-    exact = bind(part, {"f.gate": rng.normal(size=(136, 72)) * 0.3, "f.up": rng.normal(size=(136, 72)) * 0.3,
-                        "f.down": rng.normal(size=(72, 136)) * 0.3}, dtype)
-    for rows in (3, 40):     # few rows take the streaming product, many the library's
+    # 72 x 320: a down projection with a long reduction (in >= 4 * out), which takes the streaming product up to 64 rows
+    part = build_part("ffn", PartSpec("swiglu", {"hidden_size": 72, "intermediate_size": 320}, names), runtime(dtype))
+    exact = bind(part, {"f.gate": rng.normal(size=(320, 72)) * 0.3, "f.up": rng.normal(size=(320, 72)) * 0.3,
+                        "f.down": rng.normal(size=(72, 320)) * 0.3}, dtype)
+    for rows in (3, 40, 100):     # few rows take the streaming product, many the library's
         x = bf16_exact(rng.normal(size=(rows, 72)))
         out = part.forward(x.to(dtype).to(DEVICE), None)
         expected = plain.swiglu_ffn(x.double().numpy(), exact["f.gate"], exact["f.up"], exact["f.down"])
