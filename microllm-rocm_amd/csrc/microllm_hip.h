@@ -97,7 +97,9 @@ int mll_gemm_skinny(const void* a, int a_packed, const void* w_packed, void* out
                     int k, hipStream_t stream);
 
 // Index of the first maximum of each row; a row that holds a non-finite value gives -1.
-int mll_argmax(const float* logits, int32_t* out, int n_rows, int vocab, hipStream_t stream);
+// `parts` is device scratch of n_rows * mll_argmax_slices(vocab) * 16 bytes (contents need not be cleared).
+int mll_argmax(const float* logits, int32_t* out, void* parts, int n_rows, int vocab, hipStream_t stream);
+int mll_argmax_slices(int vocab);
 
 // Draws one token per row from softmax(logits / temperature) restricted to the top_k largest
 // logits (top_k <= 0: all; ties at the k-th value go to the lower token ids), by inverse CDF in

@@ -57,13 +57,45 @@ __device__ inline Best block_argmax(const float* row, int vocab, bool* bad, Best
     return total;
 }
 
-__global__ __launch_bounds__(kSampleThreads) void argmax_kernel(const float* __restrict__ logits,
-                                                                int32_t* __restrict__ out, int vocab) {
-    __shared__ Best best_scratch[kSampleWaves];
-    __shared__ int bad_scratch[kSampleWaves];
-    const float* row = logits + static_cast<int64_t>(blockIdx.x) * vocab;
+// Two stages, so that a row of a large vocabulary is scanned by many blocks: blockIdx.y takes a slice of the
+// row and leaves (value, index, any non-finite) in `parts`; the second stage picks among the slices.
+constexpr int kArgmaxThreads = 256;
+
+struct ArgmaxPart {
+    float value;
+    int index;
+    int bad;
+    int pad;
+};
+
+__global__ __launch_bounds__(kArgmaxThreads) void argmax_slices_kernel(const float* __restrict__ logits,
+                                                                       ArgmaxPart* __restrict__ parts, int vocab,
+                                                                       int slice) {
+    __shared__ Best best_scratch[kArgmaxThreads / kWave];
+    __shared__ int bad_scratch[kArgmaxThreads / kWave];
+    const int begin = blockIdx.y * slice;
+    const int count = max(0, min(slice, vocab - begin));
+    const float* row = logits + static_cast<int64_t>(blockIdx.x) * vocab + begin;
     bool bad;
-    const Best best = block_argmax(row, vocab, &bad, best_scratch, bad_scratch);
+    const Best best = block_argmax(row, count, &bad, best_scratch, bad_scratch);
+    if (threadIdx.x == 0)
+        parts[blockIdx.x * gridDim.y + blockIdx.y] = ArgmaxPart{best.value, best.index == 0x7fffffff ? best.index : best.index + begin, bad ? 1 : 0, 0};
+}
+
+__global__ __launch_bounds__(kWave) void argmax_pick_kernel(const ArgmaxPart* __restrict__ parts,
+                                                           int32_t* __restrict__ out, int n_slices) {
+    Best best{-INFINITY, 0x7fffffff};
+    int bad = 0;
+    for (int index = threadIdx.x; index < n_slices; index += kWave) {
+        const ArgmaxPart part = parts[blockIdx.x * n_slices + index];
+        best = better(best, Best{part.value, part.index});
+        bad |= part.bad;
+    }
+#pragma unroll
+    for (int offset = kWave / 2; offset > 0; offset >>= 1) {
+        best = better(best, Best{__shfl_xor(best.value, offset, kWave), __shfl_xor(best.index, offset, kWave)});
+        bad |= __shfl_xor(bad, offset, kWave);
+    }
     if (threadIdx.x == 0) out[blockIdx.x] = bad ? -1 : best.index;
 }
 
@@ -210,10 +242,17 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
 
 using namespace mll;
 
-extern "C" int mll_argmax(const float* logits, int32_t* out, int n_rows, int vocab, hipStream_t stream) {
+extern "C" int mll_argmax_slices(int vocab) { return max(1, min(64, (vocab + 2047) / 2048)); }
+
+extern "C" int mll_argmax(const float* logits, int32_t* out, void* parts, int n_rows, int vocab, hipStream_t stream) {
     MLL_REQUIRE(n_rows >= 0 && vocab > 0, "argmax: sizes must be positive");
+    MLL_REQUIRE(parts != nullptr, "argmax: needs the scratch for its slices");
+    MLL_REQUIRE(n_rows <= 65535, "argmax: more than 65535 rows");
     if (n_rows == 0) return 0;
-    argmax_kernel<<<n_rows, kSampleThreads, 0, stream>>>(logits, out, vocab);
+    const int slices = mll_argmax_slices(vocab);
+    const int slice = (vocab + slices - 1) / slices;
+    argmax_slices_kernel<<<dim3(n_rows, slices), kArgmaxThreads, 0, stream>>>(logits, static_cast<ArgmaxPart*>(parts), vocab, slice);
+    argmax_pick_kernel<<<n_rows, kWave, 0, stream>>>(static_cast<const ArgmaxPart*>(parts), out, slices);
     return check_launch("argmax");
 }
 

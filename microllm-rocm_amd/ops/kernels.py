@@ -255,8 +255,10 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     lib = library.load()
     _device_tensor(logits, "logits", torch.float32)
     _need(logits.dim() == 2, "logits must be [rows, vocab]")
-    out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
-    _check(lib.mll_argmax(_ptr(logits), _ptr(out), logits.shape[0], logits.shape[1], _stream()), lib)
+    rows, vocab = logits.shape
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    parts = torch.empty((rows, lib.mll_argmax_slices(vocab), 4), dtype=torch.int32, device=logits.device)
+    _check(lib.mll_argmax(_ptr(logits), _ptr(out), _ptr(parts), rows, vocab, _stream()), lib)
     return out
 
 
