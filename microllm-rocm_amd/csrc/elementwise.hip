@@ -67,10 +67,16 @@ __global__ void rms_norm_kernel(float* __restrict__ h, const D* __restrict__ del
     }
 }
 
+__device__ inline float4 load_four(const float* source) { return *reinterpret_cast<const float4*>(source); }
+__device__ inline float4 load_four(const bf16* source) {
+    return make_float4(to_float(source[0]), to_float(source[1]), to_float(source[2]), to_float(source[3]));
+}
+
 // The same for rows of float4: one pass, the row kept in registers between the sum of squares and the
 // scaling. Taken when the width is a multiple of 4 and at most 4 * CHUNKS * blockDim.x.
 template <typename T, typename D, int CHUNKS>
 __global__ void rms_norm_vec4_kernel(float* __restrict__ h, const D* __restrict__ delta,
+                                     int n_partials, int64_t partial_stride,
                                      const int32_t* __restrict__ rows, const float* __restrict__ weight,
                                      float eps, T* __restrict__ out, int width, int write_h) {
     __shared__ float scratch[16];
@@ -90,10 +96,19 @@ __global__ void rms_norm_vec4_kernel(float* __restrict__ h, const D* __restrict_
         if (q < quads) {
             value[c] = reinterpret_cast<const float4*>(h_row)[q];
             if (delta_row) {
-                value[c].x += to_float(delta_row[4 * q + 0]);
-                value[c].y += to_float(delta_row[4 * q + 1]);
-                value[c].z += to_float(delta_row[4 * q + 2]);
-                value[c].w += to_float(delta_row[4 * q + 3]);
+                // The parts of the delta are added first, in order, and their sum to the stream.
+                float4 sum = load_four(delta_row + 4 * q);
+                for (int part = 1; part < n_partials; ++part) {
+                    const float4 more = load_four(delta_row + part * partial_stride + 4 * q);
+                    sum.x += more.x;
+                    sum.y += more.y;
+                    sum.z += more.z;
+                    sum.w += more.w;
+                }
+                value[c].x += sum.x;
+                value[c].y += sum.y;
+                value[c].z += sum.z;
+                value[c].w += sum.w;
             }
             if (write_h) reinterpret_cast<float4*>(h_row)[q] = value[c];
             partial += value[c].x * value[c].x + value[c].y * value[c].y + value[c].z * value[c].z + value[c].w * value[c].w;
@@ -118,14 +133,16 @@ template <typename T, typename D>
 static void launch_rms_norm(float* h, const D* delta, int n_partials, int64_t partial_stride, const int32_t* rows,
                             const float* weight, float eps, T* out, int n_rows, int width, int write_h,
                             hipStream_t stream) {
-    const bool aligned = width % 4 == 0 && n_partials == 1 &&
+    const bool delta_aligned = delta == nullptr || sizeof(D) != sizeof(float) ||
+                               (reinterpret_cast<uintptr_t>(delta) % 16 == 0 && (n_partials == 1 || partial_stride % 4 == 0));
+    const bool aligned = width % 4 == 0 && delta_aligned &&
                          reinterpret_cast<uintptr_t>(h) % 16 == 0 && reinterpret_cast<uintptr_t>(weight) % 16 == 0;
     const int quads = width / 4;
     if (aligned && quads <= 1024) {
         const int threads = max(64, (quads + 63) / 64 * 64);
-        rms_norm_vec4_kernel<T, D, 1><<<n_rows, threads, 0, stream>>>(h, delta, rows, weight, eps, out, width, write_h);
+        rms_norm_vec4_kernel<T, D, 1><<<n_rows, threads, 0, stream>>>(h, delta, n_partials, partial_stride, rows, weight, eps, out, width, write_h);
     } else if (aligned && quads <= 4096) {
-        rms_norm_vec4_kernel<T, D, 4><<<n_rows, 1024, 0, stream>>>(h, delta, rows, weight, eps, out, width, write_h);
+        rms_norm_vec4_kernel<T, D, 4><<<n_rows, 1024, 0, stream>>>(h, delta, n_partials, partial_stride, rows, weight, eps, out, width, write_h);
     } else {
         const int threads = width >= 2048 ? 512 : 256;
         rms_norm_kernel<T, D><<<n_rows, threads, 0, stream>>>(h, delta, n_partials, partial_stride, rows, weight, eps,
@@ -241,11 +258,9 @@ __global__ void silu_mul_kernel(const T* __restrict__ gate, const T* __restrict_
     out[static_cast<int64_t>(token) * width + column] = from_float<T>(g * stable_sigmoid(g) * u);
 }
 
-// The same for bfloat16 rows whose width is a multiple of 8: 16 bytes of gate and of up per thread. With
-// `packed` the result is written in the piece order of the streaming matrix product
-// ([rows/16][width/32][4][16][8], rows padded with whatever the buffer holds) instead of row-major.
+// The same for bfloat16 rows whose width is a multiple of 8: 16 bytes of gate and of up per thread.
 __global__ void silu_mul_bf16x8_kernel(const bf16* __restrict__ gate, const bf16* __restrict__ up, int64_t in_stride,
-                                       bf16* __restrict__ out, int width, int packed) {
+                                       bf16* __restrict__ out, int width) {
     const int token = blockIdx.y;
     const int chunk = blockIdx.x * blockDim.x + threadIdx.x;
     if (chunk * 8 >= width) return;
@@ -257,12 +272,7 @@ __global__ void silu_mul_bf16x8_kernel(const bf16* __restrict__ gate, const bf16
         const float gv = to_float(g.v[i]);
         z.v[i] = from_float<bf16>(gv * stable_sigmoid(gv) * to_float(u.v[i]));
     }
-    int64_t target = static_cast<int64_t>(token) * width + chunk * 8;
-    if (packed) {
-        const int k_steps = (width + 31) / 32;
-        target = ((static_cast<int64_t>(token / 16) * k_steps + chunk / 4) * 64 + (chunk % 4) * 16 + token % 16) * 8;
-    }
-    *reinterpret_cast<uint4*>(out + target) = z.raw;
+    *reinterpret_cast<uint4*>(out + static_cast<int64_t>(token) * width + chunk * 8) = z.raw;
 }
 
 }  // namespace mll
@@ -364,10 +374,8 @@ int mll_qkv_rope_store(const void* qkv, int in_dtype, int n_partials, int64_t pa
 }
 
 int mll_silu_mul(const void* gate, const void* up, int64_t in_stride, void* out, int dtype,
-                 int n_tokens, int width, int packed, hipStream_t stream) {
+                 int n_tokens, int width, hipStream_t stream) {
     MLL_REQUIRE(n_tokens >= 0 && width > 0 && in_stride >= width, "silu_mul: bad sizes");
-    MLL_REQUIRE(!packed || (dtype == kBF16 && width % 32 == 0 && in_stride % 8 == 0),
-                "silu_mul: the packed output needs bfloat16 and a width that is a multiple of 32");
     if (n_tokens == 0) return 0;
     MLL_REQUIRE(n_tokens <= 65535, "silu_mul: more than 65535 tokens in one call");
     const dim3 grid((width + 255) / 256, n_tokens);
@@ -378,9 +386,7 @@ int mll_silu_mul(const void* gate, const void* up, int64_t in_stride, void* out,
                reinterpret_cast<uintptr_t>(up) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
         const dim3 wide_grid((width / 8 + 255) / 256, n_tokens);
         silu_mul_bf16x8_kernel<<<wide_grid, 256, 0, stream>>>(static_cast<const bf16*>(gate), static_cast<const bf16*>(up),
-                                                             in_stride, static_cast<bf16*>(out), width, packed);
-    } else if (packed) {
-        return fail("silu_mul: the packed output needs 16-byte aligned operands");
+                                                             in_stride, static_cast<bf16*>(out), width);
     } else if (dtype == kBF16) {
         silu_mul_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(gate), static_cast<const bf16*>(up),
                                                         in_stride, static_cast<bf16*>(out), width);

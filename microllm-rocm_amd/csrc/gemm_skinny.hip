@@ -30,11 +30,9 @@ __device__ inline float silu_f(float value) {
 }
 
 // EPILOGUE: 0 = float32 [M, N]; 1 = bfloat16 [M, N]; 2 = bfloat16 [M, N / 2] = silu(even rows of W) * (odd rows).
-// A_PACKED: the activations come in the same piece order as the weight ([M/16][K/32][4][16][8], zero padded),
-// so a wave's load of a piece of A is one contiguous KB too; otherwise A is row-major [M, K].
 // TEMPORAL: W is read with ordinary loads instead of non-temporal ones (measured on MI355X: better for weights
 // of a few tens of MB, worse for the large ones).
-template <int MT, int NT, int EPILOGUE, bool A_PACKED, bool TEMPORAL>
+template <int MT, int NT, int EPILOGUE, bool TEMPORAL>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w_packed, void* __restrict__ out,
     int m, int n, int k, int n_tiles, int k_steps) {
@@ -63,9 +61,8 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int row = mt * 16 + col;
-        a_live[mt] = A_PACKED ? mt * 16 < m : row < m;
-        a_ptr[mt] = A_PACKED ? a + static_cast<int64_t>(mt) * k_steps * 512 + lane * 8
-                             : a + static_cast<int64_t>(a_live[mt] ? row : 0) * k + quad * 8;
+        a_live[mt] = row < m;
+        a_ptr[mt] = a + static_cast<int64_t>(a_live[mt] ? row : 0) * k + quad * 8;
     }
 
     // A wave takes kChunk consecutive k steps at a time, then skips what the other waves take; which k steps a
@@ -95,12 +92,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
                     a_piece[u][mt].raw = uintx4{0u, 0u, 0u, 0u};
-                    if (A_PACKED) {
-                        if (a_live[mt] && live)
-                            a_piece[u][mt].raw = *reinterpret_cast<const uintx4*>(a_ptr[mt] + static_cast<int64_t>(ks) * 512);
-                    } else if (a_live[mt] && in_k) {
-                        a_piece[u][mt].raw = *reinterpret_cast<const uintx4*>(a_ptr[mt] + k_offset);
-                    }
+                    if (a_live[mt] && in_k) a_piece[u][mt].raw = *reinterpret_cast<const uintx4*>(a_ptr[mt] + k_offset);
                 }
             }
 #pragma unroll
@@ -167,7 +159,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
 }
 
 template <int MT, int NT, int EPILOGUE>
-static void launch_one(const bf16* a, int a_packed, const bf16* w, void* out, int m, int n, int k, int n_tiles,
+static void launch_one(const bf16* a, const bf16* w, void* out, int m, int n, int k, int n_tiles,
                        int k_steps, hipStream_t stream) {
     const int groups = (n_tiles + NT - 1) / NT;
     // Waves per workgroup: enough that about eight thousand waves would stream W one tile each, at most 16, and
@@ -176,18 +168,14 @@ static void launch_one(const bf16* a, int a_packed, const bf16* w, void* out, in
     while (waves < 16 && n_tiles * waves * 2 <= 8192 && waves * 2 * kChunk <= k_steps) waves *= 2;
     const size_t lds = waves > 1 ? static_cast<size_t>(waves - 1) * NT * MT * kWave * sizeof(floatx4) : 0;
     const bool temporal = static_cast<int64_t>(n_tiles) * k_steps * 1024 < (64ll << 20);   // bytes of the packed weight
-    if (a_packed && temporal)
-        gemm_skinny_kernel<MT, NT, EPILOGUE, true, true><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps);
-    else if (a_packed)
-        gemm_skinny_kernel<MT, NT, EPILOGUE, true, false><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps);
-    else if (temporal)
-        gemm_skinny_kernel<MT, NT, EPILOGUE, false, true><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps);
+    if (temporal)
+        gemm_skinny_kernel<MT, NT, EPILOGUE, true><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps);
     else
-        gemm_skinny_kernel<MT, NT, EPILOGUE, false, false><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps);
+        gemm_skinny_kernel<MT, NT, EPILOGUE, false><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps);
 }
 
 template <int EPILOGUE>
-static int launch_skinny(const void* a, int a_packed, const void* w_packed, void* out, int m, int n, int k,
+static int launch_skinny(const void* a, const void* w_packed, void* out, int m, int n, int k,
                          hipStream_t stream) {
     const int n_tiles = (n + 15) / 16;
     const int k_steps = (k + 31) / 32;
@@ -200,15 +188,15 @@ static int launch_skinny(const void* a, int a_packed, const void* w_packed, void
     const bool wide = n_tiles >= 2048;
     switch (m_tiles) {
         case 1:
-            if (wide || (m > 4 && n_tiles >= 256)) launch_one<1, 2, EPILOGUE>(a_, a_packed, w_, out, m, n, k, n_tiles, k_steps, stream);
-            else launch_one<1, 1, EPILOGUE>(a_, a_packed, w_, out, m, n, k, n_tiles, k_steps, stream);
+            if (wide || (m > 4 && n_tiles >= 256)) launch_one<1, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream);
+            else launch_one<1, 1, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream);
             break;
         case 2:
-            if (wide) launch_one<2, 2, EPILOGUE>(a_, a_packed, w_, out, m, n, k, n_tiles, k_steps, stream);
-            else launch_one<2, 1, EPILOGUE>(a_, a_packed, w_, out, m, n, k, n_tiles, k_steps, stream);
+            if (wide) launch_one<2, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream);
+            else launch_one<2, 1, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream);
             break;
-        case 3: launch_one<3, 2, EPILOGUE>(a_, a_packed, w_, out, m, n, k, n_tiles, k_steps, stream); break;
-        case 4: launch_one<4, 2, EPILOGUE>(a_, a_packed, w_, out, m, n, k, n_tiles, k_steps, stream); break;
+        case 3: launch_one<3, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream); break;
+        case 4: launch_one<4, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream); break;
         default: return fail("gemm_skinny: more than 64 rows");
     }
     return check_launch("gemm_skinny");
@@ -218,16 +206,16 @@ static int launch_skinny(const void* a, int a_packed, const void* w_packed, void
 
 using namespace mll;
 
-extern "C" int mll_gemm_skinny(const void* a, int a_packed, const void* w_packed, void* out, int epilogue, int m,
-                               int n, int k, hipStream_t stream) {
+extern "C" int mll_gemm_skinny(const void* a, const void* w_packed, void* out, int epilogue, int m, int n, int k,
+                               hipStream_t stream) {
     MLL_REQUIRE(m >= 0 && m <= 64, "gemm_skinny: takes at most 64 rows");
     MLL_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_skinny: k must be a positive multiple of 8");
     MLL_REQUIRE(epilogue != 2 || n % 2 == 0, "gemm_skinny: the gated epilogue needs an even number of weight rows");
     if (m == 0) return 0;
     switch (epilogue) {
-        case 0: return launch_skinny<0>(a, a_packed, w_packed, out, m, n, k, stream);
-        case 1: return launch_skinny<1>(a, a_packed, w_packed, out, m, n, k, stream);
-        case 2: return launch_skinny<2>(a, a_packed, w_packed, out, m, n, k, stream);
+        case 0: return launch_skinny<0>(a, w_packed, out, m, n, k, stream);
+        case 1: return launch_skinny<1>(a, w_packed, out, m, n, k, stream);
+        case 2: return launch_skinny<2>(a, w_packed, out, m, n, k, stream);
         default: return fail("gemm_skinny: unknown epilogue");
     }
 }

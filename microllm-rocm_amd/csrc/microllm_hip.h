@@ -65,22 +65,8 @@ int mll_paged_attention_prefill(const void* q, const void* k_cache, const void* 
 int mll_paged_attention_prefill_tile();
 
 // out[t, c] = silu(gate[t, c]) * up[t, c]; gate and up rows are `in_stride` elements apart.
-// The same attention for bfloat16 with MFMA, one workgroup per (token, kv head, split of the keys): meant
-// for steps whose requests bring one token each, right for any. head_dim a multiple of 16 up to 256,
-// page_size a multiple of 16. n_splits > 1 needs part_o [tokens, heads, n_splits, head_dim] and
-// part_ml [tokens, heads, n_splits, 2] (float32 device scratch, contents need not be cleared).
-// token_ids (nullable) lists the n_tokens rows of q / out to work on; without it all rows 0 .. n_tokens-1.
-int mll_paged_attention_decode(const void* q, const void* k_cache, const void* v_cache,
-                               const int32_t* block_table, int table_width, const int32_t* seq_of_token,
-                               const int32_t* positions, const int32_t* token_ids, void* out, float* part_o,
-                               float* part_ml, float scale, int window, int n_tokens, int heads, int kv_heads,
-                               int head_dim, int page_size, int n_splits, hipStream_t stream);
-
-// out[t, c] = silu(gate[t, c]) * up[t, c]; gate and up rows are `in_stride` elements apart. With `packed`
-// (bfloat16, width a multiple of 32) out is written in the piece order mll_gemm_skinny reads activations in,
-// [tokens/16][width/32][4][16][8]; rows past n_tokens in the last group of 16 are not written.
 int mll_silu_mul(const void* gate, const void* up, int64_t in_stride, void* out, int dtype,
-                 int n_tokens, int width, int packed, hipStream_t stream);
+                 int n_tokens, int width, hipStream_t stream);
 
 // C[m, n] = sum_k A[m, k] * W[n, k] (+ bias[n]), all float32, k summed in ascending order by one
 // thread per output element, so a row's result does not depend on the other rows.
@@ -91,10 +77,16 @@ int mll_gemm_f32(const float* a, const float* w, const float* bias, float* c,
 // element (row, col) of W sits at piece (row / 16, col / 32), position ((col % 32) / 8, row % 16, col % 8).
 // epilogue 0: float32 [m, n]; 1: bfloat16 [m, n]; 2: bfloat16 [m, n / 2] = silu(even weight rows' results) *
 // (odd rows' results). The order of additions is fixed by (n, k): the same in every run and whatever the
-// other rows of A. With a_packed the activations
-// come in the weight's piece order too ([m/16][k/32][4][16][8], zero padded) instead of row-major [m, k].
-int mll_gemm_skinny(const void* a, int a_packed, const void* w_packed, void* out, int epilogue, int m, int n,
-                    int k, hipStream_t stream);
+// other rows of A.
+int mll_gemm_skinny(const void* a, const void* w_packed, void* out, int epilogue, int m, int n, int k,
+                    hipStream_t stream);
+
+// The same product for up to 64 rows with the activations shared through LDS by the waves of a workgroup
+// (faster than mll_gemm_skinny from 17 rows on). A wave takes tiles_per_wave (1 or 2) tiles of W. With
+// splits > 1 (epilogue 0 only) k is cut into that many ranges and out is [splits][m][n]: partial sums that the
+// caller adds in order. The order of additions is fixed by (n, k, splits).
+int mll_gemm_medium(const void* a, const void* w_packed, void* out, int epilogue, int m, int n, int k,
+                    int tiles_per_wave, int waves, int splits, hipStream_t stream);
 
 // Index of the first maximum of each row; a row that holds a non-finite value gives -1.
 // `parts` is device scratch of n_rows * mll_argmax_slices(vocab) * 16 bytes (contents need not be cleared).

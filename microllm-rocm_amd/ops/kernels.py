@@ -7,7 +7,7 @@ a kernel never sees operands that do not fit what its grid assumes.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -197,32 +197,24 @@ def paged_attention_rowwise(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     return out
 
 
-def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None, packed: bool = False) -> torch.Tensor:
-    """``silu(gate) * up`` of fused rows ``[tokens, 2 * width]`` (gate first).
-
-    With ``packed`` (bfloat16, width a multiple of 32, at most 64 tokens) the result comes in the piece order of
-    ``gemm_skinny``'s activations, ``[tokens/16, width/32, 4, 16, 8]``; padding rows are not written."""
+def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``silu(gate) * up`` of fused rows ``[tokens, 2 * width]`` (gate first)."""
     lib = library.load()
     _device_tensor(gate_up, "gate/up")
     _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "gate/up must be [tokens, 2 * width]")
     n_tokens, double = gate_up.shape
     width = double // 2
-    if packed:
-        _need(gate_up.dtype == torch.bfloat16 and width % 32 == 0 and n_tokens <= 65535, "packed silu_mul needs bfloat16 and width % 32 == 0")
-        _need(out is None, "packed silu_mul allocates its output")
-        # Rows past the last token are left as they are: a row of A only ever reaches its own row of the product.
-        out = torch.empty((-(-n_tokens // 16), width // 32, 4, 16, 8), dtype=gate_up.dtype, device=gate_up.device)
-    elif out is None:
+    if out is None:
         out = torch.empty((n_tokens, width), dtype=gate_up.dtype, device=gate_up.device)
     _device_tensor(out, "silu_mul output", gate_up.dtype)
-    _need(packed or tuple(out.shape) == (n_tokens, width), "silu_mul output has the wrong shape")
+    _need(tuple(out.shape) == (n_tokens, width), "silu_mul output has the wrong shape")
     element = gate_up.element_size()
     for start in range(0, n_tokens, 65535):
         count = min(65535, n_tokens - start)
         gate_ptr = gate_up.data_ptr() + start * double * element
         _check(lib.mll_silu_mul(ctypes.c_void_p(gate_ptr), ctypes.c_void_p(gate_ptr + width * element),
-                                ctypes.c_int64(double), ctypes.c_void_p(out.data_ptr() + (0 if packed else start * width * element)),
-                                _code(gate_up.dtype), count, width, int(packed), _stream()), lib)
+                                ctypes.c_int64(double), ctypes.c_void_p(out.data_ptr() + start * width * element),
+                                _code(gate_up.dtype), count, width, _stream()), lib)
     return out
 
 
@@ -414,8 +406,7 @@ def pack_weight(weight: torch.Tensor, interleave_halves: bool = False) -> torch.
 SKINNY_MAX_ROWS = 64
 
 
-def gemm_skinny(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f32",
-                rows: Optional[int] = None) -> torch.Tensor:
+def gemm_skinny(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f32") -> torch.Tensor:
     """``x @ W.T`` for at most 64 bfloat16 rows and a packed weight.
 
     ``f32``: float32 ``[m, n]``; ``bf16``: bfloat16 ``[m, n]``; ``gated``: bfloat16 ``[m, n / 2]`` of
@@ -425,14 +416,8 @@ def gemm_skinny(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "
     _device_tensor(x, "gemm input", torch.bfloat16)
     _device_tensor(packed, "packed weight", torch.bfloat16)
     _need(packed.dim() == 5 and tuple(packed.shape[2:]) == (4, 16, 8), "gemm_skinny takes a packed weight")
-    a_packed = x.dim() == 5       # activations in piece order [m/16, k/32, 4, 16, 8]; `rows` says how many are real
-    if a_packed:
-        _need(tuple(x.shape[2:]) == (4, 16, 8) and rows is not None and rows <= x.shape[0] * 16, "bad packed activations")
-        m, k = rows, packed.shape[1] * 32
-        _need(x.shape[1] == packed.shape[1], "packed activations and weight differ in k")
-    else:
-        _need(x.dim() == 2, "gemm_skinny takes [m, k] activations")
-        m, k = x.shape
+    _need(x.dim() == 2, "gemm_skinny takes [m, k] activations")
+    m, k = x.shape
     _need(m <= SKINNY_MAX_ROWS, "gemm_skinny takes at most 64 rows")
     _need(k % 8 == 0, "gemm_skinny needs k to be a multiple of 8")
     _need(packed.shape[0] == -(-n // 16) and packed.shape[1] == -(-k // 32), "the packed weight does not fit n and k")
@@ -444,5 +429,61 @@ def gemm_skinny(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "
         code, out = 2, torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
     else:
         raise KernelLibraryError(f"unknown epilogue {epilogue!r}")
-    _check(lib.mll_gemm_skinny(_ptr(x), int(a_packed), _ptr(packed), _ptr(out), code, m, n, k, _stream()), lib)
+    _check(lib.mll_gemm_skinny(_ptr(x), _ptr(packed), _ptr(out), code, m, n, k, _stream()), lib)
+    return out
+
+
+MEDIUM_WORKGROUPS = 224     # workgroups of 8 waves that gemm_medium wants at least (MI355X has 256 compute units)
+
+
+def medium_plan(n: int, k: int, may_split: bool = True) -> Tuple[int, int, int]:
+    """(tiles of W a wave takes, waves a workgroup, splits of k) for ``gemm_medium``.
+
+    A function of the weight's shape alone, so that a row's sum does not depend on the other rows. Two tiles a
+    wave halve the reads of the activations; they are taken where splitting k (at most 16 times, a stage of 256
+    at least per split) still gives enough workgroups.
+    """
+    n_tiles = -(-n // 16)
+    stages = -(-k // 256)
+    most = 1
+    while may_split and most * 2 <= min(16, stages):
+        most *= 2
+    tiles_per_wave = 2 if -(-n_tiles // 16) * most >= MEDIUM_WORKGROUPS else 1
+    groups = -(-n_tiles // (8 * tiles_per_wave))
+    splits = 1
+    while splits < most and groups * splits < MEDIUM_WORKGROUPS:
+        splits *= 2
+    return tiles_per_wave, 8, splits
+
+
+def gemm_medium(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f32",
+                plan: Optional[Tuple[int, int, int]] = None) -> torch.Tensor:
+    """``x @ W.T`` for at most 64 bfloat16 rows ``[m, k]`` and a packed weight, activations shared through LDS.
+
+    ``plan`` is ``medium_plan``'s by default; pass ``medium_plan(n, k, may_split=False)`` for a plain ``[m, n]``.
+
+    ``f32``: float32 ``[m, n]``, or ``[splits, m, n]`` partial sums to be added in order when the plan splits k;
+    ``bf16`` and ``gated`` as in ``gemm_skinny`` (they never split).
+    """
+    lib = library.load()
+    _device_tensor(x, "gemm input", torch.bfloat16)
+    _device_tensor(packed, "packed weight", torch.bfloat16)
+    _need(packed.dim() == 5 and tuple(packed.shape[2:]) == (4, 16, 8), "gemm_medium takes a packed weight")
+    _need(x.dim() == 2, "gemm_medium takes [m, k] activations")
+    m, k = x.shape
+    _need(m <= SKINNY_MAX_ROWS, "gemm_medium takes at most 64 rows")
+    _need(k % 8 == 0, "gemm_medium needs k to be a multiple of 8")
+    _need(packed.shape[0] == -(-n // 16) and packed.shape[1] == -(-k // 32), "the packed weight does not fit n and k")
+    tiles_per_wave, waves, splits = plan if plan is not None else medium_plan(n, k, may_split=epilogue == "f32")
+    _need(epilogue == "f32" or splits == 1, "only float32 partial sums can be split over k")
+    if epilogue == "f32":
+        code = 0
+        out = torch.empty((splits, m, n) if splits > 1 else (m, n), dtype=torch.float32, device=x.device)
+    elif epilogue == "bf16":
+        code, out = 1, torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    elif epilogue == "gated":
+        code, out = 2, torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
+    else:
+        raise KernelLibraryError(f"unknown epilogue {epilogue!r}")
+    _check(lib.mll_gemm_medium(_ptr(x), _ptr(packed), _ptr(out), code, m, n, k, tiles_per_wave, waves, splits, _stream()), lib)
     return out

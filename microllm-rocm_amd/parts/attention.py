@@ -78,7 +78,7 @@ class PagedAttention(Mixer):
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
         view = ctx.paged[cache.group]
         kv_heads = cache.need.kv_heads
-        qkv = linear(x, self.qkv_weight, out_dtype=torch.float32)   # rounded once, after bias and rotation
+        qkv = linear(x, self.qkv_weight, out_dtype=torch.float32, partials=True)   # rounded once, after bias and rotation
         stored_heads = self.kv_heads if self.owns_kv else 0
         slot_mapping = view.slot_mapping if self.owns_kv else None
         k_pages = cache.k if self.owns_kv else None
@@ -98,7 +98,7 @@ class PagedAttention(Mixer):
         window = int(self.window) if self.window else 0
         o = kernels.paged_attention(q, cache.k, cache.v, view, ctx, self.scale, window,
                                     self.heads, kv_heads, self.head_dim)
-        return linear(o, self.o_weight, out_dtype=torch.float32)   # summed into the residual stream in float32
+        return linear(o, self.o_weight, out_dtype=torch.float32, partials=True)   # summed into the residual stream in float32
 
 
 register_part("mixer", "paged_attention", PagedAttention)

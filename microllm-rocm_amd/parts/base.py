@@ -82,7 +82,9 @@ class Mixer(Part):
     def cache_need(self) -> CacheNeed:
         return None
 
-    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:  # [tokens, hidden] -> [tokens, hidden]
+    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+        """``[tokens, hidden]`` -> the delta for the residual stream: ``[tokens, hidden]``, or float32 partial
+        sums ``[parts, tokens, hidden]`` that the next norm adds in order."""
         raise NotImplementedError
 
 
@@ -90,6 +92,7 @@ class FeedForward(Part):
     category = "ffn"
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        """``[tokens, hidden]`` -> the delta for the residual stream, as a mixer's."""
         raise NotImplementedError
 
 
@@ -98,7 +101,9 @@ class Norm(Part):
 
     def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor] = None, write_h: bool = True,
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """Normalise ``h + delta`` (float32 residual stream); with ``write_h`` the sum replaces ``h``."""
+        """Normalise ``h + delta`` (float32 residual stream); with ``write_h`` the sum replaces ``h``.
+
+        ``delta`` is ``[tokens, hidden]`` or float32 partial sums ``[parts, tokens, hidden]``, added in order first."""
         raise NotImplementedError
 
 

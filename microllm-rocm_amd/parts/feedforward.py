@@ -12,7 +12,7 @@ import torch
 
 from ..ops import kernels
 from .base import FeedForward, MATRIX, Runtime, TensorDecl
-from .linear import Weight, linear, streams_tall
+from .linear import Weight, linear
 from .registry import register_part
 from .spec import PartSpec
 
@@ -42,15 +42,8 @@ class SwiGLU(FeedForward):
         self.down_weight = Weight(tensors[self.name("down_proj.weight")])
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        rows = x.shape[0]
-        if x.dtype == torch.bfloat16 and streams_tall(self.down_weight, rows) and self.gate_up_weight.dtype == torch.bfloat16:
-            # Between 17 and 64 rows the library takes gate/up and the streaming kernel takes the long reduction of
-            # down, with the activation written in the order that kernel reads.
-            gate_up = kernels.gemm_bf16(x, self.gate_up_weight.tensor, torch.bfloat16)
-            z = kernels.silu_mul(gate_up, packed=True)
-            return linear(z, self.down_weight, out_dtype=torch.float32, rows=rows)
         z = linear(x, self.gate_up_weight, gated=True)
-        return linear(z, self.down_weight, out_dtype=torch.float32)
+        return linear(z, self.down_weight, out_dtype=torch.float32, partials=True)
 
 
 register_part("ffn", "swiglu", SwiGLU)

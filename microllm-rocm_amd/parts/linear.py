@@ -4,8 +4,9 @@ The reference stores ``[in, out]`` and transposes every linear at load
 (src/model/model.cpp:285, 1939-1973); keeping ``[out, in]`` removes that pass and
 lets several weights that share an input be stacked along ``out``. A bfloat16
 weight is held twice on the GPU: as stored, for the library product that steps
-with many rows use, and packed in the order the MFMA consumes it, for the kernel
-that streams it once when a step has few rows (decoding).
+with many rows use, and packed in the order the MFMA consumes it, for the two
+kernels that stream it once when a step has few rows (decoding): one for up to
+16 rows, one that shares the activations between waves for up to 64.
 """
 from __future__ import annotations
 
@@ -32,23 +33,19 @@ class Weight:
         return self.tensor.dtype
 
 
-SKINNY_ROWS = 16        # up to this many rows the streaming kernel beats the library on MI355X for every weight
-SKINNY_TALL_ROWS = 64   # and up to this many for a weight with a long reduction (in >= 4 * out), where the library
-                        # does not split k, if the activations come in the kernel's piece order
-
-
-def streams_tall(weight: "Weight", rows: int) -> bool:
-    """Whether ``linear`` wants packed activations for this weight and this many rows (see ``SKINNY_TALL_ROWS``)."""
-    return (weight.packed is not None and SKINNY_ROWS < rows <= SKINNY_TALL_ROWS
-            and weight.in_features >= 4 * weight.out_features and weight.in_features % 32 == 0)
+SKINNY_ROWS = 16        # up to this many rows gemm_skinny beats the library on MI355X for every weight
+MEDIUM_ROWS = 64        # and up to this many gemm_medium does, except for
+MEDIUM_WIDE_TILES = 2048   # weights with this many tiles of 16 rows or more (gate/up, the head), where the
+MEDIUM_WIDE_ROWS = 40      # library is as fast from about this many rows on
 
 
 def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None, gated: bool = False,
-           rows: Optional[int] = None) -> torch.Tensor:
+           partials: bool = False) -> torch.Tensor:
     """``x @ W.T`` with float32 accumulation; the result has ``out_dtype`` (default: x's).
 
     With ``gated`` the weight's rows are [gate; up] and the result is ``silu(gate) * up`` of half the
-    width, in x's dtype. ``x`` may come in the streaming kernel's piece order (5 dimensions) with ``rows`` real rows.
+    width, in x's dtype. With ``partials`` a float32 result may come as ``[parts, rows, out]``: sums over
+    ranges of ``in`` that the caller adds in order (the norms and ``qkv_rope_store`` do).
     """
     if isinstance(weight, torch.Tensor):
         weight = Weight(weight, pack=False)
@@ -63,14 +60,17 @@ def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None, gat
         return y if out_dtype == torch.float32 else y.to(out_dtype)
     if x.dtype != w.dtype:
         raise TypeError(f"cannot multiply {x.dtype} activations with a {w.dtype} weight")
-    if x.dim() == 5:      # activations in piece order, made for streams_tall(weight, rows)
-        return kernels.gemm_skinny(x, weight.packed, weight.out_features, "bf16" if out_dtype == torch.bfloat16 else "f32",
-                                   rows=rows)
     rows = x.shape[0]
     if weight.packed is not None and rows <= SKINNY_ROWS:
         if gated:
             return kernels.gemm_skinny(x, weight.packed, weight.out_features, "gated")
         return kernels.gemm_skinny(x, weight.packed, weight.out_features, "bf16" if out_dtype == torch.bfloat16 else "f32")
+    wide = -(-weight.out_features // 16) >= MEDIUM_WIDE_TILES
+    if weight.packed is not None and not gated and rows <= (MEDIUM_WIDE_ROWS if wide else MEDIUM_ROWS):
+        if out_dtype == torch.float32:
+            plan = kernels.medium_plan(weight.out_features, weight.in_features, may_split=partials)
+            return kernels.gemm_medium(x, weight.packed, weight.out_features, "f32", plan=plan)
+        return kernels.gemm_medium(x, weight.packed, weight.out_features, "bf16")
     if gated:
         return kernels.silu_mul(kernels.gemm_bf16(x, w, torch.bfloat16))
     return kernels.gemm_bf16(x, w, out_dtype)

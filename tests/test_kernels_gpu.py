@@ -319,10 +319,6 @@ def test_silu_mul(dtype, width):
     out = kernels().silu_mul(gate_up)
     expected = plain.silu(reference[:, :width]) * reference[:, width:]
     np.testing.assert_allclose(out.float().cpu().numpy(), expected, **tolerance(dtype))
-    if dtype == torch.bfloat16 and width % 32 == 0:
-        packed = kernels().silu_mul(gate_up, packed=True)       # the same numbers in the streaming product's piece order
-        rows = packed.permute(0, 3, 1, 2, 4).reshape(-1, width)[:out.shape[0]]
-        assert torch.equal(rows, out)
     vector = kernels().silu_mul(torch.tensor([[-1.0, 0.0, 1.0, 2.0, 2.0, 2.0]], device=DEVICE)).cpu().numpy()[0]
     np.testing.assert_allclose(vector, [-2 / (1 + math.e), 0.0, 2 / (1 + math.exp(-1))], rtol=1e-6)   # ops_test.cpp:487-495
 
@@ -425,8 +421,6 @@ def test_gemm_skinny(m, n, k):
     assert np.abs(full.double().cpu().numpy() - expected).max() <= 1e-5 * scale
     out = ka.gemm_skinny(a, packed, n, "bf16")
     assert out.dtype == torch.bfloat16 and np.abs(out.float().cpu().numpy() - expected).max() <= 5e-3 * scale
-    # activations given in the weight's piece order give the same numbers
-    assert torch.equal(ka.gemm_skinny(ka.pack_weight(a), packed, n, "f32", rows=m), full)
     # the same in every run, and a row's result does not depend on the other rows of the call
     assert torch.equal(ka.gemm_skinny(a, packed, n, "f32"), full)
     alone = ka.gemm_skinny(a[m - 1:m].contiguous(), packed, n, "f32")
@@ -445,17 +439,77 @@ def test_gemm_skinny_gated_epilogue(m, width, k):
     np.testing.assert_allclose(out.float().cpu().numpy(), expected, rtol=1.2e-2, atol=1.2e-2 * np.abs(expected).max())
 
 
-def test_consumers_add_partial_sums_in_order():
+@pytest.mark.parametrize("m", [17, 33, 40, 64, 5])
+@pytest.mark.parametrize("n,k", [(331, 120), (1000, 200), (4608, 3584), (176, 24), (3584, 18944), (40000, 256), (896, 4864)])
+def test_gemm_medium(m, n, k):
+    rng = np.random.default_rng(m * 11 + n)
+    a_ref, a = to_bf16_exact(rng.normal(size=(m, k)))
+    w_ref, w = to_bf16_exact(rng.normal(size=(n, k)) * 0.1)
+    ka = kernels()
+    packed = ka.pack_weight(w)
+    expected = a_ref @ w_ref.T
+    scale = np.abs(expected).max()
+    parts = ka.gemm_medium(a, packed, n, "f32")                # its own plan: may split k
+    tiles, waves, splits = ka.medium_plan(n, k)
+    assert parts.dtype == torch.float32 and tuple(parts.shape) == ((splits, m, n) if splits > 1 else (m, n))
+    total = parts.double().sum(dim=0) if splits > 1 else parts.double()
+    assert np.abs(total.cpu().numpy() - expected).max() <= 1e-5 * scale
+    whole = ka.gemm_medium(a, packed, n, "f32", plan=ka.medium_plan(n, k, may_split=False))
+    assert tuple(whole.shape) == (m, n) and np.abs(whole.double().cpu().numpy() - expected).max() <= 1e-5 * scale
+    out = ka.gemm_medium(a, packed, n, "bf16")
+    assert out.dtype == torch.bfloat16 and np.abs(out.float().cpu().numpy() - expected).max() <= 5e-3 * scale
+    # every plan the kernel takes gives the product
+    for plan in ((1, 4, 1), (2, 4, 3), (2, 8, 2), (1, 8, 64)):
+        other = ka.gemm_medium(a, packed, n, "f32", plan=plan)
+        other = other.double().sum(dim=0) if other.dim() == 3 else other.double()
+        assert np.abs(other.cpu().numpy() - expected).max() <= 1e-5 * scale, plan
+    # the same in every run, and a row's result does not depend on the other rows of the call
+    assert torch.equal(ka.gemm_medium(a, packed, n, "f32"), parts)
+    alone = ka.gemm_medium(a[m - 1:m].contiguous(), packed, n, "f32")
+    assert torch.equal(alone[..., 0, :], parts[..., m - 1, :])
+
+
+@pytest.mark.parametrize("m,width,k", [(20, 203, 96), (64, 176, 64), (33, 1000, 520)])
+def test_gemm_medium_gated_epilogue(m, width, k):
+    rng = np.random.default_rng(width + 1)
+    a_ref, a = to_bf16_exact(rng.normal(size=(m, k)))
+    w_ref, w = to_bf16_exact(rng.normal(size=(2 * width, k)) * 0.2)      # rows: [gate; up]
+    packed = kernels().pack_weight(w, interleave_halves=True)
+    out = kernels().gemm_medium(a, packed, 2 * width, "gated")
+    expected = plain.silu(a_ref @ w_ref[:width].T) * (a_ref @ w_ref[width:].T)
+    assert out.shape == (m, width)
+    np.testing.assert_allclose(out.float().cpu().numpy(), expected, rtol=1.2e-2, atol=1.2e-2 * np.abs(expected).max())
+
+
+def test_gemm_medium_refuses_what_it_cannot_do():
+    ka = kernels()
+    a = torch.zeros((65, 64), dtype=torch.bfloat16, device=DEVICE)
+    packed = ka.pack_weight(torch.zeros((32, 64), dtype=torch.bfloat16, device=DEVICE))
+    with pytest.raises(Exception, match="at most 64 rows"):
+        ka.gemm_medium(a, packed, 32)
+    with pytest.raises(Exception, match="split"):
+        ka.gemm_medium(a[:20], packed, 32, "bf16", plan=(1, 8, 2))
+    with pytest.raises(Exception, match="4 or 8 waves"):
+        ka.gemm_medium(a[:20], packed, 32, "f32", plan=(1, 16, 1))
+
+
+@pytest.mark.parametrize("width", [120, 203, 3584, 5000])
+def test_consumers_add_partial_sums_in_order(width):
     rng = np.random.default_rng(3)
     k = kernels()
-    h_ref = rng.normal(size=(5, 120)).astype(np.float32)
-    parts = rng.normal(size=(4, 5, 120)).astype(np.float32)
-    weight = np.ones(120, dtype=np.float32)
+    h_ref = rng.normal(size=(5, width)).astype(np.float32)
+    parts = rng.normal(size=(4, 5, width)).astype(np.float32)
+    weight = np.ones(width, dtype=np.float32)
     h = torch.from_numpy(h_ref.copy()).to(DEVICE)
     out = k.rms_norm(h, torch.from_numpy(weight).to(DEVICE), 1e-5, torch.float32, delta=torch.from_numpy(parts).to(DEVICE), write_h=True)
     total = h_ref.astype(np.float64) + parts.astype(np.float64).sum(axis=0)
     np.testing.assert_allclose(h.cpu().numpy(), total, rtol=1e-6, atol=1e-6)
     np.testing.assert_allclose(out.cpu().numpy(), plain.rms_norm(total, weight, 1e-5), rtol=1e-5, atol=1e-5)
+    picked = torch.tensor([3, 1], dtype=torch.int32, device=DEVICE)      # chosen rows, the stream left as it is
+    h = torch.from_numpy(h_ref.copy()).to(DEVICE)
+    some = k.rms_norm(h, torch.from_numpy(weight).to(DEVICE), 1e-5, torch.float32, delta=torch.from_numpy(parts).to(DEVICE), rows=picked)
+    np.testing.assert_allclose(some.cpu().numpy(), plain.rms_norm(total[[3, 1]], weight, 1e-5), rtol=1e-5, atol=1e-5)
+    assert torch.equal(h.cpu(), torch.from_numpy(h_ref))
     heads, kv_heads, hd = 3, 1, 16
     qkv_parts = rng.normal(size=(3, 6, (heads + 2 * kv_heads) * hd)).astype(np.float32)
     positions = torch.arange(6, dtype=torch.int32, device=DEVICE)
