@@ -63,7 +63,7 @@ def main() -> int:
     achieved = bytes_step / (main_result["ms_per_step"] * 1e-3) / 1e9
 
     line = {
-        "metric": "decode tok/s (ctx 4096) Qwen2-7B bf16",
+        "metric": f"decode tok/s (ctx {args.context}) Qwen2-7B {'bf16' if args.dtype == 'bfloat16' else 'fp32'}",
         "value": round(main_result["tokens_per_second"], 2),
         "unit": "tok/s",
         "n_gpus": 1,

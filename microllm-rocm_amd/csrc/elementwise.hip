@@ -157,9 +157,18 @@ __global__ void residual_add_kernel(float* __restrict__ h, const T* __restrict__
 }
 
 // ---------------------------------------------------------------------------------------------
-// One block per token. Angles are position * inv_freq in float64, so cos and sin are the
-// correctly rounded float32 values for any position; they are computed once per token into LDS
-// and shared by all heads.
+// cos and sin of position * inv_freq for every token of a step: angles in float64, so that the float32 values
+// are the correctly rounded ones for any position. out[token][pair] = (cos, sin).
+__global__ void rope_table_kernel(const int32_t* __restrict__ positions, const double* __restrict__ inv_freq,
+                                  int n_freq, int64_t count, float2* __restrict__ out) {
+    const int64_t index = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (index >= count) return;
+    const double angle = static_cast<double>(positions[index / n_freq]) * inv_freq[index % n_freq];
+    out[index] = make_float2(static_cast<float>(cos(angle)), static_cast<float>(sin(angle)));
+}
+
+// One block per token (and group of heads). cos and sin come from the step's table, or are computed here
+// the same way; they are put into LDS once and shared by the block's heads.
 constexpr int kMaxHeadDim = 512;
 
 template <typename In, typename T>
@@ -167,9 +176,9 @@ __global__ void qkv_rope_store_kernel(const In* __restrict__ qkv, int n_partials
                                       const float* __restrict__ bias,
                                       const int32_t* __restrict__ positions,
                                       const int32_t* __restrict__ slot_mapping,
-                                      const double* __restrict__ inv_freq, int n_freq,
+                                      const double* __restrict__ inv_freq, const float2* __restrict__ cos_sin, int n_freq,
                                       T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                      int heads, int kv_heads, int head_dim, int page_size) {
+                                      int heads, int kv_heads, int head_dim, int page_size, int pair_order) {
     __shared__ float cos_table[kMaxHeadDim / 2];
     __shared__ float sin_table[kMaxHeadDim / 2];
     const int token = blockIdx.x;
@@ -177,9 +186,15 @@ __global__ void qkv_rope_store_kernel(const In* __restrict__ qkv, int n_partials
     const int heads_per_block = gridDim.y == 1 ? heads + 2 * kv_heads : max(1, static_cast<int>(blockDim.x) / (head_dim / 2));
     const int first_head = blockIdx.y * heads_per_block;
     for (int index = threadIdx.x; index < n_freq; index += blockDim.x) {
-        const double angle = static_cast<double>(position) * inv_freq[index];
-        cos_table[index] = static_cast<float>(cos(angle));
-        sin_table[index] = static_cast<float>(sin(angle));
+        if (cos_sin) {
+            const float2 both = cos_sin[static_cast<int64_t>(token) * n_freq + index];
+            cos_table[index] = both.x;
+            sin_table[index] = both.y;
+        } else {
+            const double angle = static_cast<double>(position) * inv_freq[index];
+            cos_table[index] = static_cast<float>(cos(angle));
+            sin_table[index] = static_cast<float>(sin(angle));
+        }
     }
     __syncthreads();
 
@@ -208,11 +223,14 @@ __global__ void qkv_rope_store_kernel(const In* __restrict__ qkv, int n_partials
             rotate = false;
         }
         const int column = head * head_dim;
-        float x1 = to_float(qkv[in_row + column + first]);
-        float x2 = to_float(qkv[in_row + column + second]);
+        // With pair_order the input's query and key heads hold the two dims of a rotary pair side by side.
+        const bool paired = pair_order && !is_value && pair < n_freq;
+        const int in_first = paired ? 2 * pair : first, in_second = paired ? 2 * pair + 1 : second;
+        float x1 = to_float(qkv[in_row + column + in_first]);
+        float x2 = to_float(qkv[in_row + column + in_second]);
         for (int part = 1; part < n_partials; ++part) {
-            x1 += to_float(qkv[part * partial_stride + in_row + column + first]);
-            x2 += to_float(qkv[part * partial_stride + in_row + column + second]);
+            x1 += to_float(qkv[part * partial_stride + in_row + column + in_first]);
+            x2 += to_float(qkv[part * partial_stride + in_row + column + in_second]);
         }
         if (bias) {
             x1 += bias[column + first];
@@ -337,15 +355,16 @@ int mll_residual_add(float* h, const void* delta, int dtype, int n_rows, int wid
 
 int mll_qkv_rope_store(const void* qkv, int in_dtype, int n_partials, int64_t partial_stride, int dtype,
                        const float* bias, const int32_t* positions,
-                       const int32_t* slot_mapping, const double* inv_freq, int n_freq,
+                       const int32_t* slot_mapping, const double* inv_freq, const void* cos_sin, int n_freq,
                        void* q_out, void* k_cache, void* v_cache,
-                       int n_tokens, int heads, int kv_heads, int head_dim, int page_size,
+                       int n_tokens, int heads, int kv_heads, int head_dim, int page_size, int pair_order,
                        hipStream_t stream) {
     MLL_REQUIRE(heads > 0 && kv_heads >= 0 && head_dim > 0, "qkv_rope_store: sizes must be positive");
     MLL_REQUIRE(n_partials >= 1, "qkv_rope_store: the input needs at least one part");
     MLL_REQUIRE(head_dim % 2 == 0 && head_dim <= kMaxHeadDim, "qkv_rope_store: head_dim must be even and at most 512");
     MLL_REQUIRE(n_freq >= 0 && 2 * n_freq <= head_dim, "qkv_rope_store: rotary part exceeds head_dim");
-    MLL_REQUIRE(inv_freq != nullptr || n_freq == 0, "qkv_rope_store: n_freq without a frequency table");
+    MLL_REQUIRE(inv_freq != nullptr || cos_sin != nullptr || n_freq == 0, "qkv_rope_store: n_freq without frequencies or a table of cos and sin");
+    MLL_REQUIRE(cos_sin == nullptr || reinterpret_cast<uintptr_t>(cos_sin) % 8 == 0, "qkv_rope_store: the table of cos and sin must be 8-byte aligned");
     MLL_REQUIRE(slot_mapping == nullptr || (k_cache && v_cache && page_size > 0 && page_size % 16 == 0),
                 "qkv_rope_store: slot_mapping needs both caches and a page size that is a multiple of 16");
     if (n_tokens == 0) return 0;
@@ -354,23 +373,34 @@ int mll_qkv_rope_store(const void* qkv, int in_dtype, int n_partials, int64_t pa
     const dim3 grid(n_tokens, (heads + 2 * kv_heads + heads_per_block - 1) / heads_per_block);
     if (dtype == kF32 && in_dtype == kF32) {
         qkv_rope_store_kernel<float, float><<<grid, 256, 0, stream>>>(
-            static_cast<const float*>(qkv), n_partials, partial_stride, bias, positions, slot_mapping, inv_freq, n_freq,
+            static_cast<const float*>(qkv), n_partials, partial_stride, bias, positions, slot_mapping, inv_freq, static_cast<const float2*>(cos_sin), n_freq,
             static_cast<float*>(q_out), static_cast<float*>(k_cache), static_cast<float*>(v_cache),
-            heads, kv_heads, head_dim, page_size);
+            heads, kv_heads, head_dim, page_size, pair_order);
     } else if (dtype == kBF16 && in_dtype == kF32) {
         qkv_rope_store_kernel<float, bf16><<<grid, 256, 0, stream>>>(
-            static_cast<const float*>(qkv), n_partials, partial_stride, bias, positions, slot_mapping, inv_freq, n_freq,
+            static_cast<const float*>(qkv), n_partials, partial_stride, bias, positions, slot_mapping, inv_freq, static_cast<const float2*>(cos_sin), n_freq,
             static_cast<bf16*>(q_out), static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache),
-            heads, kv_heads, head_dim, page_size);
+            heads, kv_heads, head_dim, page_size, pair_order);
     } else if (dtype == kBF16 && in_dtype == kBF16) {
         qkv_rope_store_kernel<bf16, bf16><<<grid, 256, 0, stream>>>(
-            static_cast<const bf16*>(qkv), n_partials, partial_stride, bias, positions, slot_mapping, inv_freq, n_freq,
+            static_cast<const bf16*>(qkv), n_partials, partial_stride, bias, positions, slot_mapping, inv_freq, static_cast<const float2*>(cos_sin), n_freq,
             static_cast<bf16*>(q_out), static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache),
-            heads, kv_heads, head_dim, page_size);
+            heads, kv_heads, head_dim, page_size, pair_order);
     } else {
         return fail("qkv_rope_store: unsupported combination of input and output dtypes");
     }
     return check_launch("qkv_rope_store");
+}
+
+int mll_rope_table(const int32_t* positions, const double* inv_freq, int n_freq, int n_tokens, float* out,
+                   hipStream_t stream) {
+    MLL_REQUIRE(n_freq > 0 && n_tokens >= 0, "rope_table: sizes must be positive");
+    MLL_REQUIRE(reinterpret_cast<uintptr_t>(out) % 8 == 0, "rope_table: the table must be 8-byte aligned");
+    if (n_tokens == 0) return 0;
+    const int64_t count = static_cast<int64_t>(n_tokens) * n_freq;
+    rope_table_kernel<<<static_cast<unsigned>((count + 255) / 256), 256, 0, stream>>>(positions, inv_freq, n_freq, count,
+                                                                                      reinterpret_cast<float2*>(out));
+    return check_launch("rope_table");
 }
 
 int mll_silu_mul(const void* gate, const void* up, int64_t in_stride, void* out, int dtype,

@@ -8,6 +8,7 @@
 // A workgroup owns NT tiles of W; its waves (1 to 16, more when W has few rows, so that the GPU is filled)
 // take the k steps in turn and their sums are added in wave order through LDS: the result is the same in
 // every run and does not depend on the other rows of A.
+#include "cache_layout.h"
 #include "common.h"
 #include "microllm_hip.h"
 
@@ -30,12 +31,14 @@ __device__ inline float silu_f(float value) {
 }
 
 // EPILOGUE: 0 = float32 [M, N]; 1 = bfloat16 [M, N]; 2 = bfloat16 [M, N / 2] = silu(even rows of W) * (odd rows).
+// 3 = the q/k/v projection of an attention layer finished in place: bias, rotation of the position, queries to
+// `q_out`, keys and values into their pages (at most 16 rows; see MllQkvStore).
 // TEMPORAL: W is read with ordinary loads instead of non-temporal ones (measured on MI355X: better for weights
 // of a few tens of MB, worse for the large ones).
 template <int MT, int NT, int EPILOGUE, bool TEMPORAL>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w_packed, void* __restrict__ out,
-    int m, int n, int k, int n_tiles, int k_steps) {
+    int m, int n, int k, int n_tiles, int k_steps, MllQkvStore store) {
     extern __shared__ float reduce_shared[];   // [waves][NT * MT][64 lanes][4]
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
@@ -146,12 +149,56 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
                     const int column = n_tile * 16 + quad * 4 + i;
                     if (column < n) target[column] = from_float<bf16>(acc[nt][mt][i]);
                 }
-            } else {
+            } else if (EPILOGUE == 2) {
                 bf16* target = static_cast<bf16*>(out) + static_cast<int64_t>(row) * (n / 2);
 #pragma unroll
                 for (int i = 0; i < 4; i += 2) {
                     const int column = n_tile * 8 + quad * 2 + i / 2;
                     if (column < n / 2) target[column] = from_float<bf16>(silu_f(acc[nt][mt][i]) * acc[nt][mt][i + 1]);
+                }
+            } else {
+                // The lane's 4 columns lie in one head (head_dim is a multiple of 16). In a query or key head the
+                // weight's rows were ordered so that columns 2p and 2p + 1 hold dims p and p + n_freq: the two that
+                // rotate together.
+                const int column = n_tile * 16 + quad * 4;
+                if (column >= n) continue;
+                const int head = column / store.head_dim, within = column % store.head_dim;
+                const bool is_query = head < store.heads;
+                const bool is_value = head >= store.heads + store.kv_heads;
+                const int slot = store.slot_mapping ? store.slot_mapping[row] : -1;
+                const CacheLayout layout(store.kv_heads, store.page_size, store.head_dim);
+                bf16* q_row = static_cast<bf16*>(store.q_out) + (static_cast<int64_t>(row) * store.heads + head) * store.head_dim;
+#pragma unroll
+                for (int i = 0; i < 4; i += 2) {
+                    const bool rotate = !is_value && within + i < 2 * store.n_freq;
+                    const int pair = (within + i) / 2;
+                    const int first = rotate ? pair : within + i;
+                    const int second = rotate ? pair + store.n_freq : within + i + 1;
+                    float x1 = acc[nt][mt][i], x2 = acc[nt][mt][i + 1];
+                    if (store.bias) {
+                        x1 += store.bias[head * store.head_dim + first];
+                        x2 += store.bias[head * store.head_dim + second];
+                    }
+                    float y1 = x1, y2 = x2;
+                    if (rotate) {
+                        const float2 both = reinterpret_cast<const float2*>(store.cos_sin)[static_cast<int64_t>(row) * store.n_freq + pair];
+                        const float c = both.x, sn = both.y;
+                        y1 = x1 * c - x2 * sn;
+                        y2 = x1 * sn + x2 * c;
+                    }
+                    if (is_query) {
+                        q_row[first] = from_float<bf16>(y1);
+                        q_row[second] = from_float<bf16>(y2);
+                    } else if (slot >= 0 && !is_value) {
+                        bf16* pages = static_cast<bf16*>(store.k_cache);
+                        pages[layout.k_at(slot / store.page_size, head - store.heads, slot % store.page_size, first)] = from_float<bf16>(y1);
+                        pages[layout.k_at(slot / store.page_size, head - store.heads, slot % store.page_size, second)] = from_float<bf16>(y2);
+                    } else if (slot >= 0) {
+                        bf16* pages = static_cast<bf16*>(store.v_cache);
+                        const int kv_head = head - store.heads - store.kv_heads;
+                        pages[layout.v_at(slot / store.page_size, kv_head, slot % store.page_size, first)] = from_float<bf16>(y1);
+                        pages[layout.v_at(slot / store.page_size, kv_head, slot % store.page_size, second)] = from_float<bf16>(y2);
+                    }
                 }
             }
         }
@@ -160,7 +207,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
 
 template <int MT, int NT, int EPILOGUE>
 static void launch_one(const bf16* a, const bf16* w, void* out, int m, int n, int k, int n_tiles,
-                       int k_steps, hipStream_t stream) {
+                       int k_steps, const MllQkvStore& store, hipStream_t stream) {
     const int groups = (n_tiles + NT - 1) / NT;
     // Waves per workgroup: enough that about eight thousand waves would stream W one tile each, at most 16, and
     // no more than there are chunks of k for them. A function of (n, k) alone, like the split of k it implies.
@@ -169,14 +216,14 @@ static void launch_one(const bf16* a, const bf16* w, void* out, int m, int n, in
     const size_t lds = waves > 1 ? static_cast<size_t>(waves - 1) * NT * MT * kWave * sizeof(floatx4) : 0;
     const bool temporal = static_cast<int64_t>(n_tiles) * k_steps * 1024 < (64ll << 20);   // bytes of the packed weight
     if (temporal)
-        gemm_skinny_kernel<MT, NT, EPILOGUE, true><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps);
+        gemm_skinny_kernel<MT, NT, EPILOGUE, true><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps, store);
     else
-        gemm_skinny_kernel<MT, NT, EPILOGUE, false><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps);
+        gemm_skinny_kernel<MT, NT, EPILOGUE, false><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps, store);
 }
 
 template <int EPILOGUE>
 static int launch_skinny(const void* a, const void* w_packed, void* out, int m, int n, int k,
-                         hipStream_t stream) {
+                         const MllQkvStore& store, hipStream_t stream) {
     const int n_tiles = (n + 15) / 16;
     const int k_steps = (k + 31) / 32;
     const bf16* a_ = static_cast<const bf16*>(a);
@@ -186,17 +233,23 @@ static int launch_skinny(const void* a, const void* w_packed, void* out, int m, 
     // least 128 workgroups left: two, so that every piece of A is used twice (all measured on MI355X; four tiles
     // a workgroup were slower).
     const bool wide = n_tiles >= 2048;
+    if constexpr (EPILOGUE == 3) {
+        if (m_tiles != 1) return fail("gemm_skinny: the q/k/v epilogue takes at most 16 rows");
+        if (m > 4 && n_tiles >= 256) launch_one<1, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, store, stream);
+        else launch_one<1, 1, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, store, stream);
+        return check_launch("gemm_skinny");
+    }
     switch (m_tiles) {
         case 1:
-            if (wide || (m > 4 && n_tiles >= 256)) launch_one<1, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream);
-            else launch_one<1, 1, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream);
+            if (wide || (m > 4 && n_tiles >= 256)) launch_one<1, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, store, stream);
+            else launch_one<1, 1, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, store, stream);
             break;
         case 2:
-            if (wide) launch_one<2, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream);
-            else launch_one<2, 1, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream);
+            if (wide) launch_one<2, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, store, stream);
+            else launch_one<2, 1, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, store, stream);
             break;
-        case 3: launch_one<3, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream); break;
-        case 4: launch_one<4, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, stream); break;
+        case 3: launch_one<3, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, store, stream); break;
+        case 4: launch_one<4, 2, EPILOGUE>(a_, w_, out, m, n, k, n_tiles, k_steps, store, stream); break;
         default: return fail("gemm_skinny: more than 64 rows");
     }
     return check_launch("gemm_skinny");
@@ -213,9 +266,26 @@ extern "C" int mll_gemm_skinny(const void* a, const void* w_packed, void* out, i
     MLL_REQUIRE(epilogue != 2 || n % 2 == 0, "gemm_skinny: the gated epilogue needs an even number of weight rows");
     if (m == 0) return 0;
     switch (epilogue) {
-        case 0: return launch_skinny<0>(a, w_packed, out, m, n, k, stream);
-        case 1: return launch_skinny<1>(a, w_packed, out, m, n, k, stream);
-        case 2: return launch_skinny<2>(a, w_packed, out, m, n, k, stream);
+        case 0: return launch_skinny<0>(a, w_packed, out, m, n, k, MllQkvStore{}, stream);
+        case 1: return launch_skinny<1>(a, w_packed, out, m, n, k, MllQkvStore{}, stream);
+        case 2: return launch_skinny<2>(a, w_packed, out, m, n, k, MllQkvStore{}, stream);
         default: return fail("gemm_skinny: unknown epilogue");
     }
+}
+
+extern "C" int mll_gemm_skinny_qkv(const void* a, const void* w_packed, int m, int k, const MllQkvStore* store,
+                                   hipStream_t stream) {
+    MLL_REQUIRE(store != nullptr, "gemm_skinny_qkv: no epilogue description");
+    MLL_REQUIRE(m >= 0 && m <= 16, "gemm_skinny_qkv: takes at most 16 rows");
+    MLL_REQUIRE(k > 0 && k % 8 == 0, "gemm_skinny_qkv: k must be a positive multiple of 8");
+    MLL_REQUIRE(store->heads > 0 && store->kv_heads >= 0, "gemm_skinny_qkv: bad head counts");
+    MLL_REQUIRE(store->head_dim >= 16 && store->head_dim % 16 == 0, "gemm_skinny_qkv: head_dim must be a multiple of 16");
+    MLL_REQUIRE(store->n_freq >= 0 && 2 * store->n_freq <= store->head_dim, "gemm_skinny_qkv: more rotary pairs than dims");
+    MLL_REQUIRE(store->n_freq == 0 || store->cos_sin, "gemm_skinny_qkv: rotation needs the table of cos and sin");
+    MLL_REQUIRE(store->q_out, "gemm_skinny_qkv: the query output is needed");
+    MLL_REQUIRE(!store->slot_mapping || (store->k_cache && store->v_cache && store->page_size > 0 && store->page_size % 16 == 0),
+                "gemm_skinny_qkv: writing pages needs both caches and a page size that is a multiple of 16");
+    if (m == 0) return 0;
+    const int n = (store->heads + 2 * store->kv_heads) * store->head_dim;
+    return launch_skinny<3>(a, w_packed, nullptr, m, n, k, *store, stream);
 }

@@ -29,19 +29,24 @@ int mll_rms_norm(float* h, const void* delta, int delta_dtype, int n_partials, i
 // Adds a pending delta into the residual stream: h[r] += delta[r] for all rows.
 int mll_residual_add(float* h, const void* delta, int dtype, int n_rows, int width, hipStream_t stream);
 
+// out[t][i] = (cos, sin) of positions[t] * inv_freq[i], the angle in float64: float32 [n_tokens][n_freq][2].
+int mll_rope_table(const int32_t* positions, const double* inv_freq, int n_freq, int n_tokens, float* out,
+                   hipStream_t stream);
+
 // Splits fused projections qkv[t] = [q (H*hd) | k (KVH*hd) | v (KVH*hd)], adds `bias` (nullable),
-// rotates q and k by the split-half rule with angle position * inv_freq[i] in float64 (inv_freq nullable:
-// no rotation; rotary_dim = 2 * n_freq <= hd), writes q to q_out[t] and k, v into the pages:
-// slot = slot_mapping[t] (negative: not stored) addresses key pages [page, kv_head, offset, dim] and
-// value pages [page, kv_head, dim, offset] (transposed, so that a dim's keys are contiguous) with
-// page = slot / page_size, offset = slot % page_size.  k_cache / v_cache nullable together with slot_mapping. qkv has element type
+// rotates q and k by the split-half rule with angle position * inv_freq[i] in float64, or with the cos and sin
+// of mll_rope_table's `cos_sin` if that is given (both null: no rotation; rotary_dim = 2 * n_freq <= hd), writes q to q_out[t] and k, v into the pages (laid out as
+// cache_layout.h says): slot = slot_mapping[t] (negative: not stored), page = slot / page_size,
+// offset = slot % page_size. k_cache / v_cache nullable together with slot_mapping. qkv has element type
 // `in_dtype` (float32, or the same as `dtype`) and may come in n_partials parts, partial_stride elements
-// apart, which are added in order; q_out and the pages have `dtype`.
+// apart, which are added in order; q_out and the pages have `dtype`. With pair_order the query and key heads
+// of qkv hold dims p and p + n_freq side by side (columns 2p, 2p + 1), as a weight in rotary pair order gives
+// them (see MllQkvStore); bias and outputs are in the ordinary order.
 int mll_qkv_rope_store(const void* qkv, int in_dtype, int n_partials, int64_t partial_stride, int dtype,
                        const float* bias, const int32_t* positions,
-                       const int32_t* slot_mapping, const double* inv_freq, int n_freq,
+                       const int32_t* slot_mapping, const double* inv_freq, const void* cos_sin, int n_freq,
                        void* q_out, void* k_cache, void* v_cache,
-                       int n_tokens, int heads, int kv_heads, int head_dim, int page_size,
+                       int n_tokens, int heads, int kv_heads, int head_dim, int page_size, int pair_order,
                        hipStream_t stream);
 
 // Attention of every query token over its request's pages, one wave per (token, head).
@@ -80,6 +85,25 @@ int mll_gemm_f32(const float* a, const float* w, const float* bias, float* c,
 // other rows of A.
 int mll_gemm_skinny(const void* a, const void* w_packed, void* out, int epilogue, int m, int n, int k,
                     hipStream_t stream);
+
+// What the q/k/v projection's product does with its result instead of writing it out: the work of
+// mll_qkv_rope_store. The packed weight's rows must be in rotary pair order: in every query and key head, row
+// 2p holds dim p and row 2p + 1 dim p + n_freq for p < n_freq, the other dims follow in place; value heads are
+// as they are. bias (float32, may be null) and the outputs are in the ordinary order.
+struct MllQkvStore {
+    const float* bias;
+    const int32_t* slot_mapping;   // [m] page * page_size + offset, or null: keys and values are not kept
+    const float* cos_sin;          // [m][n_freq][2]: mll_rope_table's
+    int n_freq;
+    void* q_out;                   // bfloat16 [m, heads * head_dim]
+    void* k_cache;                 // bfloat16 pages
+    void* v_cache;
+    int heads, kv_heads, head_dim, page_size;
+};
+// Queries, keys and values of at most 16 rows: A [m, k] . W^T with n = (heads + 2 kv_heads) * head_dim, finished
+// as `store` says.
+int mll_gemm_skinny_qkv(const void* a, const void* w_packed, int m, int k, const MllQkvStore* store,
+                        hipStream_t stream);
 
 // The same product for up to 64 rows with the activations shared through LDS by the waves of a workgroup
 // (faster than mll_gemm_skinny from 17 rows on). A wave takes tiles_per_wave (1 or 2) tiles of W. With

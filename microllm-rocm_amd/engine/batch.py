@@ -60,6 +60,8 @@ class StepContext:
     max_total: int = 0
     planned_total: int = 0      # the longest request this step's launch shapes are planned for (>= max_total)
     max_single_total: int = 0   # the longest of the requests listed in single_tokens
+    # what a part computes once for the step and its likes in other layers take from here (key: the part's choice)
+    memo: dict = field(default_factory=dict)
 
 
 class BatchBuilder:

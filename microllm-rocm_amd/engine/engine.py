@@ -139,6 +139,7 @@ class Engine:
             # the same keys and values to the same slots each time, so running it twice changes nothing.
             self.model.forward(ctx, self._bindings, ctx.want_rows)
             torch.cuda.synchronize(self.device)
+            ctx.memo.clear()     # what the parts computed once for the step is computed inside the graph too
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 state.logits = self.model.forward(ctx, self._bindings, ctx.want_rows)

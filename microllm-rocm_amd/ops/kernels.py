@@ -109,14 +109,28 @@ def residual_add(h: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
     return h
 
 
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """``[tokens, n_freq, 2]`` float32: cos and sin of ``position * inv_freq``, the angle taken in float64."""
+    lib = library.load()
+    _device_tensor(positions, "positions", torch.int32)
+    _device_tensor(inv_freq, "inverse frequencies", torch.float64)
+    _need(positions.dim() == 1 and inv_freq.dim() == 1 and inv_freq.shape[0] > 0, "rope_table takes [tokens] and [n_freq]")
+    out = torch.empty((positions.shape[0], inv_freq.shape[0], 2), dtype=torch.float32, device=positions.device)
+    _check(lib.mll_rope_table(_ptr(positions), _ptr(inv_freq), inv_freq.shape[0], positions.shape[0], _ptr(out), _stream()), lib)
+    return out
+
+
 def qkv_rope_store(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
                    slot_mapping: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor],
                    k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
                    heads: int, kv_heads: int, head_dim: int, page_size: int, out_dtype: torch.dtype,
-                   q_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   q_out: Optional[torch.Tensor] = None, pair_order: bool = False,
+                   cos_sin: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Bias, rotation and page write of fused projections ``[tokens, (heads + 2 kv_heads) * head_dim]``.
 
-    ``qkv`` is float32 or ``out_dtype``; the rotated queries and the pages have ``out_dtype``."""
+    ``qkv`` is float32 or ``out_dtype``; the rotated queries and the pages have ``out_dtype``. The rotation
+    takes ``cos_sin`` (``rope_table``'s, for these tokens) or computes the same from ``inv_freq``. With
+    ``pair_order`` the query and key heads of ``qkv`` come in ``rotary_pair_order``."""
     lib = library.load()
     _device_tensor(qkv, "qkv")
     _need(qkv.dtype in (torch.float32, out_dtype), "qkv must be float32 or have the output's dtype")
@@ -136,6 +150,11 @@ def qkv_rope_store(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: t
     if inv_freq is not None:
         _device_tensor(inv_freq, "inverse frequencies", torch.float64)
         n_freq = inv_freq.shape[0]
+    if cos_sin is not None:
+        _device_tensor(cos_sin, "cos/sin table", torch.float32)
+        _need(cos_sin.dim() == 3 and cos_sin.shape[0] == n_tokens and cos_sin.shape[2] == 2, "the cos/sin table must be [tokens, n_freq, 2]")
+        _need(inv_freq is None or cos_sin.shape[1] == n_freq, "the cos/sin table and inv_freq differ in size")
+        n_freq = cos_sin.shape[1]
     if slot_mapping is not None:
         _device_tensor(slot_mapping, "slot mapping", torch.int32)
         _need(tuple(slot_mapping.shape) == (n_tokens,), "slot mapping must hold one entry per token")
@@ -147,8 +166,69 @@ def qkv_rope_store(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: t
     _need(tuple(q_out.shape) == (n_tokens, heads * head_dim), "q output has the wrong shape")
     _check(lib.mll_qkv_rope_store(_ptr(qkv), _code(qkv.dtype), n_partials, ctypes.c_int64(n_tokens * total),
                                   _code(out_dtype), _ptr(bias), _ptr(positions), _ptr(slot_mapping),
-                                  _ptr(inv_freq), n_freq, _ptr(q_out), _ptr(k_cache), _ptr(v_cache),
-                                  n_tokens, heads, kv_heads, head_dim, page_size, _stream()), lib)
+                                  _ptr(inv_freq), _ptr(cos_sin), n_freq, _ptr(q_out), _ptr(k_cache), _ptr(v_cache),
+                                  n_tokens, heads, kv_heads, head_dim, page_size, int(pair_order), _stream()), lib)
+    return q_out
+
+
+def rotary_pair_order(heads: int, kv_heads: int, head_dim: int, n_freq: int) -> torch.Tensor:
+    """Row order of a stacked q/k/v weight that puts the two dims of a rotary pair side by side.
+
+    In every query and key head rows ``2p`` and ``2p + 1`` become dims ``p`` and ``p + n_freq`` for
+    ``p < n_freq``; the dims beyond the rotary part and the value heads stay where they are. Returns the
+    old row of every new row."""
+    _need(0 <= 2 * n_freq <= head_dim, "more rotary pairs than dims")
+    within = torch.arange(head_dim)
+    pairs = torch.stack([torch.arange(n_freq), torch.arange(n_freq) + n_freq], dim=1).reshape(-1)
+    within[: 2 * n_freq] = pairs
+    rows = []
+    for head in range(heads + 2 * kv_heads):
+        rotated = head < heads + kv_heads
+        rows.append(head * head_dim + (within if rotated else torch.arange(head_dim)))
+    return torch.cat(rows)
+
+
+class _QkvStore(ctypes.Structure):
+    _fields_ = [("bias", ctypes.c_void_p), ("slot_mapping", ctypes.c_void_p),
+                ("cos_sin", ctypes.c_void_p), ("n_freq", ctypes.c_int), ("q_out", ctypes.c_void_p),
+                ("k_cache", ctypes.c_void_p), ("v_cache", ctypes.c_void_p), ("heads", ctypes.c_int),
+                ("kv_heads", ctypes.c_int), ("head_dim", ctypes.c_int), ("page_size", ctypes.c_int)]
+
+
+def gemm_skinny_qkv(x: torch.Tensor, packed: torch.Tensor, bias: Optional[torch.Tensor],
+                    slot_mapping: Optional[torch.Tensor], cos_sin: Optional[torch.Tensor],
+                    k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                    heads: int, kv_heads: int, head_dim: int, page_size: int) -> torch.Tensor:
+    """Queries, keys and values of at most 16 bfloat16 rows in one kernel: ``gemm_skinny`` finished by the work
+    of ``qkv_rope_store``. ``packed`` is the stacked weight packed in ``rotary_pair_order``; ``cos_sin`` is
+    ``rope_table``'s for these rows (none: no rotation). Returns the queries."""
+    lib = library.load()
+    _device_tensor(x, "gemm input", torch.bfloat16)
+    _device_tensor(packed, "packed weight", torch.bfloat16)
+    _need(x.dim() == 2 and x.shape[0] <= 16, "gemm_skinny_qkv takes [m <= 16, k] activations")
+    m, k = x.shape
+    total = (heads + 2 * kv_heads) * head_dim
+    _need(k % 8 == 0 and head_dim % 16 == 0, "gemm_skinny_qkv needs k % 8 == 0 and head_dim % 16 == 0")
+    _need(packed.dim() == 5 and tuple(packed.shape[2:]) == (4, 16, 8) and packed.shape[0] == total // 16
+          and packed.shape[1] == -(-k // 32), "the packed weight does not fit the heads and k")
+    if bias is not None:
+        _device_tensor(bias, "qkv bias", torch.float32)
+        _need(tuple(bias.shape) == (total,), "qkv bias has the wrong size")
+    n_freq = 0
+    if cos_sin is not None:
+        _device_tensor(cos_sin, "cos/sin table", torch.float32)
+        _need(cos_sin.dim() == 3 and cos_sin.shape[0] == m and cos_sin.shape[2] == 2, "the cos/sin table must be [rows, n_freq, 2]")
+        n_freq = cos_sin.shape[1]
+        _need(2 * n_freq <= head_dim, "more rotary pairs than dims")
+    if slot_mapping is not None:
+        _device_tensor(slot_mapping, "slot mapping", torch.int32)
+        _need(tuple(slot_mapping.shape) == (m,), "slot mapping must hold one entry per token")
+        _need(k_cache is not None and v_cache is not None, "slot mapping needs both caches")
+        _check_pages(k_cache, v_cache, torch.bfloat16, kv_heads, head_dim, page_size)
+    q_out = torch.empty((m, heads * head_dim), dtype=torch.bfloat16, device=x.device)
+    store = _QkvStore(_ptr(bias), _ptr(slot_mapping), _ptr(cos_sin), n_freq, _ptr(q_out),
+                      _ptr(k_cache), _ptr(v_cache), heads, kv_heads, head_dim, page_size)
+    _check(lib.mll_gemm_skinny_qkv(_ptr(x), _ptr(packed), m, k, ctypes.byref(store), _stream()), lib)
     return q_out
 
 
@@ -383,14 +463,19 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                    scale, window, heads, kv_heads, head_dim)
 
 
-def pack_weight(weight: torch.Tensor, interleave_halves: bool = False) -> torch.Tensor:
+def pack_weight(weight: torch.Tensor, interleave_halves: bool = False,
+                row_order: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The weight ``[n, k]`` in the order ``gemm_skinny`` streams it: ``[n/16, k/32, 4, 16, 8]``, zero padded.
 
     With ``interleave_halves`` rows ``i`` and ``n/2 + i`` become neighbours first (gate and up of a gated
-    feed-forward), which is what the gated epilogue expects.
+    feed-forward), which is what the gated epilogue expects. With ``row_order`` new row ``i`` is old row
+    ``row_order[i]``.
     """
     _need(weight.dim() == 2 and weight.dtype == torch.bfloat16, "pack_weight takes a bfloat16 matrix")
     n, k = weight.shape
+    if row_order is not None:
+        _need(not interleave_halves and tuple(row_order.shape) == (n,), "row_order must name every row once")
+        weight = weight[row_order.to(weight.device)]
     if interleave_halves:
         _need(n % 2 == 0, "interleaving needs an even number of rows")
         weight = torch.stack([weight[: n // 2], weight[n // 2:]], dim=1).reshape(n, k)

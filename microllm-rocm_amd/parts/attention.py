@@ -17,7 +17,7 @@ import torch
 
 from ..ops import kernels
 from .base import MATRIX, Mixer, PagedKVNeed, Runtime, TensorDecl, VECTOR
-from .linear import Weight, linear
+from .linear import SKINNY_ROWS, Weight, linear, takes_packed
 from .registry import build_part, register_part
 from .spec import PartSpec
 
@@ -63,7 +63,13 @@ class PagedAttention(Mixer):
         weights = [tensors[self.name(f"{role}_proj.weight")] for role, _ in self._projections()]
         if len({w.dtype for w in weights}) != 1:
             raise TypeError("the q, k and v weights of one layer must share a dtype to be stacked")
-        self.qkv_weight = Weight(torch.cat(weights, dim=0).contiguous() if len(weights) > 1 else weights[0])
+        # The packed copy of a weight whose heads rotate by the split-half rule holds the two dims of a rotary pair
+        # side by side, so that the product for few rows can rotate and store in its epilogue.
+        order = None
+        if (self.position is None or self.position.fused_split_half) and self.head_dim % 16 == 0:
+            n_freq = self.position.inv_freq.shape[0] if self.position is not None else 0
+            order = kernels.rotary_pair_order(self.heads, self.kv_heads if self.owns_kv else 0, self.head_dim, n_freq)
+        self.qkv_weight = Weight(torch.cat(weights, dim=0).contiguous() if len(weights) > 1 else weights[0], row_order=order)
         if self.qkv_bias:
             biases = [tensors[self.name(f"{role}_proj.bias")] for role, _ in self._projections()]
             self.qkv_bias_vector = torch.cat(biases, dim=0).contiguous() if len(biases) > 1 else biases[0]
@@ -78,23 +84,28 @@ class PagedAttention(Mixer):
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
         view = ctx.paged[cache.group]
         kv_heads = cache.need.kv_heads
-        qkv = linear(x, self.qkv_weight, out_dtype=torch.float32, partials=True)   # rounded once, after bias and rotation
         stored_heads = self.kv_heads if self.owns_kv else 0
         slot_mapping = view.slot_mapping if self.owns_kv else None
         k_pages = cache.k if self.owns_kv else None
         v_pages = cache.v if self.owns_kv else None
         bias = self.qkv_bias_vector
-        inv_freq = None
-        if self.position is not None:
-            if self.position.fused_split_half:
-                inv_freq = self.position.inv_freq
-            else:
+        weight = self.qkv_weight
+        fused = self.position is None or self.position.fused_split_half
+        cos_sin = self.position.table(ctx) if self.position is not None and fused else None
+        pair_order = weight.row_order is not None and x.dtype == weight.dtype and takes_packed(weight, x.shape[0])
+        if pair_order and x.shape[0] <= SKINNY_ROWS:
+            q = kernels.gemm_skinny_qkv(x, weight.packed, bias, slot_mapping, cos_sin, k_pages, v_pages,
+                                        self.heads, stored_heads, self.head_dim, view.page_size)
+        else:
+            qkv = linear(x, weight, out_dtype=torch.float32, partials=fused)   # rounded once, after bias and rotation
+            if not fused:
                 if bias is not None:
                     qkv = qkv + bias
                     bias = None
                 qkv = self.position.apply(qkv, ctx.positions, self.heads, stored_heads, self.head_dim).contiguous()
-        q = kernels.qkv_rope_store(qkv, bias, ctx.positions, slot_mapping, inv_freq, k_pages, v_pages,
-                                   self.heads, stored_heads, self.head_dim, view.page_size, self.runtime.dtype)
+            q = kernels.qkv_rope_store(qkv, bias, ctx.positions, slot_mapping, None, k_pages, v_pages,
+                                       self.heads, stored_heads, self.head_dim, view.page_size, self.runtime.dtype,
+                                       pair_order=pair_order, cos_sin=cos_sin)
         window = int(self.window) if self.window else 0
         o = kernels.paged_attention(q, cache.k, cache.v, view, ctx, self.scale, window,
                                     self.heads, kv_heads, self.head_dim)

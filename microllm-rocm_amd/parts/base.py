@@ -109,7 +109,7 @@ class Norm(Part):
 
 class PositionEncoding(Part):
     category = "position"
-    fused_split_half = False  # True: the mixer's fused kernel applies it from ``inv_freq``
+    fused_split_half = False  # True: the mixer's fused kernels rotate by the split-half rule with ``table(ctx)``'s cos and sin
 
     def apply(self, qkv: torch.Tensor, positions: torch.Tensor, heads: int, kv_heads: int,
               head_dim: int) -> torch.Tensor:

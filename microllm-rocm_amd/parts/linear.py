@@ -20,13 +20,15 @@ from ..ops import kernels
 class Weight:
     """A linear's weight ``[out, in]`` and, for bfloat16, its packed copy."""
 
-    def __init__(self, tensor: torch.Tensor, gated: bool = False, pack: bool = True):
+    def __init__(self, tensor: torch.Tensor, gated: bool = False, pack: bool = True,
+                 row_order: Optional[torch.Tensor] = None):
         self.tensor = tensor
         self.out_features, self.in_features = tensor.shape
         self.gated = gated   # rows are [gate; up]: the packed copy interleaves them for the fused epilogue
+        self.row_order = row_order   # the packed copy's rows in another order: its products' columns come in that order
         self.packed: Optional[torch.Tensor] = None
         if pack and tensor.is_cuda and tensor.dtype == torch.bfloat16 and self.in_features % 8 == 0:
-            self.packed = kernels.pack_weight(tensor, interleave_halves=gated)
+            self.packed = kernels.pack_weight(tensor, interleave_halves=gated, row_order=row_order)
 
     @property
     def dtype(self) -> torch.dtype:
@@ -39,13 +41,24 @@ MEDIUM_WIDE_TILES = 2048   # weights with this many tiles of 16 rows or more (ga
 MEDIUM_WIDE_ROWS = 40      # library is as fast from about this many rows on
 
 
+def takes_packed(weight: "Weight", rows: int, gated: bool = False) -> bool:
+    """Whether ``linear`` multiplies this many rows with the packed copy (whose rows may be in ``row_order``)."""
+    if weight.packed is None:
+        return False
+    if rows <= SKINNY_ROWS:
+        return True
+    wide = -(-weight.out_features // 16) >= MEDIUM_WIDE_TILES
+    return not gated and rows <= (MEDIUM_WIDE_ROWS if wide else MEDIUM_ROWS)
+
+
 def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None, gated: bool = False,
            partials: bool = False) -> torch.Tensor:
     """``x @ W.T`` with float32 accumulation; the result has ``out_dtype`` (default: x's).
 
     With ``gated`` the weight's rows are [gate; up] and the result is ``silu(gate) * up`` of half the
     width, in x's dtype. With ``partials`` a float32 result may come as ``[parts, rows, out]``: sums over
-    ranges of ``in`` that the caller adds in order (the norms and ``qkv_rope_store`` do).
+    ranges of ``in`` that the caller adds in order (the norms and ``qkv_rope_store`` do). For a weight with a
+    ``row_order`` the columns of the result are in that order whenever ``takes_packed`` says so.
     """
     if isinstance(weight, torch.Tensor):
         weight = Weight(weight, pack=False)
@@ -65,8 +78,7 @@ def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None, gat
         if gated:
             return kernels.gemm_skinny(x, weight.packed, weight.out_features, "gated")
         return kernels.gemm_skinny(x, weight.packed, weight.out_features, "bf16" if out_dtype == torch.bfloat16 else "f32")
-    wide = -(-weight.out_features // 16) >= MEDIUM_WIDE_TILES
-    if weight.packed is not None and not gated and rows <= (MEDIUM_WIDE_ROWS if wide else MEDIUM_ROWS):
+    if takes_packed(weight, rows, gated):
         if out_dtype == torch.float32:
             plan = kernels.medium_plan(weight.out_features, weight.in_features, may_split=partials)
             return kernels.gemm_medium(x, weight.packed, weight.out_features, "f32", plan=plan)

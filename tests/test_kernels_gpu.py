@@ -439,6 +439,53 @@ def test_gemm_skinny_gated_epilogue(m, width, k):
     np.testing.assert_allclose(out.float().cpu().numpy(), expected, rtol=1.2e-2, atol=1.2e-2 * np.abs(expected).max())
 
 
+@pytest.mark.parametrize("m", [1, 7, 16])
+@pytest.mark.parametrize("heads,kv_heads,hd,rotary,hidden,bias", [(4, 2, 16, 16, 64, True), (3, 1, 32, 32, 96, True), (28, 4, 128, 128, 512, True),
+                                                                   (5, 5, 48, 24, 40, False), (2, 0, 64, 64, 72, True)])
+def test_gemm_skinny_qkv_is_product_then_rope_store(m, heads, kv_heads, hd, rotary, hidden, bias):
+    """The fused epilogue against the two kernels it replaces: the product in float32, then bias, rotation and page write."""
+    rng = np.random.default_rng(m + heads)
+    ka = kernels()
+    total = (heads + 2 * kv_heads) * hd
+    _, x = to_bf16_exact(rng.normal(size=(m, hidden)))
+    _, w = to_bf16_exact(rng.normal(size=(total, hidden)) * 0.2)
+    b = torch.from_numpy(rng.normal(size=total).astype(np.float32)).to(DEVICE) if bias else None
+    inv_freq = torch.from_numpy(1e4 ** -(np.arange(0, rotary, 2) / rotary)).to(DEVICE)
+    positions = torch.from_numpy(rng.integers(0, 30000, size=m).astype(np.int32)).to(DEVICE)
+    page_size, n_pages = 32, 6
+    slots = torch.from_numpy(rng.permutation(page_size * n_pages)[:m].astype(np.int32)).to(DEVICE) if kv_heads else None
+
+    def pages():
+        if not kv_heads:
+            return None, None
+        from microllm_rocm_amd.cache.layout import key_page_shape, value_page_shape
+        return (torch.zeros(key_page_shape(n_pages, kv_heads, page_size, hd), dtype=torch.bfloat16, device=DEVICE),
+                torch.zeros(value_page_shape(n_pages, kv_heads, page_size, hd), dtype=torch.bfloat16, device=DEVICE))
+
+    k_two, v_two = pages()
+    q_two = ka.qkv_rope_store(ka.gemm_skinny(x, ka.pack_weight(w), total, "f32"), b, positions, slots, inv_freq, k_two, v_two,
+                              heads, kv_heads, hd, page_size, torch.bfloat16)
+    order = ka.rotary_pair_order(heads, kv_heads, hd, rotary // 2)
+    assert sorted(order.tolist()) == list(range(total))
+    packed = ka.pack_weight(w, row_order=order)
+    k_one, v_one = pages()
+    table = ka.rope_table(positions, inv_freq)
+    angles = positions.cpu().numpy().astype(np.float64)[:, None] * inv_freq.cpu().numpy()[None, :]
+    assert np.abs(table.cpu().numpy().astype(np.float64) - np.stack([np.cos(angles), np.sin(angles)], axis=-1)).max() <= 6e-8
+    q_one = ka.gemm_skinny_qkv(x, packed, b, slots, table, k_one, v_one, heads, kv_heads, hd, page_size)
+    assert torch.equal(q_one, q_two)
+    if kv_heads:
+        assert torch.equal(k_one, k_two) and torch.equal(v_one, v_two)
+        assert k_one.float().abs().sum() > 0 and v_one.float().abs().sum() > 0
+    # the unfused kernel reads products whose columns are in pair order
+    k_three, v_three = pages()
+    q_three = ka.qkv_rope_store(ka.gemm_skinny(x, packed, total, "f32"), b, positions, slots, None, k_three, v_three,
+                                heads, kv_heads, hd, page_size, torch.bfloat16, pair_order=True, cos_sin=table)
+    assert torch.equal(q_three, q_two)
+    if kv_heads:
+        assert torch.equal(k_three, k_two) and torch.equal(v_three, v_two)
+
+
 @pytest.mark.parametrize("m", [17, 33, 40, 64, 5])
 @pytest.mark.parametrize("n,k", [(331, 120), (1000, 200), (4608, 3584), (176, 24), (3584, 18944), (40000, 256), (896, 4864)])
 def test_gemm_medium(m, n, k):
