@@ -83,8 +83,17 @@ int mll_gemm_f32(const float* a, const float* w, const float* bias, float* c,
 // epilogue 0: float32 [m, n]; 1: bfloat16 [m, n]; 2: bfloat16 [m, n / 2] = silu(even weight rows' results) *
 // (odd rows' results). The order of additions is fixed by (n, k): the same in every run and whatever the
 // other rows of A.
+// With `scale` (may be null; at most 16 rows) row r of the product is first multiplied by
+// 1 / sqrt(sum_{g < groups} sumsq[r][g] / width + eps): the factor of an RMS norm whose input came without it.
+struct MllRowScale {
+    const float* sumsq;   // [m][stride], 16-byte aligned; the first `groups` of a row count
+    int groups;
+    int stride;           // a multiple of 4
+    int width;
+    float eps;
+};
 int mll_gemm_skinny(const void* a, const void* w_packed, void* out, int epilogue, int m, int n, int k,
-                    hipStream_t stream);
+                    const MllRowScale* scale, hipStream_t stream);
 
 // What the q/k/v projection's product does with its result instead of writing it out: the work of
 // mll_qkv_rope_store. The packed weight's rows must be in rotary pair order: in every query and key head, row
@@ -103,7 +112,27 @@ struct MllQkvStore {
 // Queries, keys and values of at most 16 rows: A [m, k] . W^T with n = (heads + 2 kv_heads) * head_dim, finished
 // as `store` says.
 int mll_gemm_skinny_qkv(const void* a, const void* w_packed, int m, int k, const MllQkvStore* store,
-                        hipStream_t stream);
+                        const MllRowScale* scale, hipStream_t stream);
+
+// The product of at most 16 rows added to the residual stream, and the next RMS norm begun: h += A . W^T;
+// x_out = h * norm_weight (the norm's input without the rows' factors); sumsq_out[r][g] = the sum of h[r]^2 over
+// columns 16 g .. 16 g + 15, g < ceil(n / 16): what MllRowScale takes.
+struct MllResidualNorm {
+    float* h;                  // [m][n]
+    const float* norm_weight;  // [n]
+    void* x_out;               // bfloat16 [m][n]
+    float* sumsq_out;          // [m][sumsq_stride]; the first ceil(n / 16) of a row are written
+    int sumsq_stride;
+};
+int mll_gemm_skinny_residual(const void* a, const void* w_packed, int m, int n, int k, const MllResidualNorm* residual,
+                             const MllRowScale* scale, hipStream_t stream);
+
+// What the kernel takes beside the product's operands (internal to the library's launches).
+struct MllSkinnyExtras {
+    MllQkvStore store;
+    MllRowScale scale;
+    MllResidualNorm residual;
+};
 
 // The same product for up to 64 rows with the activations shared through LDS by the waves of a workgroup
 // (faster than mll_gemm_skinny from 17 rows on). A wave takes tiles_per_wave (1 or 2) tiles of W. With

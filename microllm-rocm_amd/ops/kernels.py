@@ -7,7 +7,7 @@ a kernel never sees operands that do not fit what its grid assumes.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional, Tuple
+from typing import NamedTuple, Optional, Tuple
 
 import torch
 
@@ -188,6 +188,34 @@ def rotary_pair_order(heads: int, kv_heads: int, head_dim: int, n_freq: int) -> 
     return torch.cat(rows)
 
 
+class _RowScale(ctypes.Structure):
+    _fields_ = [("sumsq", ctypes.c_void_p), ("groups", ctypes.c_int), ("stride", ctypes.c_int), ("width", ctypes.c_int),
+                ("eps", ctypes.c_float)]
+
+
+class _ResidualNorm(ctypes.Structure):
+    _fields_ = [("h", ctypes.c_void_p), ("norm_weight", ctypes.c_void_p), ("x_out", ctypes.c_void_p),
+                ("sumsq_out", ctypes.c_void_p), ("sumsq_stride", ctypes.c_int)]
+
+
+class RowScale(NamedTuple):
+    """The rows' factors of an RMS norm that a product applies to its result: row ``r`` is multiplied by
+    ``1 / sqrt(sumsq[r, :groups].sum() / width + eps)``. ``gemm_skinny_residual`` makes these."""
+    sumsq: torch.Tensor     # float32 [rows, stride]; stride is a multiple of 4
+    groups: int
+    width: int
+    eps: float
+
+
+def _scale_argument(scale: Optional[RowScale], rows: int):
+    if scale is None:
+        return None
+    _device_tensor(scale.sumsq, "sums of squares", torch.float32)
+    _need(scale.sumsq.dim() == 2 and scale.sumsq.shape[0] == rows and rows <= 16, "row factors are [rows <= 16, stride]")
+    _need(scale.sumsq.shape[1] % 4 == 0 and 0 < scale.groups <= scale.sumsq.shape[1], "rows of sums must be a multiple of 4 long")
+    return ctypes.byref(_RowScale(_ptr(scale.sumsq), int(scale.groups), scale.sumsq.shape[1], int(scale.width), float(scale.eps)))
+
+
 class _QkvStore(ctypes.Structure):
     _fields_ = [("bias", ctypes.c_void_p), ("slot_mapping", ctypes.c_void_p),
                 ("cos_sin", ctypes.c_void_p), ("n_freq", ctypes.c_int), ("q_out", ctypes.c_void_p),
@@ -198,7 +226,8 @@ class _QkvStore(ctypes.Structure):
 def gemm_skinny_qkv(x: torch.Tensor, packed: torch.Tensor, bias: Optional[torch.Tensor],
                     slot_mapping: Optional[torch.Tensor], cos_sin: Optional[torch.Tensor],
                     k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                    heads: int, kv_heads: int, head_dim: int, page_size: int) -> torch.Tensor:
+                    heads: int, kv_heads: int, head_dim: int, page_size: int,
+                    scale: Optional[RowScale] = None) -> torch.Tensor:
     """Queries, keys and values of at most 16 bfloat16 rows in one kernel: ``gemm_skinny`` finished by the work
     of ``qkv_rope_store``. ``packed`` is the stacked weight packed in ``rotary_pair_order``; ``cos_sin`` is
     ``rope_table``'s for these rows (none: no rotation). Returns the queries."""
@@ -228,8 +257,36 @@ def gemm_skinny_qkv(x: torch.Tensor, packed: torch.Tensor, bias: Optional[torch.
     q_out = torch.empty((m, heads * head_dim), dtype=torch.bfloat16, device=x.device)
     store = _QkvStore(_ptr(bias), _ptr(slot_mapping), _ptr(cos_sin), n_freq, _ptr(q_out),
                       _ptr(k_cache), _ptr(v_cache), heads, kv_heads, head_dim, page_size)
-    _check(lib.mll_gemm_skinny_qkv(_ptr(x), _ptr(packed), m, k, ctypes.byref(store), _stream()), lib)
+    _check(lib.mll_gemm_skinny_qkv(_ptr(x), _ptr(packed), m, k, ctypes.byref(store), _scale_argument(scale, m), _stream()), lib)
     return q_out
+
+
+def gemm_skinny_residual(x: torch.Tensor, packed: torch.Tensor, h: torch.Tensor, norm_weight: torch.Tensor,
+                         width: int, eps: float, scale: Optional[RowScale] = None) -> Tuple[torch.Tensor, RowScale]:
+    """``h += x @ W.T`` for at most 16 bfloat16 rows, and the RMS norm of the sum begun.
+
+    Returns ``(h * norm_weight)`` in bfloat16, the norm's result but for the rows' factors, and those factors as
+    a ``RowScale`` for the product that takes it."""
+    lib = library.load()
+    _device_tensor(x, "gemm input", torch.bfloat16)
+    _device_tensor(packed, "packed weight", torch.bfloat16)
+    _device_tensor(h, "residual stream", torch.float32)
+    _device_tensor(norm_weight, "norm weight", torch.float32)
+    _need(x.dim() == 2 and x.shape[0] <= 16, "gemm_skinny_residual takes [m <= 16, k] activations")
+    m, k = x.shape
+    _need(h.dim() == 2 and h.shape[0] == m and h.shape[1] == width, "the residual stream must be [m, n]")
+    n = h.shape[1]
+    _need(tuple(norm_weight.shape) == (n,), "the norm's weight must be [n]")
+    _need(k % 8 == 0, "gemm_skinny_residual needs k to be a multiple of 8")
+    _need(packed.dim() == 5 and tuple(packed.shape[2:]) == (4, 16, 8) and packed.shape[0] == -(-n // 16)
+          and packed.shape[1] == -(-k // 32), "the packed weight does not fit n and k")
+    groups = -(-n // 16)
+    x_out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    sumsq = torch.empty((m, -(-groups // 4) * 4), dtype=torch.float32, device=x.device)
+    residual = _ResidualNorm(_ptr(h), _ptr(norm_weight), _ptr(x_out), _ptr(sumsq), sumsq.shape[1])
+    _check(lib.mll_gemm_skinny_residual(_ptr(x), _ptr(packed), m, n, k, ctypes.byref(residual), _scale_argument(scale, m),
+                                        _stream()), lib)
+    return x_out, RowScale(sumsq, groups, width, eps)
 
 
 def _check_pages(k_cache, v_cache, dtype, kv_heads, head_dim, page_size=None) -> int:
@@ -491,11 +548,13 @@ def pack_weight(weight: torch.Tensor, interleave_halves: bool = False,
 SKINNY_MAX_ROWS = 64
 
 
-def gemm_skinny(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f32") -> torch.Tensor:
+def gemm_skinny(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f32",
+                scale: Optional[RowScale] = None) -> torch.Tensor:
     """``x @ W.T`` for at most 64 bfloat16 rows and a packed weight.
 
     ``f32``: float32 ``[m, n]``; ``bf16``: bfloat16 ``[m, n]``; ``gated``: bfloat16 ``[m, n / 2]`` of
-    silu(gate) * up for interleaved rows.
+    silu(gate) * up for interleaved rows. With ``scale`` (at most 16 rows) the rows of the product are
+    multiplied by its factors first.
     """
     lib = library.load()
     _device_tensor(x, "gemm input", torch.bfloat16)
@@ -514,7 +573,7 @@ def gemm_skinny(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "
         code, out = 2, torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
     else:
         raise KernelLibraryError(f"unknown epilogue {epilogue!r}")
-    _check(lib.mll_gemm_skinny(_ptr(x), _ptr(packed), _ptr(out), code, m, n, k, _stream()), lib)
+    _check(lib.mll_gemm_skinny(_ptr(x), _ptr(packed), _ptr(out), code, m, n, k, _scale_argument(scale, m), _stream()), lib)
     return out
 
 

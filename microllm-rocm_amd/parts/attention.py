@@ -17,12 +17,13 @@ import torch
 
 from ..ops import kernels
 from .base import MATRIX, Mixer, PagedKVNeed, Runtime, TensorDecl, VECTOR
-from .linear import SKINNY_ROWS, Weight, linear, takes_packed
+from .linear import SKINNY_ROWS, UnscaledRows, Weight, linear, linear_into_stream, takes_packed, takes_unscaled
 from .registry import build_part, register_part
 from .spec import PartSpec
 
 
 class PagedAttention(Mixer):
+    fuses_residual = True
     graph_safe = True
     def __init__(self, spec: PartSpec, runtime: Runtime):
         super().__init__(spec, runtime)
@@ -81,8 +82,14 @@ class PagedAttention(Mixer):
         return PagedKVNeed(self.kv_heads, self.head_dim, self.window)
 
     # ---- forward -------------------------------------------------------------------------
-    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+    def takes_unscaled(self, rows: int) -> bool:
+        return self.qkv_weight.row_order is not None and takes_unscaled(self.qkv_weight, rows)
+
+    def forward(self, x, ctx, cache, residual=None):
         view = ctx.paged[cache.group]
+        scale = None
+        if isinstance(x, UnscaledRows):     # only where takes_unscaled said so: the q/k/v product applies the factors
+            x, scale = x.values, x.scale
         kv_heads = cache.need.kv_heads
         stored_heads = self.kv_heads if self.owns_kv else 0
         slot_mapping = view.slot_mapping if self.owns_kv else None
@@ -95,8 +102,10 @@ class PagedAttention(Mixer):
         pair_order = weight.row_order is not None and x.dtype == weight.dtype and takes_packed(weight, x.shape[0])
         if pair_order and x.shape[0] <= SKINNY_ROWS:
             q = kernels.gemm_skinny_qkv(x, weight.packed, bias, slot_mapping, cos_sin, k_pages, v_pages,
-                                        self.heads, stored_heads, self.head_dim, view.page_size)
+                                        self.heads, stored_heads, self.head_dim, view.page_size, scale=scale)
         else:
+            if scale is not None:
+                raise TypeError("rows without their factors reached a q/k/v product that cannot apply them")
             qkv = linear(x, weight, out_dtype=torch.float32, partials=fused)   # rounded once, after bias and rotation
             if not fused:
                 if bias is not None:
@@ -109,6 +118,10 @@ class PagedAttention(Mixer):
         window = int(self.window) if self.window else 0
         o = kernels.paged_attention(q, cache.k, cache.v, view, ctx, self.scale, window,
                                     self.heads, kv_heads, self.head_dim)
+        if residual is not None:
+            begun = linear_into_stream(o, self.o_weight, residual)
+            if begun is not None:
+                return begun
         return linear(o, self.o_weight, out_dtype=torch.float32, partials=True)   # summed into the residual stream in float32
 
 

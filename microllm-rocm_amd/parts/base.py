@@ -78,18 +78,30 @@ class Part:
 class Mixer(Part):
     """Mixes information between the positions of one request (attention, or a layer with state)."""
     category = "mixer"
+    fuses_residual = False
+
+    def takes_unscaled(self, rows: int) -> bool:
+        return False
 
     def cache_need(self) -> CacheNeed:
         return None
 
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
         """``[tokens, hidden]`` -> the delta for the residual stream: ``[tokens, hidden]``, or float32 partial
-        sums ``[parts, tokens, hidden]`` that the next norm adds in order."""
+        sums ``[parts, tokens, hidden]`` that the next norm adds in order.
+
+        A part with ``fuses_residual`` also takes ``residual=`` (a ``linear.Residual``, or None) and may then add
+        its delta to the stream itself and return the next norm's result as ``linear.UnscaledRows``; a part whose
+        ``takes_unscaled(rows)`` says so takes such rows as ``x``. A block only uses either where both sides agree."""
         raise NotImplementedError
 
 
 class FeedForward(Part):
     category = "ffn"
+    fuses_residual = False
+
+    def takes_unscaled(self, rows: int) -> bool:
+        return False
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         """``[tokens, hidden]`` -> the delta for the residual stream, as a mixer's."""
@@ -98,6 +110,11 @@ class FeedForward(Part):
 
 class Norm(Part):
     category = "norm"
+
+    def weight_then_factor(self):
+        """``(weight, width, eps)`` if the norm is ``x * weight * (1 / sqrt(mean(x^2) + eps))``, so that a product
+        before it can multiply by the weight and the product after it by the rows' factors; else None."""
+        return None
 
     def forward(self, h: torch.Tensor, delta: Optional[torch.Tensor] = None, write_h: bool = True,
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:

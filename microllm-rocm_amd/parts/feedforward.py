@@ -12,13 +12,14 @@ import torch
 
 from ..ops import kernels
 from .base import FeedForward, MATRIX, Runtime, TensorDecl
-from .linear import Weight, linear
+from .linear import Weight, linear, linear_into_stream, takes_unscaled
 from .registry import register_part
 from .spec import PartSpec
 
 
 class SwiGLU(FeedForward):
     graph_safe = True
+    fuses_residual = True
     def __init__(self, spec: PartSpec, runtime: Runtime):
         super().__init__(spec, runtime)
         self.hidden = int(spec.params["hidden_size"])
@@ -41,8 +42,15 @@ class SwiGLU(FeedForward):
         self.gate_up_weight = Weight(torch.cat([gate, up], dim=0).contiguous(), gated=True)
         self.down_weight = Weight(tensors[self.name("down_proj.weight")])
 
-    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+    def takes_unscaled(self, rows: int) -> bool:
+        return takes_unscaled(self.gate_up_weight, rows)
+
+    def forward(self, x, ctx, residual=None):
         z = linear(x, self.gate_up_weight, gated=True)
+        if residual is not None:
+            begun = linear_into_stream(z, self.down_weight, residual)
+            if begun is not None:
+                return begun
         return linear(z, self.down_weight, out_dtype=torch.float32, partials=True)
 
 

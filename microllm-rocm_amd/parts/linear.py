@@ -10,7 +10,8 @@ kernels that stream it once when a step has few rows (decoding): one for up to
 """
 from __future__ import annotations
 
-from typing import Optional
+from dataclasses import dataclass
+from typing import Optional, Union
 
 import torch
 
@@ -35,10 +36,54 @@ class Weight:
         return self.tensor.dtype
 
 
+MAX_FACTOR_WIDTH = 8192   # the widest norm whose rows' factors the streaming product applies (its sums sit in LDS)
 SKINNY_ROWS = 16        # up to this many rows gemm_skinny beats the library on MI355X for every weight
 MEDIUM_ROWS = 64        # and up to this many gemm_medium does, except for
 MEDIUM_WIDE_TILES = 2048   # weights with this many tiles of 16 rows or more (gate/up, the head), where the
 MEDIUM_WIDE_ROWS = 40      # library is as fast from about this many rows on
+
+
+@dataclass
+class UnscaledRows:
+    """A norm's result but for the rows' factors: ``values`` is ``(h * norm weight)`` rounded to bfloat16, and a
+    product that takes it multiplies its own rows by ``scale``'s factors (the product is linear in them).
+    ``linear_into_stream`` makes these; ``linear`` takes them where ``takes_unscaled`` says so."""
+    values: torch.Tensor
+    scale: kernels.RowScale
+
+    @property
+    def shape(self):
+        return self.values.shape
+
+    @property
+    def dtype(self):
+        return self.values.dtype
+
+
+@dataclass
+class Residual:
+    """What the last product of a mixer or feed-forward needs to add its result to the residual stream itself
+    and begin the norm that follows: the stream and that norm's weight, width and eps."""
+    h: torch.Tensor
+    norm_weight: torch.Tensor
+    width: int
+    eps: float
+
+
+def takes_unscaled(weight: "Weight", rows: int) -> bool:
+    """Whether ``linear`` (and the q/k/v product) can apply rows' factors for this weight and this many rows."""
+    return weight.packed is not None and rows <= SKINNY_ROWS
+
+
+def linear_into_stream(x: torch.Tensor, weight: "Weight", residual: Residual) -> Optional[UnscaledRows]:
+    """``residual.h += x @ W.T`` and the next norm begun, in the product's epilogue; None where that cannot be
+    done (then nothing was changed and the caller returns its delta as usual)."""
+    if not isinstance(x, torch.Tensor) or x.dtype != torch.bfloat16 or not takes_unscaled(weight, x.shape[0]):
+        return None
+    if weight.row_order is not None or residual.norm_weight.dtype != torch.float32 or residual.width > MAX_FACTOR_WIDTH:
+        return None
+    values, scale = kernels.gemm_skinny_residual(x, weight.packed, residual.h, residual.norm_weight, residual.width, residual.eps)
+    return UnscaledRows(values, scale)
 
 
 def takes_packed(weight: "Weight", rows: int, gated: bool = False) -> bool:
@@ -51,7 +96,7 @@ def takes_packed(weight: "Weight", rows: int, gated: bool = False) -> bool:
     return not gated and rows <= (MEDIUM_WIDE_ROWS if wide else MEDIUM_ROWS)
 
 
-def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None, gated: bool = False,
+def linear(x: Union[torch.Tensor, UnscaledRows], weight, out_dtype: Optional[torch.dtype] = None, gated: bool = False,
            partials: bool = False) -> torch.Tensor:
     """``x @ W.T`` with float32 accumulation; the result has ``out_dtype`` (default: x's).
 
@@ -63,6 +108,11 @@ def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None, gat
     if isinstance(weight, torch.Tensor):
         weight = Weight(weight, pack=False)
     out_dtype = out_dtype or x.dtype
+    scale = None
+    if isinstance(x, UnscaledRows):
+        if not takes_unscaled(weight, x.shape[0]) or x.dtype != weight.dtype:
+            raise TypeError("this product cannot apply the rows' factors; see takes_unscaled")
+        x, scale = x.values, x.scale
     w = weight.tensor
     if w.dtype == torch.float32:
         # True 32-bit product, also for a 32-bit weight inside a bfloat16 engine.
@@ -76,8 +126,9 @@ def linear(x: torch.Tensor, weight, out_dtype: Optional[torch.dtype] = None, gat
     rows = x.shape[0]
     if weight.packed is not None and rows <= SKINNY_ROWS:
         if gated:
-            return kernels.gemm_skinny(x, weight.packed, weight.out_features, "gated")
-        return kernels.gemm_skinny(x, weight.packed, weight.out_features, "bf16" if out_dtype == torch.bfloat16 else "f32")
+            return kernels.gemm_skinny(x, weight.packed, weight.out_features, "gated", scale=scale)
+        return kernels.gemm_skinny(x, weight.packed, weight.out_features, "bf16" if out_dtype == torch.bfloat16 else "f32",
+                                   scale=scale)
     if takes_packed(weight, rows, gated):
         if out_dtype == torch.float32:
             plan = kernels.medium_plan(weight.out_features, weight.in_features, may_split=partials)

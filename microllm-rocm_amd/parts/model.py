@@ -126,8 +126,10 @@ class Model:
         """
         h = self.embedding.forward(ctx.tokens)
         pending = None
-        for index, entry in enumerate(self.spec.order):
-            pending = self.blocks[entry.layer].forward(h, pending, ctx, caches[index])
+        order = self.spec.order
+        for index, entry in enumerate(order):
+            next_block = self.blocks[order[index + 1].layer] if index + 1 < len(order) else None
+            pending = self.blocks[entry.layer].forward(h, pending, ctx, caches[index], next_block)
         if want_rows is None or want_rows.numel() == 0:
             return None
         x = self.final_norm.forward(h, delta=pending, write_h=False, rows=want_rows)

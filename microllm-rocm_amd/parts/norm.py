@@ -30,6 +30,9 @@ class RMSNorm(Norm):
     def bind(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.weight = tensors[self.name("weight")]
 
+    def weight_then_factor(self):
+        return (self.weight, self.size, self.eps) if self.weight is not None and self.weight.dtype == torch.float32 else None
+
     def forward(self, h, delta=None, write_h=True, rows=None):
         return kernels.rms_norm(h, self.weight, self.eps, self.runtime.dtype, delta=delta, rows=rows,
                                 write_h=write_h and delta is not None and rows is None)

@@ -486,6 +486,45 @@ def test_gemm_skinny_qkv_is_product_then_rope_store(m, heads, kv_heads, hd, rota
         assert torch.equal(k_three, k_two) and torch.equal(v_three, v_two)
 
 
+@pytest.mark.parametrize("m", [1, 5, 16])
+@pytest.mark.parametrize("n,k,n2", [(72, 320, 144), (3584, 512, 1024), (104, 96, 5000), (4096, 64, 96)])
+def test_product_adds_to_the_stream_and_begins_the_norm(m, n, k, n2):
+    """``gemm_skinny_residual`` then a product with the rows' factors, against sum, RMS norm and product done apart."""
+    rng = np.random.default_rng(m + n)
+    ka = kernels()
+    x_ref, x = to_bf16_exact(rng.normal(size=(m, k)))
+    w1_ref, w1 = to_bf16_exact(rng.normal(size=(n, k)) * 0.1)
+    w2_ref, w2 = to_bf16_exact(rng.normal(size=(n2, n)) * 0.1)
+    h_ref = rng.normal(size=(m, n)).astype(np.float32)
+    norm_ref = (1.0 + 0.1 * rng.normal(size=n)).astype(np.float32)
+    eps = 1e-5
+    h = torch.from_numpy(h_ref.copy()).to(DEVICE)
+    norm = torch.from_numpy(norm_ref).to(DEVICE)
+    values, scale = ka.gemm_skinny_residual(x, ka.pack_weight(w1), h, norm, n, eps)
+    total = h_ref.astype(np.float64) + x_ref @ w1_ref.T
+    np.testing.assert_allclose(h.cpu().numpy(), total, rtol=1e-5, atol=1e-5 * np.abs(total).max())
+    assert values.dtype == torch.bfloat16 and scale.sumsq.shape[0] == m and scale.width == n
+    np.testing.assert_allclose(values.float().cpu().numpy(), total * norm_ref, rtol=8e-3, atol=1e-6)
+    np.testing.assert_allclose(scale.sumsq[:, :scale.groups].double().sum(dim=1).cpu().numpy(), (total ** 2).sum(axis=1), rtol=1e-5)
+    expected = plain.rms_norm(total, norm_ref, eps) @ w2_ref.T
+    bound = 1.2e-2 * np.abs(expected).max()
+    packed2 = ka.pack_weight(w2)
+    out = ka.gemm_skinny(values, packed2, n2, "f32", scale=scale)
+    assert np.abs(out.double().cpu().numpy() - expected).max() <= bound
+    # the factors are the norm's: the same product of the norm's own output differs by rounding only
+    h_two = torch.from_numpy(h_ref.copy()).to(DEVICE)
+    normed = ka.rms_norm(h_two, norm, eps, torch.bfloat16, delta=ka.gemm_skinny(x, ka.pack_weight(w1), n, "f32"), write_h=True)
+    apart = ka.gemm_skinny(normed, packed2, n2, "f32")
+    assert np.abs(apart.double().cpu().numpy() - expected).max() <= bound
+    assert torch.equal(h_two, h)
+    # a row's result does not depend on the other rows
+    h_one = torch.from_numpy(h_ref[m - 1:m].copy()).to(DEVICE)
+    values_one, scale_one = ka.gemm_skinny_residual(x[m - 1:m].contiguous(), ka.pack_weight(w1), h_one, norm, n, eps)
+    assert torch.equal(values_one[0], values[m - 1]) and torch.equal(h_one[0], h[m - 1])
+    alone = ka.gemm_skinny(values_one, packed2, n2, "f32", scale=scale_one)
+    assert torch.equal(alone[0], out[m - 1])
+
+
 @pytest.mark.parametrize("m", [17, 33, 40, 64, 5])
 @pytest.mark.parametrize("n,k", [(331, 120), (1000, 200), (4608, 3584), (176, 24), (3584, 18944), (40000, 256), (896, 4864)])
 def test_gemm_medium(m, n, k):
