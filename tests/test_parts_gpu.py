@@ -155,6 +155,52 @@ def test_pre_norm_block_alone(dtype):
     np.testing.assert_allclose(total, expected, rtol=TOL[dtype]["rtol"], atol=TOL[dtype]["atol"] * np.abs(expected).max())
 
 
+def test_few_rows_take_the_norm_between_two_products():
+    """In bfloat16, with few rows, a block's last product begins the next norm and the next block's first product ends it."""
+    from microllm_rocm_amd.parts.linear import UnscaledRows
+    config = TINY_B.replace(use_sliding_window=False)
+    spec = build_spec(config)
+    dtype = torch.bfloat16
+    rng = np.random.default_rng(5)
+    blocks, exact = [], {}
+    for index in (0, 1):
+        block = build_block(spec.layers[index], runtime(dtype))
+        tensors = {}
+        for name, decl in block.tensors().items():
+            array = (1 + 0.1 * rng.normal(size=decl.shape)) if name.endswith("layernorm.weight") else rng.normal(size=decl.shape) * 0.15
+            value = bf16_exact(array)
+            exact[name] = value.double().numpy()
+            tensors[name] = value.to(torch.float32 if decl.kind == "vector" else torch.bfloat16).to(DEVICE)
+        block.bind(tensors)
+        blocks.append(block)
+    needs = [block.mixer.cache_need() for block in blocks]
+    cache = CacheManager(needs, [None, None], 16, 8, 2, dtype=dtype, device=DEVICE)
+    request = cache.open("r")
+    rows = 5
+    cache.reserve(request, rows)
+    ctx = BatchBuilder(cache, DEVICE).build([request], [[0] * rows], [[]])
+    h_ref = rng.normal(size=(rows, config.hidden_size)).astype(np.float32)
+    h = torch.from_numpy(h_ref.copy()).to(DEVICE)
+    pending = blocks[0].forward(h, None, ctx, cache.bindings()[0], blocks[1])
+    assert isinstance(pending, UnscaledRows)                   # the sum is in h already, the norm half done
+    after_first = plain.block(h_ref.astype(np.float64), exact, 0, config.to_dict(), None)
+    np.testing.assert_allclose(h.double().cpu().numpy(), after_first, rtol=TOL[dtype]["rtol"], atol=TOL[dtype]["atol"] * np.abs(after_first).max())
+    pending = blocks[1].forward(h, pending, ctx, cache.bindings()[1], None)
+    assert isinstance(pending, torch.Tensor)                   # no block follows: a plain delta (or partial sums)
+    pending = pending.sum(dim=0) if pending.dim() == 3 else pending
+    expected = plain.block(after_first, exact, 1, config.to_dict(), None)
+    total = h.double().cpu().numpy() + pending.double().cpu().numpy()
+    np.testing.assert_allclose(total, expected, rtol=TOL[dtype]["rtol"], atol=TOL[dtype]["atol"] * np.abs(expected).max())
+    # with many rows the same blocks take the ordinary way
+    cache.cancel_reservation(request)
+    cache.close("r")
+    request = cache.open("s")
+    cache.reserve(request, 40)
+    ctx = BatchBuilder(cache, DEVICE).build([request], [[0] * 40], [[]])
+    h = torch.zeros((40, config.hidden_size), dtype=torch.float32, device=DEVICE)
+    assert isinstance(blocks[0].forward(h, None, ctx, cache.bindings()[0], blocks[1]), torch.Tensor)
+
+
 def qwen_like_layer(index, hidden, heads, kv_heads, hd, inter, window=None, owns_kv=True):
     prefix = f"model.layers.{index}"
     names = {"q_proj.weight": f"{prefix}.self_attn.q_proj.weight", "q_proj.bias": f"{prefix}.self_attn.q_proj.bias",
