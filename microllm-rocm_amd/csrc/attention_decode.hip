@@ -156,8 +156,7 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
         float tile_max = score[0];
 #pragma unroll
         for (int j = 1; j < 8; ++j) tile_max = fmaxf(tile_max, score[j]);
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+        tile_max = max_lanes_16_apart(tile_max);
         const float new_max = fmaxf(running_max, tile_max);   // finite: every pair holds a visible key
         const float rescale = __expf(running_max - new_max);
         Frag8 p_frag;
@@ -168,8 +167,7 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
             tile_sum += p;
             p_frag.v[j] = static_cast<__bf16>(p);
         }
-        tile_sum += __shfl_xor(tile_sum, 16, kWave);
-        tile_sum += __shfl_xor(tile_sum, 32, kWave);
+        tile_sum = sum_lanes_16_apart(tile_sum);
         running_sum = running_sum * rescale + tile_sum;
         running_max = new_max;
 #pragma unroll

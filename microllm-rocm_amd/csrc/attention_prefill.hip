@@ -7,7 +7,13 @@
 // this one is used. As in the decode kernel, scores are computed transposed, S^T = K . Q^T, the 16 columns
 // being query positions, and O^T = V^T . P^T follows from registers; every fragment of K and V read from LDS
 // serves both column blocks. Only pairs of tiles that touch the causal diagonal or the window's edge pay
-// for the mask. The list of tiles (request, first token in the flat list, tokens) is built on the host.
+// for the mask (they run a second instance of the inner loop's body), and values that no token of the
+// workgroup can see are cleared once, on their way into LDS, so that stale memory never meets a zero weight.
+// The vector unit, not the MFMA, bounds this kernel: the scale is folded into the exponent's multiply-add and
+// the accumulators are rescaled only when some maximum has moved.
+// The list of tiles (request, first token in the flat list, tokens) is built on the host.
+#include <type_traits>
+
 #include "cache_layout.h"
 #include "common.h"
 #include "microllm_hip.h"
@@ -99,7 +105,9 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void paged_attention_prefill_ke
 
     // Copy of one block's tiles: thread i moves bytes [16 i, 16 i + 16) of every pass of every tile.
     uint4 staged[BLOCK_TILES][2][TILE_PASSES];
+    int staged_block = 0;
     auto fetch = [&](int block) {
+        staged_block = block;
 #pragma unroll
         for (int t = 0; t < BLOCK_TILES; ++t) {
             const int tile_key = block * BLOCK_KEYS + 16 * t;
@@ -123,6 +131,25 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void paged_attention_prefill_ke
     auto stash = [&](int stage) {
         bf16* base = lds + stage * STAGE_ELEMENTS;
 #pragma unroll
+        for (int t = 0; t < BLOCK_TILES; ++t) {
+            // A tile that straddles an end of what the workgroup's tokens can see holds positions that may be stale
+            // memory: their values are cleared here (their scores are masked where they are computed).
+            const int tile_key = staged_block * BLOCK_KEYS + 16 * t;
+            if (tile_key <= group_last && tile_key + 15 >= group_low && (tile_key + 15 > group_last || tile_key < group_low)) {
+#pragma unroll
+                for (int pass = 0; pass < TILE_PASSES; ++pass) {
+                    const int element = (pass * kPrefillThreads + threadIdx.x) * 8;   // 2 dims x positions 4 g .. 4 g + 3
+                    const int first_key = tile_key + 4 * ((element / 64) % 4);
+                    PFrag8 values;
+                    values.raw = staged[t][1][pass];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i)
+                        if (first_key + i % 4 > group_last || first_key + i % 4 < group_low) values.v[i] = static_cast<__bf16>(0.0f);
+                    staged[t][1][pass] = values.raw;
+                }
+            }
+        }
+#pragma unroll
         for (int t = 0; t < BLOCK_TILES; ++t)
 #pragma unroll
             for (int pass = 0; pass < TILE_PASSES; ++pass) {
@@ -132,6 +159,88 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void paged_attention_prefill_ke
                     *reinterpret_cast<uint4*>(base + (BLOCK_TILES + t) * TILE_ELEMENTS + element) = staged[t][1][pass];
                 }
             }
+    };
+
+    // One pair of key tiles (32 keys) against the wave's 32 tokens. MASKED: some key of the pair is hidden from
+    // some token of the wave (the causal diagonal, the window's edge, the end of the sequence).
+    // Scores stay in the product's units; p = 2^((s - max) * scale_log2) is one multiply-add and one exponent.
+    auto process_pair = [&](auto masked_tag, const bf16* k_lds, const bf16* v_lds, int pair, int key0) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        PFrag8 k_frag[2][K_STEPS];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int ks = 0; ks < K_STEPS; ++ks) {
+                const int piece = ks * 4 + quad;
+                k_frag[t][ks].raw = make_uint4(0, 0, 0, 0);
+                if (piece < K_CHUNKS)
+                    k_frag[t][ks].raw = *reinterpret_cast<const uint4*>(
+                        k_lds + (2 * pair + t) * TILE_ELEMENTS + piece * 128 + col * 8);
+            }
+        PFrag8 p_frag[2];
+        float rescale[2];
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            if (c >= column_blocks) {
+                p_frag[c].raw = make_uint4(0, 0, 0, 0);
+                rescale[c] = 1.0f;
+                continue;
+            }
+            float score[8];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                floatx4 s = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int ks = 0; ks < K_STEPS; ++ks)
+                    s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_frag[t][ks].v, q_frag[c][ks].v, s, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) score[4 * t + i] = s[i];
+            }
+            if (MASKED) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int key = key0 + 16 * (j / 4) + 4 * quad + (j % 4);
+                    if (key > my_position[c] || key < my_low[c]) score[j] = -INFINITY;
+                }
+            }
+            float tile_max = score[0];
+#pragma unroll
+            for (int j = 1; j < 8; ++j) tile_max = fmaxf(tile_max, score[j]);
+            tile_max = max_lanes_16_apart(tile_max);
+            const float new_max = fmaxf(running_max[c], tile_max);
+            // A query may see nothing of a pair that others see (the window's edge): its maximum stays -inf.
+            const float safe_max = (MASKED && new_max == -INFINITY) ? 0.0f : new_max;
+            const float offset = -safe_max * scale_log2;
+            rescale[c] = __builtin_amdgcn_exp2f(fmaf(running_max[c], scale_log2, offset));
+            float tile_sum = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float p = __builtin_amdgcn_exp2f(fmaf(score[j], scale_log2, offset));
+                tile_sum += p;
+                p_frag[c].v[j] = static_cast<__bf16>(p);
+            }
+            tile_sum = sum_lanes_16_apart(tile_sum);
+            running_sum[c] = running_sum[c] * rescale[c] + tile_sum;
+            running_max[c] = new_max;
+        }
+        // Once the running maxima have settled, no column's sum needs rescaling: one branch for the whole wave.
+        if (__any(rescale[0] != 1.0f || rescale[1] != 1.0f)) {
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+#pragma unroll
+                for (int d = 0; d < HD_TILES; ++d) o_acc[c][d] *= rescale[c];
+        }
+#pragma unroll
+        for (int d = 0; d < HD_TILES; ++d) {
+            PFrag8 v_frag;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                v_frag.h[t] = *reinterpret_cast<const bf16x4*>(
+                    v_lds + (2 * pair + t) * TILE_ELEMENTS + d * 256 + (quad * 16 + col) * 4);
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+                o_acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_frag.v, p_frag[c].v, o_acc[c][d], 0, 0, 0);
+        }
     };
 
     const int first_block = group_low / BLOCK_KEYS;
@@ -150,88 +259,8 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void paged_attention_prefill_ke
             for (int pair = 0; pair < BLOCK_TILES / 2; ++pair) {
                 const int key0 = block * BLOCK_KEYS + 32 * pair;
                 if (key0 > wave_last || key0 + 31 < wave_low) continue;   // nothing of this pair is visible to the wave
-                PFrag8 k_frag[2][K_STEPS];
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-#pragma unroll
-                    for (int ks = 0; ks < K_STEPS; ++ks) {
-                        const int piece = ks * 4 + quad;
-                        k_frag[t][ks].raw = make_uint4(0, 0, 0, 0);
-                        if (piece < K_CHUNKS)
-                            k_frag[t][ks].raw = *reinterpret_cast<const uint4*>(
-                                k_lds + (2 * pair + t) * TILE_ELEMENTS + piece * 128 + col * 8);
-                    }
-                const bool needs_mask = key0 + 31 > wave_position || key0 < wave_last_low;
-                PFrag8 p_frag[2];
-                float rescale[2];
-#pragma unroll
-                for (int c = 0; c < 2; ++c) {
-                    if (c >= column_blocks) {
-                        p_frag[c].raw = make_uint4(0, 0, 0, 0);
-                        rescale[c] = 1.0f;
-                        continue;
-                    }
-                    float score[8];
-#pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-                        floatx4 s = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-                        for (int ks = 0; ks < K_STEPS; ++ks)
-                            s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_frag[t][ks].v, q_frag[c][ks].v, s, 0, 0, 0);
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) score[4 * t + i] = s[i] * scale_log2;
-                    }
-                    if (needs_mask) {
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) {
-                            const int key = key0 + 16 * (j / 4) + 4 * quad + (j % 4);
-                            if (key > my_position[c] || key < my_low[c]) score[j] = -INFINITY;
-                        }
-                    }
-                    float tile_max = score[0];
-#pragma unroll
-                    for (int j = 1; j < 8; ++j) tile_max = fmaxf(tile_max, score[j]);
-                    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
-                    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
-                    const float new_max = fmaxf(running_max[c], tile_max);
-                    // A query may see nothing of a pair that others see (the window's edge): its maximum stays -inf.
-                    const float safe_max = new_max == -INFINITY ? 0.0f : new_max;
-                    rescale[c] = __builtin_amdgcn_exp2f(running_max[c] - safe_max);
-                    float tile_sum = 0.0f;
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const float p = __builtin_amdgcn_exp2f(score[j] - safe_max);
-                        tile_sum += p;
-                        p_frag[c].v[j] = static_cast<__bf16>(p);
-                    }
-                    tile_sum += __shfl_xor(tile_sum, 16, kWave);
-                    tile_sum += __shfl_xor(tile_sum, 32, kWave);
-                    running_sum[c] = running_sum[c] * rescale[c] + tile_sum;
-                    running_max[c] = new_max;
-                }
-                // Once the running maxima have settled, no column's sum needs rescaling: skip the multiplications.
-                const bool any_rescale = __any(rescale[0] != 1.0f || rescale[1] != 1.0f);
-#pragma unroll
-                for (int d = 0; d < HD_TILES; ++d) {
-                    PFrag8 v_frag;
-#pragma unroll
-                    for (int t = 0; t < 2; ++t)
-                        v_frag.h[t] = *reinterpret_cast<const bf16x4*>(
-                            v_lds + (2 * pair + t) * TILE_ELEMENTS + d * 256 + (quad * 16 + col) * 4);
-                    if (needs_mask) {
-                        // Keys no token of the workgroup can see may be stale memory: 0 * NaN must not reach the sum.
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) {
-                            const int key = key0 + 16 * (j / 4) + 4 * quad + (j % 4);
-                            if (key > group_last || key < group_low) v_frag.v[j] = static_cast<__bf16>(0.0f);
-                        }
-                    }
-#pragma unroll
-                    for (int c = 0; c < 2; ++c) {
-                        if (any_rescale) o_acc[c][d] *= rescale[c];
-                        o_acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_frag.v, p_frag[c].v, o_acc[c][d], 0, 0, 0);
-                    }
-                }
+                if (key0 + 31 > wave_position || key0 < wave_last_low) process_pair(std::true_type{}, k_lds, v_lds, pair, key0);
+                else process_pair(std::false_type{}, k_lds, v_lds, pair, key0);
             }
         }
         if (block < last_block) stash(stage ^ 1);
@@ -245,9 +274,12 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void paged_attention_prefill_ke
             const float inverse = 1.0f / running_sum[c];
             bf16* out_row = out + (static_cast<int64_t>(tile_token + wave_first + 16 * c + col) * heads + head) * HD;
 #pragma unroll
-            for (int d = 0; d < HD_TILES; ++d)
+            for (int d = 0; d < HD_TILES; ++d) {
+                bf16x4 four;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) out_row[d * 16 + quad * 4 + i] = from_float<bf16>(o_acc[c][d][i] * inverse);
+                for (int i = 0; i < 4; ++i) four[i] = static_cast<__bf16>(o_acc[c][d][i] * inverse);
+                *reinterpret_cast<bf16x4*>(out_row + d * 16 + quad * 4) = four;
+            }
         }
     }
 }

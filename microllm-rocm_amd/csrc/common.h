@@ -27,6 +27,28 @@ __host__ __device__ inline float to_float(bf16 value) {
     return caster.f;
 }
 
+// op over the four lanes {l, l ^ 16, l ^ 32, l ^ 48} of a wave, every one of which gets the result: two
+// exchanges on the vector unit (v_permlane16_swap, v_permlane32_swap of gfx950) instead of four trips through
+// LDS. op must be commutative. (The elements of the builtins' result are copied to scalars before they are
+// reinterpreted: a reinterpretation of the element expression itself reads element 0 twice with this compiler.)
+template <typename Op>
+__device__ inline float reduce_lanes_16_apart(float value, Op op) {
+    const unsigned bits = __builtin_bit_cast(unsigned, value);
+    const auto rows = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+    const unsigned even = rows[0], odd = rows[1];
+    value = op(__builtin_bit_cast(float, even), __builtin_bit_cast(float, odd));
+    const unsigned joined = __builtin_bit_cast(unsigned, value);
+    const auto halves = __builtin_amdgcn_permlane32_swap(joined, joined, false, false);
+    const unsigned low = halves[0], high = halves[1];
+    return op(__builtin_bit_cast(float, low), __builtin_bit_cast(float, high));
+}
+__device__ inline float max_lanes_16_apart(float value) {
+    return reduce_lanes_16_apart(value, [](float a, float b) { return fmaxf(a, b); });
+}
+__device__ inline float sum_lanes_16_apart(float value) {
+    return reduce_lanes_16_apart(value, [](float a, float b) { return a + b; });
+}
+
 template <typename T> __host__ __device__ inline T from_float(float value);
 template <> __host__ __device__ inline float from_float<float>(float value) { return value; }
 template <> __host__ __device__ inline bf16 from_float<bf16>(float value) {

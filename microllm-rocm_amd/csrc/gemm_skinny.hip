@@ -200,8 +200,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
             }
         }
         float part = (parts[0] + parts[1]) + (parts[2] + parts[3]);
-        part += __shfl_xor(part, 16, kWave);
-        part += __shfl_xor(part, 32, kWave);
+        part = sum_lanes_16_apart(part);
         row_factor = 1.0f / sqrtf(part / static_cast<float>(extras.scale.width) + extras.scale.eps);
     }
 
@@ -293,8 +292,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
         if (EPILOGUE == 4) {
             // The row's sum over the tile's 16 columns: the four lanes of a row, in a fixed order. One entry per
             // tile of W, so that the sums do not depend on how many tiles a workgroup takes.
-            squares += __shfl_xor(squares, 16, kWave);
-            squares += __shfl_xor(squares, 32, kWave);
+            squares = sum_lanes_16_apart(squares);
             if (quad == 0 && col < m) extras.residual.sumsq_out[static_cast<int64_t>(col) * extras.residual.sumsq_stride + n_tile] = squares;
         }
     }
