@@ -106,46 +106,62 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void paged_attention_prefill_ke
     // Copy of one block's tiles: thread i moves bytes [16 i, 16 i + 16) of every pass of every tile.
     uint4 staged[BLOCK_TILES][2][TILE_PASSES];
     int staged_block = 0;
+    // The page of a tile: pages hold tiles_per_page tiles of 16 positions (often one, mostly a power of two).
+    const int tiles_per_page = page_size / 16;
+    const int page_shift = (tiles_per_page & (tiles_per_page - 1)) == 0 ? __ffs(tiles_per_page) - 1 : -1;
+    auto fetch_tile = [&](int t, int tile_key, bool live) {
+        const int tile_index = tile_key / 16;
+        const int slot = page_shift >= 0 ? tile_index >> page_shift : tile_index / tiles_per_page;
+        const int tile_in_page = tile_index - slot * tiles_per_page;
+        const int64_t page = live ? table[slot] : 0;
+        const bf16* k_tile = k_cache + layout.k_tile(page, kv_head, tile_in_page);
+        const bf16* v_tile = v_cache + layout.v_tile(page, kv_head, tile_in_page);
+#pragma unroll
+        for (int pass = 0; pass < TILE_PASSES; ++pass) {
+            const int element = (pass * kPrefillThreads + threadIdx.x) * 8;
+            staged[t][0][pass] = make_uint4(0, 0, 0, 0);
+            staged[t][1][pass] = make_uint4(0, 0, 0, 0);
+            if (live && element < TILE_ELEMENTS) {
+                staged[t][0][pass] = *reinterpret_cast<const uint4*>(k_tile + element);
+                staged[t][1][pass] = *reinterpret_cast<const uint4*>(v_tile + element);
+            }
+        }
+    };
+    // A block all of whose keys some token of the workgroup can see (most blocks) needs no checks per tile.
+    auto inside = [&](int block) { return block * BLOCK_KEYS >= group_low && block * BLOCK_KEYS + BLOCK_KEYS - 1 <= group_last; };
     auto fetch = [&](int block) {
         staged_block = block;
+        if (inside(block)) {
 #pragma unroll
-        for (int t = 0; t < BLOCK_TILES; ++t) {
-            const int tile_key = block * BLOCK_KEYS + 16 * t;
-            const bool live = tile_key <= group_last && tile_key + 15 >= group_low;
-            const int64_t page = live ? table[tile_key / page_size] : 0;
-            const int offset = tile_key % page_size;
-            const bf16* k_tile = k_cache + layout.k_tile(page, kv_head, offset / 16);
-            const bf16* v_tile = v_cache + layout.v_tile(page, kv_head, offset / 16);
+            for (int t = 0; t < BLOCK_TILES; ++t) fetch_tile(t, block * BLOCK_KEYS + 16 * t, true);
+        } else {
 #pragma unroll
-            for (int pass = 0; pass < TILE_PASSES; ++pass) {
-                const int element = (pass * kPrefillThreads + threadIdx.x) * 8;
-                staged[t][0][pass] = make_uint4(0, 0, 0, 0);
-                staged[t][1][pass] = make_uint4(0, 0, 0, 0);
-                if (live && element < TILE_ELEMENTS) {
-                    staged[t][0][pass] = *reinterpret_cast<const uint4*>(k_tile + element);
-                    staged[t][1][pass] = *reinterpret_cast<const uint4*>(v_tile + element);
-                }
+            for (int t = 0; t < BLOCK_TILES; ++t) {
+                const int tile_key = block * BLOCK_KEYS + 16 * t;
+                fetch_tile(t, tile_key, tile_key <= group_last && tile_key + 15 >= group_low);
             }
         }
     };
     auto stash = [&](int stage) {
         bf16* base = lds + stage * STAGE_ELEMENTS;
+        if (!inside(staged_block)) {
 #pragma unroll
-        for (int t = 0; t < BLOCK_TILES; ++t) {
-            // A tile that straddles an end of what the workgroup's tokens can see holds positions that may be stale
-            // memory: their values are cleared here (their scores are masked where they are computed).
-            const int tile_key = staged_block * BLOCK_KEYS + 16 * t;
-            if (tile_key <= group_last && tile_key + 15 >= group_low && (tile_key + 15 > group_last || tile_key < group_low)) {
+            for (int t = 0; t < BLOCK_TILES; ++t) {
+                // A tile that straddles an end of what the workgroup's tokens can see holds positions that may be
+                // stale memory: their values are cleared here (their scores are masked where they are computed).
+                const int tile_key = staged_block * BLOCK_KEYS + 16 * t;
+                if (tile_key <= group_last && tile_key + 15 >= group_low && (tile_key + 15 > group_last || tile_key < group_low)) {
 #pragma unroll
-                for (int pass = 0; pass < TILE_PASSES; ++pass) {
-                    const int element = (pass * kPrefillThreads + threadIdx.x) * 8;   // 2 dims x positions 4 g .. 4 g + 3
-                    const int first_key = tile_key + 4 * ((element / 64) % 4);
-                    PFrag8 values;
-                    values.raw = staged[t][1][pass];
+                    for (int pass = 0; pass < TILE_PASSES; ++pass) {
+                        const int element = (pass * kPrefillThreads + threadIdx.x) * 8;   // 2 dims x positions 4 g .. 4 g + 3
+                        const int first_key = tile_key + 4 * ((element / 64) % 4);
+                        PFrag8 values;
+                        values.raw = staged[t][1][pass];
 #pragma unroll
-                    for (int i = 0; i < 8; ++i)
-                        if (first_key + i % 4 > group_last || first_key + i % 4 < group_low) values.v[i] = static_cast<__bf16>(0.0f);
-                    staged[t][1][pass] = values.raw;
+                        for (int i = 0; i < 8; ++i)
+                            if (first_key + i % 4 > group_last || first_key + i % 4 < group_low) values.v[i] = static_cast<__bf16>(0.0f);
+                        staged[t][1][pass] = values.raw;
+                    }
                 }
             }
         }
