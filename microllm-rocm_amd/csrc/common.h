@@ -52,15 +52,20 @@ __device__ inline float sum_lanes_16_apart(float value) {
 template <typename T> __host__ __device__ inline T from_float(float value);
 template <> __host__ __device__ inline float from_float<float>(float value) { return value; }
 template <> __host__ __device__ inline bf16 from_float<bf16>(float value) {
+    bf16 out;
+#if defined(__HIP_DEVICE_COMPILE__)
+    // Round to nearest even in one instruction (v_cvt_pk_bf16_f32 of gfx950); a NaN stays a NaN.
+    out.bits = __builtin_bit_cast(uint16_t, static_cast<__bf16>(value));
+#else
     union { uint32_t u; float f; } caster;
     caster.f = value;
-    bf16 out;
     if ((caster.u & 0x7fffffffu) > 0x7f800000u) {  // NaN stays NaN
         out.bits = static_cast<uint16_t>((caster.u >> 16) | 0x0040u);
         return out;
     }
     const uint32_t rounding = 0x7fffu + ((caster.u >> 16) & 1u);
     out.bits = static_cast<uint16_t>((caster.u + rounding) >> 16);
+#endif
     return out;
 }
 
