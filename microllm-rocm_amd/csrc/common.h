@@ -27,6 +27,11 @@ __host__ __device__ inline float to_float(bf16 value) {
     return caster.f;
 }
 
+// A rotation by (cos, sin) with its roundings spelled out (one product rounded, then one fused multiply-add), so
+// that every kernel that rotates gives the same bits whatever the compiler would contract.
+__device__ inline float rotate_first(float x1, float x2, float c, float s) { return fmaf(x1, c, -(x2 * s)); }
+__device__ inline float rotate_second(float x1, float x2, float c, float s) { return fmaf(x1, s, x2 * c); }
+
 // op over the four lanes {l, l ^ 16, l ^ 32, l ^ 48} of a wave, every one of which gets the result: two
 // exchanges on the vector unit (v_permlane16_swap, v_permlane32_swap of gfx950) instead of four trips through
 // LDS. op must be commutative. (The elements of the builtins' result are copied to scalars before they are

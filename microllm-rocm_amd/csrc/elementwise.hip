@@ -239,8 +239,8 @@ __global__ void qkv_rope_store_kernel(const In* __restrict__ qkv, int n_partials
         float y1 = x1, y2 = x2;
         if (rotate) {
             const float c = cos_table[pair], s = sin_table[pair];
-            y1 = x1 * c - x2 * s;
-            y2 = x1 * s + x2 * c;
+            y1 = rotate_first(x1, x2, c, s);
+            y2 = rotate_second(x1, x2, c, s);
         }
         if (head < heads) {
             T* q_row = q_out + (static_cast<int64_t>(token) * heads + head) * head_dim;
@@ -255,6 +255,90 @@ __global__ void qkv_rope_store_kernel(const In* __restrict__ qkv, int n_partials
             v_cache[layout.v_at(page, kv_head, offset, first)] = from_float<T>(y1);
             v_cache[layout.v_at(page, kv_head, offset, second)] = from_float<T>(y2);
         }
+    }
+}
+
+// The same for float32 projections in the ordinary column order whose heads rotate whole (2 n_freq = head_dim, a
+// multiple of 8) with the step's table of cos and sin: a thread takes four pairs of a query or key head, or eight
+// dims of a value head, with 16-byte loads. out is bfloat16 or float32.
+template <typename T>
+__device__ inline void store_four(T* target, float a, float b, float c, float d);
+template <>
+__device__ inline void store_four<float>(float* target, float a, float b, float c, float d) {
+    *reinterpret_cast<float4*>(target) = make_float4(a, b, c, d);
+}
+template <>
+__device__ inline void store_four<bf16>(bf16* target, float a, float b, float c, float d) {
+    union { uint2 raw; bf16 v[4]; } four;
+    four.v[0] = from_float<bf16>(a);
+    four.v[1] = from_float<bf16>(b);
+    four.v[2] = from_float<bf16>(c);
+    four.v[3] = from_float<bf16>(d);
+    *reinterpret_cast<uint2*>(target) = four.raw;
+}
+
+template <typename T>
+__global__ void qkv_rope_store_vec4_kernel(const float* __restrict__ qkv, int n_partials, int64_t partial_stride,
+                                           const float* __restrict__ bias, const int32_t* __restrict__ slot_mapping,
+                                           const float2* __restrict__ cos_sin, T* __restrict__ q_out,
+                                           T* __restrict__ k_cache, T* __restrict__ v_cache, int n_tokens, int heads,
+                                           int kv_heads, int head_dim, int page_size) {
+    const int groups = head_dim / 8;                       // items per head
+    const int total_heads = heads + 2 * kv_heads;
+    const int64_t item = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (item >= static_cast<int64_t>(n_tokens) * total_heads * groups) return;
+    const int token = static_cast<int>(item / (total_heads * groups));
+    const int rest = static_cast<int>(item % (total_heads * groups));
+    const int head = rest / groups, group = rest % groups;
+    const bool is_value = head >= heads + kv_heads;
+    const int half = head_dim / 2;
+    // A query or key head: dims 4 g .. 4 g + 3 and their partners half a head on. A value head: dims 8 g .. 8 g + 7.
+    const int first = is_value ? 8 * group : 4 * group;
+    const int second = is_value ? first + 4 : first + half;
+    const int64_t column = static_cast<int64_t>(token) * total_heads * head_dim + head * head_dim;
+    float4 x1 = *reinterpret_cast<const float4*>(qkv + column + first);
+    float4 x2 = *reinterpret_cast<const float4*>(qkv + column + second);
+    for (int part = 1; part < n_partials; ++part) {
+        const float4 more1 = *reinterpret_cast<const float4*>(qkv + part * partial_stride + column + first);
+        const float4 more2 = *reinterpret_cast<const float4*>(qkv + part * partial_stride + column + second);
+        x1.x += more1.x; x1.y += more1.y; x1.z += more1.z; x1.w += more1.w;
+        x2.x += more2.x; x2.y += more2.y; x2.z += more2.z; x2.w += more2.w;
+    }
+    if (bias) {
+        const float4 b1 = *reinterpret_cast<const float4*>(bias + head * head_dim + first);
+        const float4 b2 = *reinterpret_cast<const float4*>(bias + head * head_dim + second);
+        x1.x += b1.x; x1.y += b1.y; x1.z += b1.z; x1.w += b1.w;
+        x2.x += b2.x; x2.y += b2.y; x2.z += b2.z; x2.w += b2.w;
+    }
+    float4 y1 = x1, y2 = x2;
+    if (!is_value) {
+        const float4* table = reinterpret_cast<const float4*>(cos_sin + static_cast<int64_t>(token) * half + first);
+        const float4 a = table[0], b = table[1];       // (cos, sin) of pairs first, first + 1 | first + 2, first + 3
+        y1.x = rotate_first(x1.x, x2.x, a.x, a.y);  y2.x = rotate_second(x1.x, x2.x, a.x, a.y);
+        y1.y = rotate_first(x1.y, x2.y, a.z, a.w);  y2.y = rotate_second(x1.y, x2.y, a.z, a.w);
+        y1.z = rotate_first(x1.z, x2.z, b.x, b.y);  y2.z = rotate_second(x1.z, x2.z, b.x, b.y);
+        y1.w = rotate_first(x1.w, x2.w, b.z, b.w);  y2.w = rotate_second(x1.w, x2.w, b.z, b.w);
+    }
+    if (head < heads) {
+        T* q_row = q_out + (static_cast<int64_t>(token) * heads + head) * head_dim;
+        store_four<T>(q_row + first, y1.x, y1.y, y1.z, y1.w);
+        store_four<T>(q_row + second, y2.x, y2.y, y2.z, y2.w);
+        return;
+    }
+    const int slot = slot_mapping ? slot_mapping[token] : -1;
+    if (slot < 0) return;
+    const CacheLayout layout(kv_heads, page_size, head_dim);
+    const int64_t page = slot / page_size;
+    const int offset = slot % page_size;
+    if (!is_value) {     // four dims that are a multiple of 4 lie side by side in a key page
+        const int kv_head = head - heads;
+        store_four<T>(k_cache + layout.k_at(page, kv_head, offset, first), y1.x, y1.y, y1.z, y1.w);
+        store_four<T>(k_cache + layout.k_at(page, kv_head, offset, second), y2.x, y2.y, y2.z, y2.w);
+    } else {             // in a value page the positions of a dim lie side by side, not the dims
+        const int kv_head = head - heads - kv_heads;
+        const float values[8] = {y1.x, y1.y, y1.z, y1.w, y2.x, y2.y, y2.z, y2.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v_cache[layout.v_at(page, kv_head, offset, first + i)] = from_float<T>(values[i]);
     }
 }
 
@@ -371,6 +455,25 @@ int mll_qkv_rope_store(const void* qkv, int in_dtype, int n_partials, int64_t pa
     // A block takes as many heads of one token as give its 256 threads one pair each.
     const int heads_per_block = max(1, 256 / (head_dim / 2));
     const dim3 grid(n_tokens, (heads + 2 * kv_heads + heads_per_block - 1) / heads_per_block);
+    const bool wide = in_dtype == kF32 && cos_sin != nullptr && !pair_order && 2 * n_freq == head_dim && head_dim % 8 == 0 &&
+                      n_tokens > 64 && reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && partial_stride % 4 == 0 &&
+                      reinterpret_cast<uintptr_t>(cos_sin) % 16 == 0 && (bias == nullptr || reinterpret_cast<uintptr_t>(bias) % 16 == 0) &&
+                      reinterpret_cast<uintptr_t>(q_out) % 16 == 0 && reinterpret_cast<uintptr_t>(k_cache) % 16 == 0;
+    if (wide) {
+        const int64_t items = static_cast<int64_t>(n_tokens) * (heads + 2 * kv_heads) * (head_dim / 8);
+        const unsigned blocks = static_cast<unsigned>((items + 255) / 256);
+        if (dtype == kF32)
+            qkv_rope_store_vec4_kernel<float><<<blocks, 256, 0, stream>>>(
+                static_cast<const float*>(qkv), n_partials, partial_stride, bias, slot_mapping, static_cast<const float2*>(cos_sin),
+                static_cast<float*>(q_out), static_cast<float*>(k_cache), static_cast<float*>(v_cache), n_tokens, heads, kv_heads,
+                head_dim, page_size);
+        else
+            qkv_rope_store_vec4_kernel<bf16><<<blocks, 256, 0, stream>>>(
+                static_cast<const float*>(qkv), n_partials, partial_stride, bias, slot_mapping, static_cast<const float2*>(cos_sin),
+                static_cast<bf16*>(q_out), static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache), n_tokens, heads, kv_heads,
+                head_dim, page_size);
+        return check_launch("qkv_rope_store");
+    }
     if (dtype == kF32 && in_dtype == kF32) {
         qkv_rope_store_kernel<float, float><<<grid, 256, 0, stream>>>(
             static_cast<const float*>(qkv), n_partials, partial_stride, bias, positions, slot_mapping, inv_freq, static_cast<const float2*>(cos_sin), n_freq,

@@ -270,8 +270,8 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
                     float y1 = x1, y2 = x2;
                     if (rotate) {
                         const float c = cos_sin[nt][i / 2].x, sn = cos_sin[nt][i / 2].y;
-                        y1 = x1 * c - x2 * sn;
-                        y2 = x1 * sn + x2 * c;
+                        y1 = rotate_first(x1, x2, c, sn);
+                        y2 = rotate_second(x1, x2, c, sn);
                     }
                     if (is_query) {
                         q_row[first] = from_float<bf16>(y1);

@@ -143,6 +143,37 @@ def test_qkv_rope_store(in_dtype, out_dtype, heads, kv_heads, hd, rotary, page_s
     assert np.all(k_host.transpose(0, 2, 1, 3)[~written] == 7.0) and np.all(v_host.transpose(0, 2, 1, 3)[~written] == 7.0)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv_heads,hd,page_size,parts", [(5, 5, 48, 16, 1), (6, 2, 16, 48, 3), (28, 4, 128, 16, 1), (3, 0, 24, 16, 2)])
+def test_qkv_rope_store_with_many_tokens_takes_the_same_values(out_dtype, heads, kv_heads, hd, page_size, parts):
+    """Many tokens with a table of cos and sin take the 16-byte kernel: the same bits as the kernel that goes pair by pair."""
+    rng = np.random.default_rng(heads + hd)
+    tokens, pages = 150, 12
+    total = (heads + 2 * kv_heads) * hd
+    qkv = torch.from_numpy(rng.normal(size=(parts, tokens, total)).astype(np.float32)).to(DEVICE)
+    qkv = qkv[0].contiguous() if parts == 1 else qkv
+    bias = torch.from_numpy(rng.normal(size=total).astype(np.float32)).to(DEVICE)
+    positions = torch.from_numpy(rng.integers(0, 30000, size=tokens).astype(np.int32)).to(DEVICE)
+    slots_host = rng.permutation(pages * page_size)[:tokens].astype(np.int32)
+    slots_host[5] = -1
+    slots = torch.from_numpy(slots_host).to(DEVICE) if kv_heads else None
+    inv_freq = torch.tensor(1e6 ** (-np.arange(0, hd, 2, dtype=np.float64) / hd), dtype=torch.float64, device=DEVICE)
+    table = kernels().rope_table(positions, inv_freq)
+
+    def run(**how):
+        k_pages = torch.full(key_page_shape(pages, kv_heads, page_size, hd), 7.0, dtype=out_dtype, device=DEVICE) if kv_heads else None
+        v_pages = torch.full(value_page_shape(pages, kv_heads, page_size, hd), 7.0, dtype=out_dtype, device=DEVICE) if kv_heads else None
+        q = kernels().qkv_rope_store(qkv, bias, positions, slots, how.get("inv_freq"), k_pages, v_pages, heads, kv_heads, hd,
+                                     page_size, out_dtype, cos_sin=how.get("cos_sin"))
+        return q, k_pages, v_pages
+
+    wide = run(cos_sin=table)
+    narrow = run(inv_freq=inv_freq)
+    assert torch.equal(wide[0], narrow[0])
+    if kv_heads:
+        assert torch.equal(wide[1], narrow[1]) and torch.equal(wide[2], narrow[2])
+
+
 def test_rope_vector_of_the_reference_and_large_positions():
     # tests/ops/ops_test.cpp:505-515: {5,6,7,8} at p=1, hd=4, base 10000
     qkv = torch.tensor([[5.0, 6.0, 7.0, 8.0]], device=DEVICE)
