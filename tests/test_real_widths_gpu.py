@@ -1,0 +1,75 @@
+"""Two layers at the widths of real models (the sizes the kernels are tuned and measured at) against the plain
+implementation: a head size of 128 with 7 query heads a group, a head size of 64, reductions of 18944, a vocabulary
+that is no power of two. Whole prompts, then decoding, and mixed batches on reused pages, in both dtypes."""
+import io
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from microllm_rocm_amd.config import Qwen2Config
+from microllm_rocm_amd.weights import write_model_folder
+from replay_tools import PlainModel, collect, compare, mixed, prefill_then_decode, round_up, to_lines, whole
+from tiny import random_tokens
+
+pytestmark = pytest.mark.gpu
+
+WIDE = {
+    "7b": Qwen2Config(vocab_size=20011, hidden_size=3584, num_hidden_layers=2, num_attention_heads=28, num_key_value_heads=4,
+                      head_dim=128, intermediate_size=18944, max_position_embeddings=4096, rope_theta=1e6, rms_norm_eps=1e-6,
+                      tie_word_embeddings=False),
+    "0.5b": Qwen2Config(vocab_size=15013, hidden_size=896, num_hidden_layers=2, num_attention_heads=14, num_key_value_heads=2,
+                        head_dim=64, intermediate_size=4864, max_position_embeddings=4096, rope_theta=1e6, rms_norm_eps=1e-6,
+                        tie_word_embeddings=True),
+}
+_models = {}
+
+
+def model_for(tmp_path_factory, which):
+    if which not in _models:
+        folder = os.path.join(str(tmp_path_factory.mktemp(f"wide_{which}")), "model")
+        # Larger weights than N(0, 0.02): the logits of two layers would else be all but the embedding's own.
+        write_model_folder(folder, WIDE[which], seed=11, dtype=torch.bfloat16, stds={"std": 0.04, "norm_std": 0.1})
+        _models[which] = (folder, PlainModel(folder))
+    return _models[which]
+
+
+def run_trace(folder, dtype, steps, out_dir, max_tokens):
+    from microllm_rocm_amd.engine import Engine
+    from microllm_rocm_amd.engine.replay import replay
+    engine = Engine.from_folder(folder, dtype=dtype, max_tokens=max_tokens, max_requests=8)
+    replay(engine, io.StringIO(to_lines(steps)), str(out_dir), io.StringIO())
+    engine.cache.check()
+    assert not engine.cache.requests
+    return engine
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["7b", "0.5b"])
+def test_real_widths_match_the_plain_implementation(tmp_path_factory, tmp_path, which, dtype):
+    config = WIDE[which]
+    folder, plain_model = model_for(tmp_path_factory, which)
+    requests = {f"r{index}": random_tokens(40 + index, length, config.vocab_size) for index, length in enumerate([150, 70, 40, 33, 64, 50, 81])}
+    # every request whole in one step (many rows: the library's products and the prompt kernels in bfloat16)
+    steps = whole(requests)
+    run_trace(folder, dtype, steps, tmp_path / "whole", max_tokens=round_up(sum(len(t) for t in requests.values()), 64) + 256)
+    together = collect(steps, tmp_path / "whole", config.vocab_size)
+    compare(together, requests, plain_model, dtype)
+    # most of a request in one step, the last 32 tokens one by one (few rows: the streaming products and their epilogues)
+    steps = prefill_then_decode("r0", requests["r0"], tail=32)
+    run_trace(folder, dtype, steps, tmp_path / "decode", max_tokens=round_up(len(requests["r0"]), 64))
+    decoded = collect(steps, tmp_path / "decode", config.vocab_size)
+    compare(decoded, {"r0": requests["r0"]}, plain_model, dtype)
+    # portions of some beside decoded tokens of others, on a pool so small that pages are used again
+    steps, peak = mixed(requests, seed=5)
+    engine = run_trace(folder, dtype, steps, tmp_path / "mixed", max_tokens=peak)
+    pool = engine.cache.groups[0].pool
+    assert pool.total_taken > pool.num_pages
+    got = collect(steps, tmp_path / "mixed", config.vocab_size)
+    compare(got, requests, plain_model, dtype)
+    if dtype == "float32":
+        for key, row in got.items():
+            assert np.array_equal(row, together[key]), f"mixed: {key} differs from the request run whole"
+        for key, row in decoded.items():
+            assert np.array_equal(row, together[key]), f"decoding: {key} differs from the request run whole"
