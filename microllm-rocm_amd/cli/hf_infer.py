@@ -28,7 +28,7 @@ OPTIONS: Dict[str, object] = {
     # this engine's own
     "model": None, "dtype": "bfloat16", "temperature": 0.0, "sample-top-k": 0, "seed": 1, "stop-tokens": "",
     "block-size": 16, "num-blocks": 0, "max-batched-tokens": 2048, "prefill-chunk": 512, "max-requests": 64,
-    "random-config": None, "prompt-lengths": "", "prompt-seed": 0, "use-graphs": "true",
+    "random-config": None, "prompt-lengths": "", "prompt-seed": 0, "use-graphs": "true", "weight-copies": "auto",
 }
 
 
@@ -145,7 +145,8 @@ def run(options: Dict[str, object]) -> int:
     max_tokens = None if num_blocks else max(needed, capacity * batch, block_size)
     engine_options = dict(dtype=dtype, device="cuda:0", page_size=block_size, max_tokens=max_tokens, num_pages=num_blocks,
                           max_requests=max(int(options["max-requests"]), batch),
-                          use_graphs=boolean(str(options["use-graphs"]), "--use-graphs"))
+                          use_graphs=boolean(str(options["use-graphs"]), "--use-graphs"),
+                          weight_copies=str(options["weight-copies"]))
     if model_dir is not None:
         engine = Engine.from_folder(str(model_dir), **engine_options)
     else:
@@ -163,7 +164,7 @@ def run(options: Dict[str, object]) -> int:
               "architecture": engine.spec.architecture, "compute_dtype": dtype, "workload": options["workload"],
               "load_ms": round(load_ms, 3), "token_count": len(tokens), "batch": batch,
               "kv_block_size": block_size, "kv_blocks": engine.cache.groups[0].pool.num_pages if engine.cache.groups else 0,
-              "allocated_cache_bytes": engine.cache.allocated_bytes()}
+              "allocated_cache_bytes": engine.cache.allocated_bytes(), "weight_copies": engine.weight_copies}
     stop_tokens = tuple(integers(str(options["stop-tokens"]), "--stop-tokens"))
     params = GenerationConfig(max_new_tokens=new_tokens, temperature=float(options["temperature"]),
                               top_k=int(options["sample-top-k"]), seed=int(options["seed"]), stop_tokens=stop_tokens)

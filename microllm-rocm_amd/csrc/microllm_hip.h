@@ -141,6 +141,12 @@ struct MllSkinnyExtras {
 int mll_gemm_medium(const void* a, const void* w_packed, void* out, int epilogue, int m, int n, int k,
                     int tiles_per_wave, int waves, int splits, hipStream_t stream);
 
+// The same product for many rows: 256 x 256 tiles of C per workgroup, pieces of A and W brought into LDS by
+// direct global-to-LDS loads. A is row-major [m, k] with k a multiple of 32; epilogues 0, 1 and 2 of
+// mll_gemm_skinny. For weights that are kept in the packed order alone.
+int mll_gemm_tiled(const void* a, const void* w_packed, void* out, int epilogue, int m, int n, int k,
+                   hipStream_t stream);
+
 // Index of the first maximum of each row; a row that holds a non-finite value gives -1.
 // `parts` is device scratch of n_rows * mll_argmax_slices(vocab) * 16 bytes (contents need not be cleared).
 int mll_argmax(const float* logits, int32_t* out, void* parts, int n_rows, int vocab, hipStream_t stream);

@@ -80,25 +80,33 @@ def prefill_throughput(engine: Engine, tokens: int, repeats: int = 3, seed: int 
 
 def weight_bytes(engine: Engine) -> int:
     """Bytes of every weight a decode step reads once: all layers, the final norm and the head (an embedding
-    table that is not the head's is read one row per token, which is counted apart)."""
-    seen, total = set(), 0
-    embedding_only = None
+    table that is not the head's is read one row per token, which is counted apart). A matrix counts once,
+    at its own size, whichever of its copies (as stored, packed) the step reads."""
     model = engine.model
-    if model.embedding.table.data_ptr() != model.head.weight.tensor.data_ptr():
-        embedding_only = model.embedding.table.data_ptr()
-    tensors = [model.final_norm.weight, model.head.weight.tensor]
+    total = 0
+    seen = set()
+
+    def count(value) -> int:
+        if isinstance(value, Weight):
+            kept = value.tensor if value.tensor is not None else value.packed
+            if kept.data_ptr() in seen:
+                return 0
+            seen.add(kept.data_ptr())
+            return value.out_features * value.in_features * kept.element_size()
+        if isinstance(value, torch.Tensor):
+            if value.data_ptr() in seen:
+                return 0
+            seen.add(value.data_ptr())
+            return value.numel() * value.element_size()
+        return 0
+
+    total += count(model.final_norm.weight) + count(model.head.weight)
     for block in model.blocks:
         for part in block.parts():
-            tensors += [value for value in vars(part).values() if isinstance(value, torch.Tensor)]
-            tensors += [value.tensor for value in vars(part).values() if isinstance(value, Weight)]
+            total += sum(count(value) for value in vars(part).values())
             position = getattr(part, "position", None)
             if position is not None:
-                tensors += [value for value in vars(position).values() if isinstance(value, torch.Tensor)]
-    for tensor in tensors:
-        if tensor.data_ptr() in seen or tensor.data_ptr() == embedding_only:
-            continue
-        seen.add(tensor.data_ptr())
-        total += tensor.numel() * tensor.element_size()
+                total += sum(count(value) for value in vars(position).values())
     return total
 
 
@@ -121,11 +129,11 @@ def step_flops(engine: Engine, tokens: int) -> float:
         for part in block.parts():
             for name, value in vars(part).items():
                 if isinstance(value, Weight):
-                    flops += 2.0 * value.tensor.numel() * tokens
+                    flops += 2.0 * value.out_features * value.in_features * tokens
         mixer = block.mixer
         if hasattr(mixer, "heads"):
             window = mixer.window or tokens
             pairs = sum(min(position + 1, window) for position in range(tokens))
             flops += 4.0 * mixer.heads * mixer.head_dim * pairs
-    flops += 2.0 * engine.model.head.weight.tensor.numel()
+    flops += 2.0 * engine.model.head.weight.out_features * engine.model.head.weight.in_features
     return flops

@@ -53,7 +53,12 @@ class Engine:
     def __init__(self, spec: ModelSpec, tensors: Mapping[str, torch.Tensor], dtype: Union[str, torch.dtype] = "bfloat16",
                  device: Union[str, torch.device] = "cuda:0", page_size: int = 16,
                  max_tokens: Optional[int] = None, num_pages: Optional[int] = None, max_requests: int = 64,
-                 tensors_placed: bool = False, use_graphs: bool = True):
+                 tensors_placed: bool = False, use_graphs: bool = True, weight_copies: str = "auto",
+                 consume_tensors: bool = False):
+        """``weight_copies``: a bfloat16 weight is kept ``"both"`` as stored (for the library's product of steps
+        with many rows) and packed (for the streaming products), or ``"packed"`` only, where memory is short;
+        ``"auto"`` keeps both if two copies and the cache fit the GPU's memory. With ``consume_tensors`` the
+        entries of ``tensors`` (a dict) are taken out as the parts take them."""
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU is visible; this engine has no CPU path")
         library.load()  # fail now, and loudly, if the kernels are missing and cannot be built
@@ -61,17 +66,23 @@ class Engine:
         self.device = torch.device(device)
         torch.cuda.set_device(self.device)
         self.spec = spec
-        self.runtime = Runtime(dtype=self.dtype, device=self.device)
-        self.model = Model(spec, self.runtime)
-        decls = self.model.tensors()
-        if not tensors_placed:
-            tensors = place_all(tensors, decls, self.dtype, self.device)
-        self.model.bind(tensors)
-        del tensors
         if num_pages is None:
             if max_tokens is None:
                 raise ValueError("give max_tokens or num_pages: the cache pool is sized once")
             num_pages = max(1, -(-max_tokens // page_size))
+        if weight_copies not in ("auto", "both", "packed"):
+            raise ValueError("weight_copies is 'auto', 'both' or 'packed'")
+        probe = Model(spec, Runtime(dtype=self.dtype, device=self.device))
+        decls = probe.tensors()
+        if weight_copies == "auto":
+            weight_copies = "both" if self._two_copies_fit(probe, decls, num_pages, page_size) else "packed"
+        self.weight_copies = weight_copies
+        self.runtime = Runtime(dtype=self.dtype, device=self.device, keep_plain_weights=weight_copies == "both")
+        self.model = Model(spec, self.runtime)
+        placed = tensors if tensors_placed else place_all(tensors, decls, self.dtype, self.device, consume=consume_tensors)
+        consume = consume_tensors or not tensors_placed
+        self.model.bind(placed if isinstance(placed, dict) else dict(placed), consume=consume)
+        del tensors, placed
         reads = [entry.reads_cache_of for entry in spec.order]
         self.cache = CacheManager(self.model.cache_needs(), reads, page_size, num_pages, max_requests,
                                   dtype=self.dtype, device=self.device,
@@ -85,6 +96,19 @@ class Engine:
         self._graphs: Dict[tuple, "_DecodeGraph"] = {}
         self.graph_replays = 0
 
+    def _two_copies_fit(self, model: Model, decls, num_pages: int, page_size: int) -> bool:
+        """Whether the weights as stored, their packed copies and the cache pool fit the GPU with a tenth to spare."""
+        if self.dtype != torch.bfloat16:
+            return True     # a float32 engine has no packed copies
+        element = 2
+        weights = sum(element * int(torch.Size(decl.shape).numel()) for decl in decls.values())
+        cache = 0
+        for need in model.cache_needs():
+            if need is not None and hasattr(need, "kv_heads"):
+                cache += 2 * num_pages * page_size * need.kv_heads * need.head_dim * element
+        total = torch.cuda.get_device_properties(self.device).total_memory
+        return 2 * weights + cache <= 0.9 * total
+
     # ---- construction --------------------------------------------------------------------
     @classmethod
     def from_folder(cls, folder: str, dtype: Union[str, torch.dtype] = "bfloat16", device="cuda:0", **options) -> "Engine":
@@ -94,7 +118,7 @@ class Engine:
         engine_dtype = parse_dtype(dtype)
         probe = Model(spec, Runtime(dtype=engine_dtype, device=torch.device("cpu")))
         tensors = load_folder(folder, probe.tensors(), engine_dtype, torch.device(device))
-        engine = cls(spec, tensors, dtype=engine_dtype, device=device, tensors_placed=True, **options)
+        engine = cls(spec, tensors, dtype=engine_dtype, device=device, tensors_placed=True, consume_tensors=True, **options)
         engine.config = config
         return engine
 
@@ -108,7 +132,7 @@ class Engine:
         probe = Model(spec, Runtime(dtype=engine_dtype, device=torch.device("cpu")))
         tensors = random_tensors(probe.tensors(), architecture.init_rules(config), seed, dtype=torch.bfloat16,
                                  stds=stds, device=device if on_device else "cpu")
-        engine = cls(spec, tensors, dtype=engine_dtype, device=device, **options)
+        engine = cls(spec, tensors, dtype=engine_dtype, device=device, consume_tensors=True, **options)
         engine.config = config
         return engine
 

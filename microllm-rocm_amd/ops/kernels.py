@@ -640,3 +640,26 @@ def gemm_medium(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "
         raise KernelLibraryError(f"unknown epilogue {epilogue!r}")
     _check(lib.mll_gemm_medium(_ptr(x), _ptr(packed), _ptr(out), code, m, n, k, tiles_per_wave, waves, splits, _stream()), lib)
     return out
+
+
+def gemm_tiled(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f32") -> torch.Tensor:
+    """``x @ W.T`` for many bfloat16 rows and a packed weight, on this package's tiled MFMA kernel (about half
+    the library's rate: for weights that are kept in the packed order alone). ``k`` must be a multiple of 32."""
+    lib = library.load()
+    _device_tensor(x, "gemm input", torch.bfloat16)
+    _device_tensor(packed, "packed weight", torch.bfloat16)
+    _need(x.dim() == 2 and packed.dim() == 5 and tuple(packed.shape[2:]) == (4, 16, 8), "gemm_tiled takes [m, k] and a packed weight")
+    m, k = x.shape
+    _need(k % 32 == 0, "gemm_tiled needs k to be a multiple of 32")
+    _need(packed.shape[0] == -(-n // 16) and packed.shape[1] == k // 32, "the packed weight does not fit n and k")
+    if epilogue == "f32":
+        code, out = 0, torch.empty((m, n), dtype=torch.float32, device=x.device)
+    elif epilogue == "bf16":
+        code, out = 1, torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    elif epilogue == "gated":
+        _need(n % 2 == 0, "the gated epilogue needs an even number of weight rows")
+        code, out = 2, torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
+    else:
+        raise KernelLibraryError(f"unknown epilogue {epilogue!r}")
+    _check(lib.mll_gemm_tiled(_ptr(x), _ptr(packed), _ptr(out), code, m, n, k, _stream()), lib)
+    return out

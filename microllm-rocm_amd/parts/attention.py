@@ -70,11 +70,13 @@ class PagedAttention(Mixer):
         if (self.position is None or self.position.fused_split_half) and self.head_dim % 16 == 0:
             n_freq = self.position.inv_freq.shape[0] if self.position is not None else 0
             order = kernels.rotary_pair_order(self.heads, self.kv_heads if self.owns_kv else 0, self.head_dim, n_freq)
-        self.qkv_weight = Weight(torch.cat(weights, dim=0).contiguous() if len(weights) > 1 else weights[0], row_order=order)
+        self.qkv_weight = Weight(torch.cat(weights, dim=0).contiguous() if len(weights) > 1 else weights[0], row_order=order,
+                                 keep_plain=self.runtime.keep_plain_weights)
+        del weights
         if self.qkv_bias:
             biases = [tensors[self.name(f"{role}_proj.bias")] for role, _ in self._projections()]
             self.qkv_bias_vector = torch.cat(biases, dim=0).contiguous() if len(biases) > 1 else biases[0]
-        self.o_weight = Weight(tensors[self.name("o_proj.weight")])
+        self.o_weight = Weight(tensors[self.name("o_proj.weight")], keep_plain=self.runtime.keep_plain_weights)
 
     def cache_need(self):
         if not self.owns_kv:

@@ -27,9 +27,12 @@ class TensorDecl:
 
 @dataclass(frozen=True)
 class Runtime:
-    """What a part needs of the engine: the element type of activations and pages, and the device."""
+    """What a part needs of the engine: the element type of activations and pages, the device, and whether a
+    bfloat16 weight keeps its copy as stored beside the packed one (False: one copy, where memory is short;
+    steps with many rows then go through the streaming products 64 rows at a time)."""
     dtype: torch.dtype
     device: torch.device
+    keep_plain_weights: bool = True
 
 
 @dataclass(frozen=True)

@@ -39,8 +39,9 @@ class SwiGLU(FeedForward):
         up = tensors[self.name("up_proj.weight")]
         if gate.dtype != up.dtype:
             raise TypeError("the gate and up weights of one layer must share a dtype to be stacked")
-        self.gate_up_weight = Weight(torch.cat([gate, up], dim=0).contiguous(), gated=True)
-        self.down_weight = Weight(tensors[self.name("down_proj.weight")])
+        self.gate_up_weight = Weight(torch.cat([gate, up], dim=0).contiguous(), gated=True, keep_plain=self.runtime.keep_plain_weights)
+        del gate, up
+        self.down_weight = Weight(tensors[self.name("down_proj.weight")], keep_plain=self.runtime.keep_plain_weights)
 
     def takes_unscaled(self, rows: int) -> bool:
         return takes_unscaled(self.gate_up_weight, rows)

@@ -22,18 +22,17 @@ class Weight:
     """A linear's weight ``[out, in]`` and, for bfloat16, its packed copy."""
 
     def __init__(self, tensor: torch.Tensor, gated: bool = False, pack: bool = True,
-                 row_order: Optional[torch.Tensor] = None):
-        self.tensor = tensor
+                 row_order: Optional[torch.Tensor] = None, keep_plain: bool = True):
+        self.tensor: Optional[torch.Tensor] = tensor
+        self.dtype = tensor.dtype
         self.out_features, self.in_features = tensor.shape
         self.gated = gated   # rows are [gate; up]: the packed copy interleaves them for the fused epilogue
         self.row_order = row_order   # the packed copy's rows in another order: its products' columns come in that order
         self.packed: Optional[torch.Tensor] = None
         if pack and tensor.is_cuda and tensor.dtype == torch.bfloat16 and self.in_features % 8 == 0:
             self.packed = kernels.pack_weight(tensor, interleave_halves=gated, row_order=row_order)
-
-    @property
-    def dtype(self) -> torch.dtype:
-        return self.tensor.dtype
+            if not keep_plain:
+                self.tensor = None   # the packed copy serves every number of rows
 
 
 MAX_FACTOR_WIDTH = 8192   # the widest norm whose rows' factors the streaming product applies (its sums sit in LDS)
@@ -90,7 +89,7 @@ def takes_packed(weight: "Weight", rows: int, gated: bool = False) -> bool:
     """Whether ``linear`` multiplies this many rows with the packed copy (whose rows may be in ``row_order``)."""
     if weight.packed is None:
         return False
-    if rows <= SKINNY_ROWS:
+    if rows <= SKINNY_ROWS or weight.tensor is None:
         return True
     wide = -(-weight.out_features // 16) >= MEDIUM_WIDE_TILES
     return not gated and rows <= (MEDIUM_WIDE_ROWS if wide else MEDIUM_ROWS)
@@ -114,21 +113,31 @@ def linear(x: Union[torch.Tensor, UnscaledRows], weight, out_dtype: Optional[tor
             raise TypeError("this product cannot apply the rows' factors; see takes_unscaled")
         x, scale = x.values, x.scale
     w = weight.tensor
-    if w.dtype == torch.float32:
+    if weight.dtype == torch.float32:
         # True 32-bit product, also for a 32-bit weight inside a bfloat16 engine.
         a = x if x.dtype == torch.float32 else x.to(torch.float32)
         y = kernels.gemm_f32(a, w)
         if gated:
             return kernels.silu_mul(y if x.dtype == torch.float32 else y.to(x.dtype))
         return y if out_dtype == torch.float32 else y.to(out_dtype)
-    if x.dtype != w.dtype:
-        raise TypeError(f"cannot multiply {x.dtype} activations with a {w.dtype} weight")
+    if x.dtype != weight.dtype:
+        raise TypeError(f"cannot multiply {x.dtype} activations with a {weight.dtype} weight")
     rows = x.shape[0]
     if weight.packed is not None and rows <= SKINNY_ROWS:
         if gated:
             return kernels.gemm_skinny(x, weight.packed, weight.out_features, "gated", scale=scale)
         return kernels.gemm_skinny(x, weight.packed, weight.out_features, "bf16" if out_dtype == torch.bfloat16 else "f32",
                                    scale=scale)
+    if w is None:
+        # Only the packed copy is kept: many rows go through this package's tiled product, or, where the
+        # reduction is no multiple of 32, through the product for 64 rows, a piece at a time.
+        epilogue = "gated" if gated else ("f32" if out_dtype == torch.float32 else "bf16")
+        if weight.in_features % 32 == 0:
+            return kernels.gemm_tiled(x, weight.packed, weight.out_features, epilogue)
+        plan = kernels.medium_plan(weight.out_features, weight.in_features, may_split=False)
+        pieces = [kernels.gemm_medium(x[first:first + MEDIUM_ROWS], weight.packed, weight.out_features, epilogue, plan=plan)
+                  for first in range(0, rows, MEDIUM_ROWS)]
+        return pieces[0] if len(pieces) == 1 else torch.cat(pieces)
     if takes_packed(weight, rows, gated):
         if out_dtype == torch.float32:
             plan = kernels.medium_plan(weight.out_features, weight.in_features, may_split=partials)

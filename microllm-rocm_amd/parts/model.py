@@ -56,7 +56,7 @@ class LMHead(Part):
         return {self.name("weight"): TensorDecl((self.vocab, self.width), MATRIX)}
 
     def bind(self, tensors):
-        self.weight = Weight(tensors[self.name("weight")])
+        self.weight = Weight(tensors[self.name("weight")], keep_plain=self.runtime.keep_plain_weights)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return linear(x, self.weight, out_dtype=torch.float32)
@@ -64,6 +64,24 @@ class LMHead(Part):
 
 register_part("embedding", "token_embedding", TokenEmbedding)
 register_part("head", "lm_head", LMHead)
+
+
+class _HandOver:
+    """A mapping that lets go of an entry when it has been looked up as often as parts declared it."""
+
+    def __init__(self, tensors: dict, declarations):
+        self._tensors = tensors
+        self._uses: Dict[str, int] = {}
+        for declared in declarations:
+            for name in declared:
+                self._uses[name] = self._uses.get(name, 0) + 1
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        self._uses[name] = self._uses.get(name, 1) - 1
+        return self._tensors.pop(name) if self._uses[name] <= 0 else self._tensors[name]
+
+    def __contains__(self, name: str) -> bool:
+        return name in self._tensors
 
 
 class Model:
@@ -93,7 +111,12 @@ class Model:
         add(self.head.tensors())
         return decls
 
-    def bind(self, tensors: Mapping[str, torch.Tensor]) -> None:
+    def bind(self, tensors: Mapping[str, torch.Tensor], consume: bool = False) -> None:
+        """Hand every part its tensors. With ``consume`` (``tensors`` must be a dict) an entry is taken out of
+        ``tensors`` when the last part that declared it has looked it up, so that what a part does not keep
+        (a weight it only needed to pack or stack) is freed at once, not when loading ends."""
+        if consume:
+            tensors = _HandOver(tensors, [part.tensors() for part in self.parts()])
         self.embedding.bind(tensors)
         for block in self.blocks:
             block.bind(tensors)

@@ -82,7 +82,12 @@ def load_folder(folder: str, decls: Mapping[str, TensorDecl], engine_dtype: torc
 
 
 def place_all(tensors: Mapping[str, torch.Tensor], decls: Mapping[str, TensorDecl], engine_dtype: torch.dtype,
-              device: torch.device) -> Dict[str, torch.Tensor]:
-    """The same checks and placement for tensors that are already in memory."""
+              device: torch.device, consume: bool = False) -> Dict[str, torch.Tensor]:
+    """The same checks and placement for tensors that are already in memory. With ``consume`` (``tensors`` must
+    be a dict) every entry is taken out of ``tensors`` as it is placed, so that a copy replaces its source
+    instead of standing beside it."""
     check_names_and_shapes(decls, {name: tuple(t.shape) for name, t in tensors.items()})
-    return {name: place(tensors[name], decl, engine_dtype, device) for name, decl in decls.items()}
+    placed: Dict[str, torch.Tensor] = {}
+    for name, decl in decls.items():
+        placed[name] = place(tensors.pop(name) if consume else tensors[name], decl, engine_dtype, device)
+    return placed

@@ -586,6 +586,32 @@ def test_gemm_medium(m, n, k):
     assert torch.equal(alone[..., 0, :], parts[..., m - 1, :])
 
 
+@pytest.mark.parametrize("m,n,k", [(300, 1000, 256), (257, 272, 64), (65, 331, 96), (2048, 4608, 512), (700, 3584, 2048)])
+def test_gemm_tiled(m, n, k):
+    """The tiled product for many rows over a packed weight (what an engine with one copy of its weights takes)."""
+    rng = np.random.default_rng(m + n)
+    a_ref, a = to_bf16_exact(rng.normal(size=(m, k)))
+    w_ref, w = to_bf16_exact(rng.normal(size=(n, k)) * 0.1)
+    ka = kernels()
+    packed = ka.pack_weight(w)
+    expected = a_ref @ w_ref.T
+    scale = np.abs(expected).max()
+    full = ka.gemm_tiled(a, packed, n, "f32")
+    assert full.dtype == torch.float32 and full.shape == (m, n)
+    assert np.abs(full.double().cpu().numpy() - expected).max() <= 1e-5 * scale
+    out = ka.gemm_tiled(a, packed, n, "bf16")
+    assert out.dtype == torch.bfloat16 and np.abs(out.float().cpu().numpy() - expected).max() <= 5e-3 * scale
+    if n % 2 == 0:
+        gated = ka.gemm_tiled(a, ka.pack_weight(w, interleave_halves=True), n, "gated")
+        wanted = plain.silu(expected[:, : n // 2]) * expected[:, n // 2:]
+        np.testing.assert_allclose(gated.float().cpu().numpy(), wanted, rtol=1.2e-2, atol=1.2e-2 * np.abs(wanted).max())
+    # the same in every run, and a row's result does not depend on the other rows of the call
+    assert torch.equal(ka.gemm_tiled(a, packed, n, "f32"), full)
+    assert torch.equal(ka.gemm_tiled(a[m - 70:].contiguous(), packed, n, "f32"), full[m - 70:]) if m > 70 else True
+    with pytest.raises(Exception, match="multiple of 32"):
+        ka.gemm_tiled(a[:, :k - 8].contiguous(), ka.pack_weight(w[:, :k - 8].contiguous()), n)
+
+
 @pytest.mark.parametrize("m,width,k", [(20, 203, 96), (64, 176, 64), (33, 1000, 520)])
 def test_gemm_medium_gated_epilogue(m, width, k):
     rng = np.random.default_rng(width + 1)

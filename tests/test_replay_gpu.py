@@ -30,11 +30,11 @@ def model_for(tmp_path_factory, which, stds):
     return _models[key]
 
 
-def run_trace(folder, dtype, steps, out_dir, max_tokens):
+def run_trace(folder, dtype, steps, out_dir, max_tokens, **options):
     """In-process replay: the same ``replay`` that bin/trace_run calls, on a fresh engine."""
     from microllm_rocm_amd.engine import Engine
     from microllm_rocm_amd.engine.replay import replay
-    engine = Engine.from_folder(folder, dtype=dtype, max_tokens=max_tokens, max_requests=8)
+    engine = Engine.from_folder(folder, dtype=dtype, max_tokens=max_tokens, max_requests=8, **options)
     report = io.StringIO()
     replay(engine, io.StringIO(to_lines(steps)), str(out_dir), report)
     assert report.getvalue().split() == [word for step in steps for word in ("done", str(step["step"]))]
@@ -120,6 +120,26 @@ def test_the_first_tokens_and_long_decoding(tmp_path_factory, tmp_path, dtype):
         steps = whole({"first": tokens[:count]})
         run_trace(folder, dtype, steps, tmp_path / f"first{count}", max_tokens=64)
         compare(collect(steps, tmp_path / f"first{count}", config.vocab_size), {"first": tokens[:count]}, plain_model, dtype)
+
+
+@pytest.mark.parametrize("which", ["B", "C"])
+def test_one_copy_of_the_weights(tmp_path_factory, tmp_path, which):
+    """With the packed copy alone, steps with many rows go through the streaming products 64 rows at a time."""
+    config = CONFIGS[which]
+    folder, plain_model = model_for(tmp_path_factory, which, SHARP)
+    requests = requests_for(config, [150, 64, 37, 70, 90], seed=30)
+    steps = whole(requests)
+    engine = run_trace(folder, "bfloat16", steps, tmp_path / "whole", max_tokens=512, weight_copies="packed")
+    assert engine.weight_copies == "packed"
+    block = engine.model.blocks[0]
+    assert block.ffn.down_weight.tensor is None and block.ffn.down_weight.packed is not None
+    assert block.mixer.qkv_weight.tensor is None and engine.model.head.weight.packed is not None
+    compare(collect(steps, tmp_path / "whole", config.vocab_size), requests, plain_model, "bfloat16")
+    steps, peak = mixed(requests, seed=9)
+    run_trace(folder, "bfloat16", steps, tmp_path / "mixed", max_tokens=peak, weight_copies="packed")
+    compare(collect(steps, tmp_path / "mixed", config.vocab_size), requests, plain_model, "bfloat16")
+    both = run_trace(folder, "bfloat16", whole({"r0": requests["r0"]}), tmp_path / "both", max_tokens=256)
+    assert both.weight_copies == "both" and both.model.blocks[0].ffn.down_weight.tensor is not None
 
 
 def test_logits_only_where_wanted_and_requests_left_out(tmp_path_factory, tmp_path):
