@@ -1,4 +1,4 @@
-"""Decode and prefill throughput of the engine at Qwen2-7B size with random weights on one MI355X.
+"""Decode and prefill throughput of the engine at Qwen2-7B size (or, with --size, 72B or 0.5B) with random weights on one MI355X.
 
     python bench.py --gpus 1 --steps K --warmup W
 
@@ -16,6 +16,14 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+SIZES = {
+    "7b": dict(vocab_size=152064, hidden_size=3584, num_hidden_layers=28, num_attention_heads=28, num_key_value_heads=4,
+               head_dim=128, intermediate_size=18944, tie_word_embeddings=False),
+    "72b": dict(vocab_size=152064, hidden_size=8192, num_hidden_layers=80, num_attention_heads=64, num_key_value_heads=8,
+                head_dim=128, intermediate_size=29568, tie_word_embeddings=False),
+    "0.5b": dict(vocab_size=151936, hidden_size=896, num_hidden_layers=24, num_attention_heads=14, num_key_value_heads=2,
+                 head_dim=64, intermediate_size=4864, tie_word_embeddings=True),
+}
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 BF16_PEAK_FLOPS = 2.5e15       # MI355X dense bf16 MFMA, published
 FP32_PEAK_FLOPS = 157.3e12
@@ -28,7 +36,8 @@ def main() -> int:
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--context", type=int, default=4096)
-    parser.add_argument("--layers", type=int, default=28, help="fewer than 28 only where memory or time needs it")
+    parser.add_argument("--size", default="7b", choices=sorted(SIZES), help="layer sizes: Qwen2-7B's (the default), 72B's or 0.5B's")
+    parser.add_argument("--layers", type=int, default=None, help="fewer than the model has only where memory or time needs it")
     parser.add_argument("--prefill-tokens", type=int, default=2048)
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--points", default="1,64", help="other decode batch sizes to report")
@@ -42,10 +51,11 @@ def main() -> int:
     from microllm_rocm_amd import Engine, Qwen2Config
     from microllm_rocm_amd.engine.benchmark import decode_throughput, prefill_throughput, step_bytes, step_flops
 
-    full_layers = 28
-    config = Qwen2Config(vocab_size=152064, hidden_size=3584, num_hidden_layers=args.layers, num_attention_heads=28,
-                         num_key_value_heads=4, head_dim=128, intermediate_size=18944, max_position_embeddings=32768,
-                         rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False)
+    sizes = dict(SIZES[args.size])
+    full_layers = sizes.pop("num_hidden_layers")
+    if args.layers is None:
+        args.layers = full_layers
+    config = Qwen2Config(num_hidden_layers=args.layers, max_position_embeddings=32768, rope_theta=1e6, rms_norm_eps=1e-6, **sizes)
     page_size = 16
     points = sorted({int(b) for b in args.points.split(",") if b} | {args.batch})
     largest = max(points)
@@ -63,7 +73,7 @@ def main() -> int:
     achieved = bytes_step / (main_result["ms_per_step"] * 1e-3) / 1e9
 
     line = {
-        "metric": f"decode tok/s (ctx {args.context}) Qwen2-7B {'bf16' if args.dtype == 'bfloat16' else 'fp32'}",
+        "metric": f"decode tok/s (ctx {args.context}) Qwen2-{args.size.upper()} {'bf16' if args.dtype == 'bfloat16' else 'fp32'}",
         "value": round(main_result["tokens_per_second"], 2),
         "unit": "tok/s",
         "n_gpus": 1,
@@ -76,11 +86,11 @@ def main() -> int:
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: random N(0,0.02) weights, uniform-random token ids, caches filled with random keys and values",
         "config": {
-            "model": "Qwen2-7B size", "layers": args.layers, "layers_of_full_model": full_layers,
+            "model": f"Qwen2-{args.size.upper()} size", "layers": args.layers, "layers_of_full_model": full_layers,
             "hidden_size": config.hidden_size, "heads": config.num_attention_heads,
             "kv_heads": config.num_key_value_heads, "head_dim": config.head_dim,
             "intermediate_size": config.intermediate_size, "vocab_size": config.vocab_size,
-            "tie_word_embeddings": False, "global_batch": args.batch, "seq_len": args.context,
+            "tie_word_embeddings": config.tie_word_embeddings, "weight_copies": engine.weight_copies, "global_batch": args.batch, "seq_len": args.context,
             "kv_block_size": page_size, "prefill_tokens": args.prefill_tokens, "parallelism": "single GPU",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

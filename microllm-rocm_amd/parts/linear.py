@@ -128,7 +128,7 @@ def linear(x: Union[torch.Tensor, UnscaledRows], weight, out_dtype: Optional[tor
             return kernels.gemm_skinny(x, weight.packed, weight.out_features, "gated", scale=scale)
         return kernels.gemm_skinny(x, weight.packed, weight.out_features, "bf16" if out_dtype == torch.bfloat16 else "f32",
                                    scale=scale)
-    if w is None:
+    if w is None and rows > MEDIUM_ROWS:
         # Only the packed copy is kept: many rows go through this package's tiled product, or, where the
         # reduction is no multiple of 32, through the product for 64 rows, a piece at a time.
         epilogue = "gated" if gated else ("f32" if out_dtype == torch.float32 else "bf16")
@@ -137,8 +137,10 @@ def linear(x: Union[torch.Tensor, UnscaledRows], weight, out_dtype: Optional[tor
         plan = kernels.medium_plan(weight.out_features, weight.in_features, may_split=False)
         pieces = [kernels.gemm_medium(x[first:first + MEDIUM_ROWS], weight.packed, weight.out_features, epilogue, plan=plan)
                   for first in range(0, rows, MEDIUM_ROWS)]
-        return pieces[0] if len(pieces) == 1 else torch.cat(pieces)
-    if takes_packed(weight, rows, gated):
+        return torch.cat(pieces)
+    if w is None or takes_packed(weight, rows, gated):
+        if gated:
+            return kernels.gemm_medium(x, weight.packed, weight.out_features, "gated")
         if out_dtype == torch.float32:
             plan = kernels.medium_plan(weight.out_features, weight.in_features, may_split=partials)
             return kernels.gemm_medium(x, weight.packed, weight.out_features, "f32", plan=plan)
