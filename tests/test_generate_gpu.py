@@ -5,6 +5,7 @@ import subprocess
 import sys
 
 import numpy as np
+import torch
 import pytest
 
 import plain_qwen2 as plain
@@ -67,6 +68,53 @@ def test_sampling_in_batches_equals_requests_run_alone_and_follows_the_plain_rul
                 target = plain.uniform_for(p.seed, draw)
                 assert min(abs(cumulative - target)) < 1e-4
                 break
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_every_replay_of_a_decode_graph_equals_the_eager_step(tmp_path, dtype):
+    """Decode steps replayed from HIP graphs, with eager steps (a portion of a prompt beside decoded tokens, requests
+    that come and go, a wider block table) and synchronisations between the replays: every replay gives the bits
+    of the same step run without graphs."""
+    from microllm_rocm_amd.engine import StepEntry
+    folder = make_folder(tmp_path, "B", SHARP)
+    config = CONFIGS["B"]
+    graphs = engine_for(folder, dtype, use_graphs=True)
+    eager = engine_for(folder, dtype, use_graphs=False)
+    rng = np.random.default_rng(7)
+    prompts = {name: random_tokens(60 + index, length, config.vocab_size) for index, (name, length) in
+               enumerate({"a": 20, "b": 33, "c": 50}.items())}
+
+    def both(entries):
+        out = [engine.step([StepEntry(*entry) for entry in entries]) for engine in (graphs, eager)]
+        torch.cuda.synchronize()
+        assert (out[0] is None) == (out[1] is None)
+        if out[0] is not None:
+            assert torch.equal(out[0], out[1]), "a replayed step differs from the eager step"
+        return out[0]
+
+    for engine in (graphs, eager):
+        engine.open("a"), engine.open("b")
+    both([("a", prompts["a"], [19]), ("b", prompts["b"], [32])])
+    replays = 0
+    for step in range(40):
+        tokens = rng.integers(0, config.vocab_size, size=3).tolist()
+        if step == 10:      # an eager step between replays: a new request's prompt beside two decoded tokens
+            for engine in (graphs, eager):
+                engine.open("c")
+            both([("a", [tokens[0]], [0]), ("c", prompts["c"][:30], []), ("b", [tokens[1]], [0])])
+            both([("c", prompts["c"][30:], [19])])
+            continue
+        if step == 25:      # a request leaves: the graph for two requests again
+            for engine in (graphs, eager):
+                engine.close("b")
+        live = [name for name in ("a", "b", "c") if graphs.is_open(name)]
+        wanted = [[0], [], [0]] if step % 7 == 3 else [[0]] * 3        # logits of some requests only
+        both([(name, [token], want) for name, token, want in zip(live, tokens, wanted)])
+        replays += 1
+    assert graphs.graph_replays == replays and eager.graph_replays == 0
+    assert len(graphs._graphs) >= 2, "more than one graph was captured (two and three requests)"
+    for engine in (graphs, eager):
+        engine.cache.check()
 
 
 def test_few_pages_preempt_and_recompute_to_the_same_tokens(tmp_path):
