@@ -42,6 +42,7 @@ def main() -> int:
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--points", default="1,64", help="other decode batch sizes to report")
     parser.add_argument("--no-prefill", action="store_true")
+    parser.add_argument("--no-calibration", action="store_true", help="skip measuring what a read-only and an MFMA-only kernel reach")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
@@ -103,6 +104,15 @@ def main() -> int:
         line["prefill"] = {"value": round(prefill["tokens_per_second"], 1), "tokens": args.prefill_tokens,
                            "ms": round(prefill["ms"], 3),
                            "frac": round(flops / (prefill["ms"] * 1e-3) / peak_flops, 4)}
+    if not args.no_calibration and args.dtype == "bfloat16":
+        # What kernels that do nothing but read memory, or nothing but bfloat16 MFMAs, reach on this GPU: the
+        # fractions of these stand beside the fractions of the published peaks.
+        from microllm_rocm_amd.ops.kernels import measured_peaks
+        measured = measured_peaks()
+        line["measured_peaks"] = measured
+        line["roofline"]["frac_of_measured"] = round(achieved / measured["hbm_read_GBps"], 4)
+        if "prefill" in line:
+            line["prefill"]["frac_of_measured"] = round(flops / (prefill["ms"] * 1e-3) / (measured["mfma_bf16_TFLOPs"] * 1e12), 4)
     print(json.dumps(line), flush=True)
     return 0
 

@@ -147,6 +147,12 @@ int mll_gemm_medium(const void* a, const void* w_packed, void* out, int epilogue
 int mll_gemm_tiled(const void* a, const void* w_packed, void* out, int epilogue, int m, int n, int k,
                    hipStream_t stream);
 
+// Calibration: a kernel that reads `bytes` of memory once with `blocks` workgroups, and one in which every wave of
+// `blocks` workgroups of 4 issues iterations * 16 independent v_mfma_f32_16x16x32_bf16 (16384 flops each). The caller
+// times them. `sink` is 4 bytes of device memory that are never written with ordinary data.
+int mll_measure_read(const void* data, int64_t bytes, void* sink, int blocks, hipStream_t stream);
+int mll_measure_mfma(int iterations, void* sink, int blocks, hipStream_t stream);
+
 // Index of the first maximum of each row; a row that holds a non-finite value gives -1.
 // `parts` is device scratch of n_rows * mll_argmax_slices(vocab) * 16 bytes (contents need not be cleared).
 int mll_argmax(const float* logits, int32_t* out, void* parts, int n_rows, int vocab, hipStream_t stream);

@@ -663,3 +663,33 @@ def gemm_tiled(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f
         raise KernelLibraryError(f"unknown epilogue {epilogue!r}")
     _check(lib.mll_gemm_tiled(_ptr(x), _ptr(packed), _ptr(out), code, m, n, k, _stream()), lib)
     return out
+
+
+def measured_peaks(device: Optional[torch.device] = None, read_bytes: int = 4 << 30) -> dict:
+    """What this GPU reaches on a kernel that only reads memory once and on one that only issues bfloat16 MFMAs:
+    ``{"hbm_read_GBps": ..., "mfma_bf16_TFLOPs": ...}`` (the best of a few launches each; well under a second)."""
+    lib = library.load()
+    device = device or torch.device("cuda", torch.cuda.current_device())
+    sink = torch.zeros(1, dtype=torch.int32, device=device)
+    data = torch.empty(read_bytes // 4, dtype=torch.int32, device=device).random_()
+    units = torch.cuda.get_device_properties(device).multi_processor_count
+
+    def best(launch, repeats: int = 5) -> float:
+        launch()
+        torch.cuda.synchronize(device)
+        times = []
+        for _ in range(repeats):
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            launch()
+            stop.record()
+            stop.synchronize()
+            times.append(start.elapsed_time(stop) * 1e-3)
+        return min(times)
+
+    read_time = best(lambda: _check(lib.mll_measure_read(_ptr(data), ctypes.c_int64(data.numel() * 4), _ptr(sink), units * 8, _stream()), lib))
+    iterations, blocks = 4096, units * 4       # four waves a SIMD: one wave alone issues at two thirds of this rate
+    mfma_time = best(lambda: _check(lib.mll_measure_mfma(iterations, _ptr(sink), blocks, _stream()), lib))
+    flops = blocks * 4 * iterations * 16 * 16384.0
+    del data
+    return {"hbm_read_GBps": round(read_bytes / read_time / 1e9, 1), "mfma_bf16_TFLOPs": round(flops / mfma_time / 1e12, 1)}

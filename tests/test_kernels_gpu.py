@@ -687,3 +687,9 @@ def test_attention_kernels_at_twenty_thousand_keys(window):
         np.testing.assert_allclose(decode.float().cpu().numpy(), reference, **tolerance(torch.bfloat16))
     rowwise = k.paged_attention_rowwise(t["q"], t["k"], t["v"], t["table"], t["seq"], t["pos"], scale, window, heads, kv_heads, hd)
     np.testing.assert_allclose(rowwise.float().cpu().numpy(), reference, **tolerance(torch.bfloat16))
+
+
+def test_measured_peaks_are_plausible():
+    peaks = kernels().measured_peaks(read_bytes=1 << 30)
+    assert 2000.0 < peaks["hbm_read_GBps"] <= 8000.0, "a read-only kernel reaches between a quarter of and the published HBM peak"
+    assert 500.0 < peaks["mfma_bf16_TFLOPs"] <= 2500.0, "an MFMA-only kernel reaches at most the published dense bfloat16 peak"
