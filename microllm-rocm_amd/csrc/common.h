@@ -32,6 +32,11 @@ __host__ __device__ inline float to_float(bf16 value) {
 __device__ inline float rotate_first(float x1, float x2, float c, float s) { return fmaf(x1, c, -(x2 * s)); }
 __device__ inline float rotate_second(float x1, float x2, float c, float s) { return fmaf(x1, s, x2 * c); }
 
+// Waits until every load this wave has issued has arrived. The compiler waits by itself for loads into registers;
+// loads from memory straight into LDS return nothing to wait for, so whoever reads that LDS calls this first (and
+// then a barrier, if another wave's loads are read).
+__device__ inline void wait_for_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 // op over the four lanes {l, l ^ 16, l ^ 32, l ^ 48} of a wave, every one of which gets the result: two
 // exchanges on the vector unit (v_permlane16_swap, v_permlane32_swap of gfx950) instead of four trips through
 // LDS. op must be commutative. (The elements of the builtins' result are copied to scalars before they are

@@ -59,10 +59,11 @@ int mll_paged_attention_rowwise(const void* q, int dtype, const void* k_cache, c
                                 float scale, int window, int n_tokens, int heads, int kv_heads,
                                 int head_dim, int page_size, hipStream_t stream);
 
-// The same attention for bfloat16 portions of prompts with MFMA: one workgroup per (tile of up to
+// The same attention for bfloat16 portions of prompts with MFMA: one workgroup per (two tiles of up to
 // mll_paged_attention_prefill_tile() consecutive tokens of one request, query head). `tiles` holds, for each
-// tile, (request index, first token in the flat list, number of tokens); a tile never spans two requests and
-// its tokens have consecutive positions.
+// workgroup, (request index; first token in the flat list and number of tokens of the first tile; the same of the
+// second, whose number may be 0); a tile never spans two requests and its tokens have consecutive positions.
+// Workgroups take as long as the keys of both tiles together: pair a tile late in a prompt with an early one.
 int mll_paged_attention_prefill(const void* q, const void* k_cache, const void* v_cache,
                                 const int32_t* block_table, int table_width, const int32_t* tiles,
                                 int n_tiles, const int32_t* positions, void* out, float scale, int window,

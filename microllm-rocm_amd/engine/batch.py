@@ -14,9 +14,9 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, RELEASED, RequestCache
+from ..ops import kernels
 
-
-QUERY_TILE = 128   # tokens of one request that one workgroup of the prefill attention kernel takes
+QUERY_TILE = kernels.QUERY_TILE   # tokens of one request in one tile of the prefill attention kernel
 
 
 @dataclass
@@ -48,8 +48,11 @@ class StepContext:
     seq_total: torch.Tensor     # int32 [requests]: positions in the cache once this step is done
     slots: torch.Tensor         # int32 [requests]: state slot of every request
     want_rows: Optional[torch.Tensor]  # int32 [wanted]: rows of the flat list whose logits are wanted
-    query_tiles: torch.Tensor   # int32 [tiles, 3]: (request, first token in the flat list, tokens) per tile of <= 128
-                                # tokens, for the requests that bring more than one token (all, if none brings just one)
+    query_tiles: torch.Tensor   # int32 [workgroups, 5]: (request; first token in the flat list and tokens of a tile of
+                                # <= 128 tokens; the same of a second tile, perhaps empty), for the requests that bring
+                                # more than one token (all, if none brings just one); a late tile goes with an early one
+    query_tiles_adjacent: Optional[torch.Tensor]  # the same with neighbouring tiles together, for layers with a window
+                                                  # (None where no layer has one)
     single_tokens: Optional[torch.Tensor]  # int32: rows of the requests that bring one token, when others bring more
     paged: List[PagedView]
     # the same on the host, for parts written in Python and for choosing kernels
@@ -136,23 +139,26 @@ class BatchBuilder:
             tables.append(table)
             mappings.append(mapping.astype(np.int32, copy=False))
             widths.append(width)
+        windowed = any(getattr(group.need, "window", None) is not None for group in self.cache.groups)
         if n_tokens == n_seqs:
             index = np.arange(n_seqs, dtype=np.int32)
-            query_tiles = np.stack([index, index, np.ones(n_seqs, dtype=np.int32)], axis=1)
+            zero = np.zeros(n_seqs, dtype=np.int32)
+            query_tiles = np.stack([index, index, np.ones(n_seqs, dtype=np.int32), zero, zero], axis=1)
+            adjacent_tiles = query_tiles if windowed else np.zeros((0, 5), dtype=np.int32)
             single_tokens = np.zeros(0, dtype=np.int32)
             max_single_total = 0
         else:
-            # Tiles with the most keys to walk come first, so that the longest workgroups start first.
             mixed = any(count == 1 for count in counts)
-            tile_list = sorted(((index, cu[index] + offset, min(QUERY_TILE, count - offset))
-                                for index, count in enumerate(counts) if not (mixed and count == 1)
-                                for offset in range(0, count, QUERY_TILE)),
-                               key=lambda tile: -(starts[tile[0]] + tile[1] - cu[tile[0]] + tile[2]))
-            query_tiles = np.asarray(tile_list, dtype=np.int32).reshape(-1, 3)
+            tile_list = [(index, int(cu[index]) + offset, min(QUERY_TILE, count - offset), starts[index] + offset)
+                         for index, count in enumerate(counts) if not (mixed and count == 1)
+                         for offset in range(0, count, QUERY_TILE)]
+            query_tiles = np.asarray(kernels.pair_query_tiles(tile_list), dtype=np.int32).reshape(-1, 5)
+            adjacent_tiles = np.asarray(kernels.pair_query_tiles(tile_list, adjacent=True) if windowed else [],
+                                        dtype=np.int32).reshape(-1, 5)
             single_tokens = np.asarray([cu[index] for index, count in enumerate(counts) if mixed and count == 1], dtype=np.int32)
             max_single_total = max((totals[index] for index, count in enumerate(counts) if mixed and count == 1), default=0)
         pieces = [tokens, positions, seq_of_token, cu, starts_array, totals_array, slots, want_rows,
-                  query_tiles.reshape(-1), single_tokens]
+                  query_tiles.reshape(-1), single_tokens, adjacent_tiles.reshape(-1)]
         for table, mapping in zip(tables, mappings):
             pieces += [table.reshape(-1), mapping]
         offsets, cursor = [], 0
@@ -173,13 +179,14 @@ class BatchBuilder:
 
         paged = []
         for g, group in enumerate(self.cache.groups):
-            paged.append(PagedView(piece_at(10 + 2 * g, (n_seqs, widths[g])), piece_at(11 + 2 * g),
+            paged.append(PagedView(piece_at(11 + 2 * g, (n_seqs, widths[g])), piece_at(12 + 2 * g),
                                    page_size, widths[g]))
         longest = max(totals) if totals else 0
         return StepContext(
             n_tokens=n_tokens, n_seqs=n_seqs, tokens=piece_at(0), positions=piece_at(1), seq_of_token=piece_at(2),
             cu_tokens=piece_at(3), seq_start=piece_at(4), seq_total=piece_at(5), slots=piece_at(6),
-            want_rows=piece_at(7) if want_rows.size else None, query_tiles=piece_at(8, (-1, 3)),
+            want_rows=piece_at(7) if want_rows.size else None, query_tiles=piece_at(8, (-1, 5)),
+            query_tiles_adjacent=piece_at(10, (-1, 5)) if windowed else None,
             single_tokens=piece_at(9) if single_tokens.size else None, max_single_total=max_single_total, paged=paged,
             starts=starts, counts=counts, host_slots=slots.tolist(),
             max_count=max(counts) if counts else 0, max_total=longest,

@@ -7,7 +7,7 @@ a kernel never sees operands that do not fit what its grid assumes.
 from __future__ import annotations
 
 import ctypes
-from typing import NamedTuple, Optional, Tuple
+from typing import List, NamedTuple, Optional, Sequence, Tuple
 
 import torch
 
@@ -432,6 +432,47 @@ def gemm_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = to
     return torch.mm(x, weight.t(), out_dtype=out_dtype)
 
 
+LIBRARY_TILE = 256          # the library's products of many rows work in tiles of about 256 x 256
+LIBRARY_WORKGROUPS = 224    # splitting the reduction pays while tiles x parts stay at or under this (of 256 compute units)
+LIBRARY_SPLIT_LENGTH = 2048  # and every part of the reduction keeps at least this many terms
+
+
+def library_splits(m: int, n: int, k: int) -> int:
+    """Into how many ranges of the reduction ``gemm_bf16_split`` cuts a float32 product of ``m`` rows.
+
+    The library takes one workgroup per tile of the result: a long reduction into a narrow result (a
+    feed-forward's down projection) leaves most compute units idle. Measured on MI355X (m = 2048, n = 3584,
+    k = 18944): 348 us whole, 205 us in two parts. Parts are powers of two up to 8; where the result's tiles do not
+    fill their last round over the compute units to 90 % and the reduction has 16384 terms or more, four parts
+    still gain (m = 4096 and 8192 at the sizes above)."""
+    tiles = -(-m // LIBRARY_TILE) * -(-n // LIBRARY_TILE)
+    best = 1
+    for parts in (2, 4, 8):
+        if k % (32 * parts) == 0 and k // parts >= LIBRARY_SPLIT_LENGTH and tiles * parts <= LIBRARY_WORKGROUPS:
+            best = parts
+    if best == 1 and k >= 16384 and k % 128 == 0:
+        rounds = -(-tiles // 256)
+        if tiles > LIBRARY_WORKGROUPS // 2 and tiles < 0.9 * 256 * rounds:
+            best = 4
+    return best
+
+
+def gemm_bf16_split(x: torch.Tensor, weight: torch.Tensor, parts: int) -> torch.Tensor:
+    """``x @ weight.T`` as ``[parts, m, n]`` float32 sums over ``parts`` equal ranges of the reduction, for the
+    caller to add in order: one batched library product over strided views of both operands (no copies)."""
+    _device_tensor(x, "gemm input", torch.bfloat16)
+    _device_tensor(weight, "gemm weight", torch.bfloat16)
+    _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "gemm takes [m, k] and [n, k]")
+    m, k = x.shape
+    _need(parts >= 1 and k % parts == 0, f"{parts} parts do not divide a reduction of {k}")
+    if parts == 1:
+        return torch.mm(x, weight.t(), out_dtype=torch.float32).unsqueeze(0)
+    length = k // parts
+    a = x.view(m, parts, length).transpose(0, 1)                          # [parts, m, length]
+    b = weight.view(weight.shape[0], parts, length).permute(1, 2, 0)      # [parts, length, n]
+    return torch.bmm(a, b, out_dtype=torch.float32)
+
+
 def decode_splits(n_tokens: int, kv_heads: int, longest: int) -> int:
     """How many splits of the keys: about one workgroup per compute unit, at least 256 keys each (measured on
     MI355X: more splits cost more in joining them than they gain)."""
@@ -476,16 +517,47 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     return out
 
 
+QUERY_TILE = 128   # tokens of one request in one tile of the prefill attention kernel; a workgroup takes two tiles
+
+
+def pair_query_tiles(tiles: Sequence[Tuple[int, int, int, int]], adjacent: bool = False) -> List[Tuple[int, int, int, int, int]]:
+    """The prefill attention's workgroups from its tiles. ``tiles``: (request, first token in the flat list,
+    tokens, position of the first token). Returns (request, first token, tokens, first token, tokens) rows, the
+    workgroups with the most keys to walk first, so that the longest start first.
+
+    A tile's work grows with its position (it sees every earlier key), so of one request's tiles the last goes
+    with the first, the last but one with the second and so on: every workgroup of a request then walks about as
+    many keys. With ``adjacent`` neighbours go together instead: under a window every tile sees about as many keys,
+    and neighbours see nearly the same ones. A request's odd tile goes alone."""
+    by_request: dict = {}
+    for tile in tiles:
+        by_request.setdefault(tile[0], []).append(tile)
+    pairs = []
+    for request, own in by_request.items():
+        own.sort(key=lambda tile: tile[3])
+        count = len(own)
+        if adjacent:
+            couples = [(own[i], own[i + 1] if i + 1 < count else None) for i in range(0, count, 2)]
+        else:
+            couples = [(own[count - 1 - i], own[i] if i != count - 1 - i else None) for i in range((count + 1) // 2)]
+        for first, second in couples:
+            weight = first[3] + first[2] + (second[3] + second[2] if second else 0)
+            pairs.append((weight, (request, first[1], first[2], second[1] if second else 0, second[2] if second else 0)))
+    pairs.sort(key=lambda pair: -pair[0])
+    return [pair[1] for pair in pairs]
+
+
 def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                             query_tiles: torch.Tensor, positions: torch.Tensor, scale: float, window: int,
                             heads: int, kv_heads: int, head_dim: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The MFMA kernel for bfloat16 portions of prompts; ``query_tiles`` rows are (request, first token, tokens)."""
+    """The MFMA kernel for bfloat16 portions of prompts; ``query_tiles`` rows are (request, first token, tokens,
+    first token, tokens): two tiles of up to ``QUERY_TILE`` tokens of the request (``pair_query_tiles``)."""
     lib = library.load()
     page_size = _check_paged(q, k_cache, v_cache, block_table, heads, kv_heads, head_dim)
     _need(q.dtype == torch.bfloat16, "the prefill kernel takes bfloat16")
     _need(head_dim % 16 == 0 and 16 <= head_dim <= 256, "the prefill kernel takes head sizes in steps of 16 up to 256")
     _device_tensor(query_tiles, "query tiles", torch.int32)
-    _need(query_tiles.dim() == 2 and query_tiles.shape[1] == 3, "query tiles must be [tiles, 3]")
+    _need(query_tiles.dim() == 2 and query_tiles.shape[1] == 5, "query tiles must be [workgroups, 5]")
     _device_tensor(positions, "positions", torch.int32)
     _need(positions.shape[0] == q.shape[0], "positions must hold one entry per token")
     if out is None:
@@ -517,7 +589,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         # Portions go to the tiled kernel; requests that bring one token, if any, to the split kernel.
         out = torch.empty_like(q)
         if ctx.query_tiles.shape[0] > 0:
-            paged_attention_prefill(q, k_cache, v_cache, view.block_table, ctx.query_tiles, ctx.positions,
+            tiles = ctx.query_tiles_adjacent if window > 0 and ctx.query_tiles_adjacent is not None else ctx.query_tiles
+            paged_attention_prefill(q, k_cache, v_cache, view.block_table, tiles, ctx.positions,
                                     scale, window, heads, kv_heads, head_dim, out=out)
         if ctx.single_tokens is not None:
             visible = min(ctx.max_single_total, window) if window > 0 else ctx.max_single_total

@@ -119,7 +119,8 @@ def build(verbose: bool = True) -> str:
         objects = list(pool.map(compile_one, sources))
     library = os.path.join(target_dir, LIBRARY_NAME)
     temporary = library + f".{os.getpid()}.tmp"
-    command = [hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", temporary, *objects]
+    # -z defs: a kernel whose host side the compiler dropped shows up here, not when the library is loaded
+    command = [hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-Wl,-z,defs", "-o", temporary, *objects]
     result = subprocess.run(command, env=env, capture_output=True, text=True)
     if result.returncode != 0:
         raise KernelLibraryError(f"linking {library} failed:\n{result.stdout}\n{result.stderr}")

@@ -147,4 +147,8 @@ def linear(x: Union[torch.Tensor, UnscaledRows], weight, out_dtype: Optional[tor
         return kernels.gemm_medium(x, weight.packed, weight.out_features, "bf16")
     if gated:
         return kernels.silu_mul(kernels.gemm_bf16(x, w, torch.bfloat16))
+    if partials and out_dtype == torch.float32:
+        parts = kernels.library_splits(rows, weight.out_features, weight.in_features)
+        if parts > 1:
+            return kernels.gemm_bf16_split(x, w, parts)
     return kernels.gemm_bf16(x, w, out_dtype)

@@ -24,6 +24,38 @@ def test_medium_plan_depends_on_the_weight_alone_and_is_launchable(n, k):
         assert groups * (splits // 2) < kernels.MEDIUM_WORKGROUPS, "no more splits than the GPU needs"
 
 
+@pytest.mark.parametrize("m,n,k,parts", [
+    (2048, 3584, 18944, 2), (1024, 3584, 18944, 4), (512, 3584, 18944, 8), (65, 3584, 18944, 8),     # a long reduction into a narrow result
+    (4096, 3584, 18944, 4), (8192, 3584, 18944, 4),                                                   # a last round of tiles that is not full
+    (2048, 3584, 3584, 1), (2048, 4608, 3584, 1), (512, 3584, 3584, 1),                               # short reductions stay whole
+    (2048, 8192, 29568, 1), (4096, 8192, 29568, 1), (512, 8192, 29568, 2), (256, 8192, 8192, 4),      # wide results fill the GPU by themselves
+    (2048, 896, 4864, 2), (8192, 896, 4864, 1), (100, 331, 120, 1), (300, 64, 4160, 2), (300, 64, 4128, 1)])
+def test_library_splits(m, n, k, parts):
+    assert kernels.library_splits(m, n, k) == parts
+    assert k % parts == 0 and (parts == 1 or k // parts >= kernels.LIBRARY_SPLIT_LENGTH)
+
+
+def test_query_tiles_go_in_twos_that_walk_about_as_many_keys():
+    # one prompt of 2048 tokens from position 0 (16 tiles), a portion of 300 from position 1000, one tile alone
+    tiles = [(0, offset, 128, offset) for offset in range(0, 2048, 128)]
+    tiles += [(1, 2048 + offset, min(128, 300 - offset), 1000 + offset) for offset in range(0, 300, 128)] + [(2, 2348, 17, 40)]
+    pairs = kernels.pair_query_tiles(list(tiles))
+    covered = sorted((r, first, count) for r, a, ca, b, cb in pairs for first, count in ((a, ca), (b, cb)) if count)
+    assert covered == sorted(tile[:3] for tile in tiles), "every tile once"
+    of_first = [pair for pair in pairs if pair[0] == 0]
+    position = {tile[1]: tile[3] for tile in tiles}
+    weights = [position[a] + ca + position[b] + cb for _, a, ca, b, cb in of_first]
+    assert len(of_first) == 8 and max(weights) == min(weights) == 2048 + 128, "late with early: all the same"
+    assert [pair for pair in pairs if pair[0] == 2] == [(2, 2348, 17, 0, 0)]
+    assert sorted(pair[1:] for pair in pairs if pair[0] == 1) == [(2048 + 128, 128, 0, 0), (2048 + 256, 44, 2048, 128)]
+    keys = [position[a] + ca + (position[b] + cb if cb else 0) for _, a, ca, b, cb in pairs]
+    assert keys == sorted(keys, reverse=True), "the longest first"
+    # under a window neighbours go together
+    adjacent = kernels.pair_query_tiles(list(tiles), adjacent=True)
+    assert sorted(pair[1:] for pair in adjacent if pair[0] == 0) == [(offset, 128, offset + 128, 128) for offset in range(0, 2048, 256)]
+    assert sorted(pair[1:] for pair in adjacent if pair[0] == 1) == [(2048, 128, 2048 + 128, 128), (2048 + 256, 44, 0, 0)]
+
+
 @pytest.mark.parametrize("heads,kv_heads,hd,n_freq", [(4, 2, 16, 8), (3, 1, 32, 8), (28, 4, 128, 64), (2, 0, 64, 32), (5, 5, 48, 0)])
 def test_rotary_pair_order_puts_partners_side_by_side(heads, kv_heads, hd, n_freq):
     order = kernels.rotary_pair_order(heads, kv_heads, hd, n_freq).tolist()

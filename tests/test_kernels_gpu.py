@@ -243,6 +243,15 @@ def reference_attention(q_exact, exact_k, exact_v, seq_of_token, positions, head
     return out.reshape(len(positions), heads * hd)
 
 
+def query_tile_list(lengths, counts):
+    """(request, first token in the flat list, tokens, position of the first token) of every tile of 128 tokens."""
+    tiles, start = [], 0
+    for index, (length, count) in enumerate(zip(lengths, counts)):
+        tiles += [(index, start + offset, min(128, count - offset), length - count + offset) for offset in range(0, count, 128)]
+        start += count
+    return tiles
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kv_heads,hd,page_size,window", [
     (4, 2, 16, 16, 0), (3, 1, 32, 16, 24), (5, 5, 48, 16, 100), (6, 3, 24, 48, 0), (2, 1, 128, 32, 70), (8, 1, 200, 16, 0)])
@@ -282,18 +291,24 @@ def test_decode_attention(heads, kv_heads, hd, page_size, window, splits):
     (2, 1, 80, 16, 300), (3, 3, 256, 16, 0), (7, 7, 112, 64, 129), (6, 3, 96, 48, 17)])
 def test_prefill_attention(heads, kv_heads, hd, page_size, window):
     rng = np.random.default_rng(heads + hd + window)
-    lengths, counts = [517, 1, 300, 97, 64, 131, 40], [130, 1, 300, 17, 64, 2, 33]
+    lengths, counts = [517, 1, 700, 97, 64, 131, 40], [130, 1, 700, 17, 64, 2, 33]
     t, q_exact, ek, ev, seq, pos = build_paged_case(rng, torch.bfloat16, lengths, counts, heads, kv_heads, hd, page_size)
     scale = 1.0 / math.sqrt(hd)
-    tiles, start = [], 0
-    for index, count in enumerate(counts):
-        tiles += [(index, start + offset, min(128, count - offset)) for offset in range(0, count, 128)]
-        start += count
-    query_tiles = torch.tensor(tiles, dtype=torch.int32, device=DEVICE)
-    out = kernels().paged_attention_prefill(t["q"], t["k"], t["v"], t["table"], query_tiles, t["pos"], scale, window,
-                                            heads, kv_heads, hd)
     reference = reference_attention(q_exact, ek, ev, seq, pos, heads, kv_heads, hd, scale, window)
-    np.testing.assert_allclose(out.float().cpu().numpy(), reference, **tolerance(torch.bfloat16))
+    tiles = query_tile_list(lengths, counts)
+    alone = [(tile[0], tile[1], tile[2], 0, 0) for tile in tiles]
+    backwards = [(tile[0], 0, 0, tile[1], tile[2]) for tile in tiles]
+    # every way of putting tiles together gives the same numbers: a late tile with an early one, neighbours, each
+    # tile alone as the first or as the second of its workgroup
+    results = []
+    for pairs in (kernels().pair_query_tiles(tiles), kernels().pair_query_tiles(tiles, adjacent=True), alone, backwards):
+        query_tiles = torch.tensor(pairs, dtype=torch.int32, device=DEVICE)
+        out = kernels().paged_attention_prefill(t["q"], t["k"], t["v"], t["table"], query_tiles, t["pos"], scale, window,
+                                                heads, kv_heads, hd)
+        np.testing.assert_allclose(out.float().cpu().numpy(), reference, **tolerance(torch.bfloat16))
+        results.append(out)
+    for out in results[1:]:
+        assert torch.equal(out, results[0]), "a token's result depends on which tile shares its workgroup"
 
 
 @pytest.mark.parametrize("kernel", ["rowwise_f32", "rowwise_bf16", "decode", "prefill"])
@@ -323,7 +338,7 @@ def test_a_far_key_among_hundreds_and_the_window_edge(kernel):
                                            heads, kv_heads, hd, 6)
         elif kernel == "prefill":
             out = k.paged_attention_prefill(t["q"], t["k"], t["v"], t["table"],
-                                            torch.tensor([[0, 0, 1]], dtype=torch.int32, device=DEVICE), t["pos"],
+                                            torch.tensor([[0, 0, 1, 0, 0]], dtype=torch.int32, device=DEVICE), t["pos"],
                                             scale, window, heads, kv_heads, hd)
         else:
             out = k.paged_attention_rowwise(t["q"], t["k"], t["v"], t["table"], t["seq"], t["pos"], scale, window,
@@ -586,6 +601,26 @@ def test_gemm_medium(m, n, k):
     assert torch.equal(alone[..., 0, :], parts[..., m - 1, :])
 
 
+@pytest.mark.parametrize("m,n,k,parts", [(300, 200, 4096, 2), (65, 331, 8192, 4), (700, 272, 16384, 8), (90, 64, 96, 3), (128, 256, 512, 1)])
+def test_library_product_in_parts_of_the_reduction(m, n, k, parts):
+    """The library's batched product over strided views: its parts add up to the whole product, each part is the
+    product over its own range of the reduction."""
+    rng = np.random.default_rng(m + k)
+    a_ref, a = to_bf16_exact(rng.normal(size=(m, k)))
+    w_ref, w = to_bf16_exact(rng.normal(size=(n, k)) * 0.1)
+    ka = kernels()
+    got = ka.gemm_bf16_split(a, w, parts)
+    assert got.dtype == torch.float32 and got.shape == (parts, m, n)
+    length = k // parts
+    for part in range(parts):
+        expected = a_ref[:, part * length:(part + 1) * length] @ w_ref[:, part * length:(part + 1) * length].T
+        assert np.abs(got[part].double().cpu().numpy() - expected).max() <= 1e-5 * np.abs(expected).max()
+    whole = a_ref @ w_ref.T
+    assert np.abs(got.double().sum(0).cpu().numpy() - whole).max() <= 1e-5 * np.abs(whole).max()
+    with pytest.raises(Exception, match="do not divide"):
+        ka.gemm_bf16_split(a, w, 7)
+
+
 @pytest.mark.parametrize("m,n,k", [(300, 1000, 256), (257, 272, 64), (65, 331, 96), (2048, 4608, 512), (700, 3584, 2048)])
 def test_gemm_tiled(m, n, k):
     """The tiled product for many rows over a packed weight (what an engine with one copy of its weights takes)."""
@@ -674,10 +709,7 @@ def test_attention_kernels_at_twenty_thousand_keys(window):
     scale = 1.0 / math.sqrt(hd)
     reference = reference_attention(q_exact, ek, ev, seq, pos, heads, kv_heads, hd, scale, window)
     k = kernels()
-    tiles, start = [], 0
-    for index, count in enumerate(counts):
-        tiles += [(index, start + offset, min(128, count - offset)) for offset in range(0, count, 128)]
-        start += count
+    tiles = k.pair_query_tiles(query_tile_list(lengths, counts), adjacent=window > 0)
     prefill = k.paged_attention_prefill(t["q"], t["k"], t["v"], t["table"], torch.tensor(tiles, dtype=torch.int32, device=DEVICE),
                                         t["pos"], scale, window, heads, kv_heads, hd)
     np.testing.assert_allclose(prefill.float().cpu().numpy(), reference, **tolerance(torch.bfloat16))
