@@ -144,9 +144,11 @@ int mll_gemm_medium(const void* a, const void* w_packed, void* out, int epilogue
 
 // The same product for many rows: 256 x 256 tiles of C per workgroup, pieces of A and W brought into LDS by
 // direct global-to-LDS loads. A is row-major [m, k] with k a multiple of 32; epilogues 0, 1 and 2 of
-// mll_gemm_skinny. For weights that are kept in the packed order alone.
+// mll_gemm_skinny. With epilogue 0, `splits` > 1 deals the stages of 64 of k to that many workgroups per tile:
+// out is then [splits, m, n] partial sums for the caller to add in order. For weights that are kept in the packed
+// order alone.
 int mll_gemm_tiled(const void* a, const void* w_packed, void* out, int epilogue, int m, int n, int k,
-                   hipStream_t stream);
+                   int splits, hipStream_t stream);
 
 // Calibration: a kernel that reads `bytes` of memory once with `blocks` workgroups, and one in which every wave of
 // `blocks` workgroups of 4 issues iterations * 16 independent v_mfma_f32_16x16x32_bf16 (16384 flops each). The caller

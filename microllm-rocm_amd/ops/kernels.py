@@ -715,9 +715,26 @@ def gemm_medium(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "
     return out
 
 
-def gemm_tiled(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f32") -> torch.Tensor:
-    """``x @ W.T`` for many bfloat16 rows and a packed weight, on this package's tiled MFMA kernel (about half
-    the library's rate: for weights that are kept in the packed order alone). ``k`` must be a multiple of 32."""
+TILED_TILE = 256            # gemm_tiled works in tiles of 256 x 256, stages of 64 of the reduction
+TILED_SPLIT_STAGES = 8      # a part of the reduction keeps at least this many stages
+
+
+def tiled_splits(m: int, n: int, k: int) -> int:
+    """Into how many parts ``gemm_tiled`` cuts the reduction of a float32 product: while the result's tiles leave
+    compute units idle (a workgroup a tile: 28 workgroups for 512 rows by 3584 columns), up to 8."""
+    tiles = -(-m // TILED_TILE) * -(-n // TILED_TILE)
+    stages = -(-k // 64)
+    splits = 1
+    while splits < 8 and tiles * splits * 2 <= LIBRARY_WORKGROUPS and stages // (splits * 2) >= TILED_SPLIT_STAGES:
+        splits *= 2
+    return splits
+
+
+def gemm_tiled(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f32", splits: int = 1) -> torch.Tensor:
+    """``x @ W.T`` for many bfloat16 rows and a packed weight, on this package's tiled MFMA kernel (0.85 to 0.95 of
+    the library's rate at 2048 rows and more: for weights that are kept in the packed order alone). ``k`` must be
+    a multiple of 32. With ``splits`` > 1 (float32 only) the result is ``[splits, m, n]`` sums over parts of the
+    reduction for the caller to add in order."""
     lib = library.load()
     _device_tensor(x, "gemm input", torch.bfloat16)
     _device_tensor(packed, "packed weight", torch.bfloat16)
@@ -725,8 +742,9 @@ def gemm_tiled(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f
     m, k = x.shape
     _need(k % 32 == 0, "gemm_tiled needs k to be a multiple of 32")
     _need(packed.shape[0] == -(-n // 16) and packed.shape[1] == k // 32, "the packed weight does not fit n and k")
+    _need(splits >= 1 and (splits == 1 or epilogue == "f32"), "only the float32 epilogue takes the reduction in parts")
     if epilogue == "f32":
-        code, out = 0, torch.empty((m, n), dtype=torch.float32, device=x.device)
+        code, out = 0, torch.empty((m, n) if splits == 1 else (splits, m, n), dtype=torch.float32, device=x.device)
     elif epilogue == "bf16":
         code, out = 1, torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
     elif epilogue == "gated":
@@ -734,7 +752,7 @@ def gemm_tiled(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f
         code, out = 2, torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
     else:
         raise KernelLibraryError(f"unknown epilogue {epilogue!r}")
-    _check(lib.mll_gemm_tiled(_ptr(x), _ptr(packed), _ptr(out), code, m, n, k, _stream()), lib)
+    _check(lib.mll_gemm_tiled(_ptr(x), _ptr(packed), _ptr(out), code, m, n, k, splits, _stream()), lib)
     return out
 
 

@@ -133,7 +133,8 @@ def linear(x: Union[torch.Tensor, UnscaledRows], weight, out_dtype: Optional[tor
         # reduction is no multiple of 32, through the product for 64 rows, a piece at a time.
         epilogue = "gated" if gated else ("f32" if out_dtype == torch.float32 else "bf16")
         if weight.in_features % 32 == 0:
-            return kernels.gemm_tiled(x, weight.packed, weight.out_features, epilogue)
+            splits = kernels.tiled_splits(rows, weight.out_features, weight.in_features) if partials and epilogue == "f32" else 1
+            return kernels.gemm_tiled(x, weight.packed, weight.out_features, epilogue, splits=splits)
         plan = kernels.medium_plan(weight.out_features, weight.in_features, may_split=False)
         pieces = [kernels.gemm_medium(x[first:first + MEDIUM_ROWS], weight.packed, weight.out_features, epilogue, plan=plan)
                   for first in range(0, rows, MEDIUM_ROWS)]

@@ -35,6 +35,13 @@ def test_library_splits(m, n, k, parts):
     assert k % parts == 0 and (parts == 1 or k // parts >= kernels.LIBRARY_SPLIT_LENGTH)
 
 
+@pytest.mark.parametrize("m,n,k,splits", [(512, 3584, 3584, 4), (512, 3584, 18944, 8), (2048, 3584, 18944, 2), (2048, 37888, 3584, 1),
+                                          (300, 64, 512, 1), (100, 8192, 8192, 4), (4096, 8192, 29568, 1)])
+def test_tiled_splits(m, n, k, splits):
+    assert kernels.tiled_splits(m, n, k) == splits
+    assert -(-k // 64) // splits >= (kernels.TILED_SPLIT_STAGES if splits > 1 else 0)
+
+
 def test_query_tiles_go_in_twos_that_walk_about_as_many_keys():
     # one prompt of 2048 tokens from position 0 (16 tiles), a portion of 300 from position 1000, one tile alone
     tiles = [(0, offset, 128, offset) for offset in range(0, 2048, 128)]

@@ -640,6 +640,17 @@ def test_gemm_tiled(m, n, k):
         gated = ka.gemm_tiled(a, ka.pack_weight(w, interleave_halves=True), n, "gated")
         wanted = plain.silu(expected[:, : n // 2]) * expected[:, n // 2:]
         np.testing.assert_allclose(gated.float().cpu().numpy(), wanted, rtol=1.2e-2, atol=1.2e-2 * np.abs(wanted).max())
+    # the reduction in parts: the parts add up to the product, a part is the product over its stages of 64
+    for splits in (2, 3, 8):
+        parts = ka.gemm_tiled(a, packed, n, "f32", splits=splits)
+        assert parts.shape == (splits, m, n)
+        assert np.abs(parts.double().sum(0).cpu().numpy() - expected).max() <= 1e-5 * scale
+        stages = -(-k // 64)
+        per_part = -(-stages // splits)
+        first = a_ref[:, :64 * per_part] @ w_ref[:, :64 * per_part].T
+        assert np.abs(parts[0].double().cpu().numpy() - first).max() <= 1e-5 * max(np.abs(first).max(), 1e-30)
+    with pytest.raises(Exception, match="parts"):
+        ka.gemm_tiled(a, packed, n, "bf16", splits=2)
     # the same in every run, and a row's result does not depend on the other rows of the call
     assert torch.equal(ka.gemm_tiled(a, packed, n, "f32"), full)
     assert torch.equal(ka.gemm_tiled(a[m - 70:].contiguous(), packed, n, "f32"), full[m - 70:]) if m > 70 else True
