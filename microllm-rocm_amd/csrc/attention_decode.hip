@@ -86,49 +86,33 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
     for (int d = 0; d < HD_TILES; ++d) o_acc[d] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     float running_max = -INFINITY, running_sum = 0.0f;
 
-    // The pages of a pair's two tiles are looked up one iteration ahead of their use.
-    auto page_of = [&](int tile_key) -> int {
-        return (tile_key <= position && tile_key + 15 >= low) ? table[tile_key / page_size] : -1;
-    };
-    int pair = pair_begin + wave;
-    int next_page[2] = {-1, -1};
-    if (pair < pair_end) {
-        next_page[0] = page_of(pair * 32);
-        next_page[1] = page_of(pair * 32 + 16);
-    }
-    for (; pair < pair_end; pair += kDecodeWaves) {
-        const int key0 = pair * 32;
-        const int page[2] = {next_page[0], next_page[1]};
-        if (pair + kDecodeWaves < pair_end) {
-            next_page[0] = page_of((pair + kDecodeWaves) * 32);
-            next_page[1] = page_of((pair + kDecodeWaves) * 32 + 16);
-        }
-        // Keys: A operand, row = key `col` of the tile, 8 dims (chunk 4 * ks + quad) per lane.
-        // Values: A operand of the second product, row = dim `col` of a dim tile, k-slots = keys 4*quad..+3 of
-        // tile 0, then of tile 1.
-        Frag8 k_frag[2][K_STEPS];
-        Frag8 v_frag[HD_TILES];
-#pragma unroll
-        for (int d = 0; d < HD_TILES; ++d) v_frag[d].raw = make_uint4(0, 0, 0, 0);
+    // A pair's keys and values, from the pages into registers. Keys: A operand, row = key `col` of the tile, 8
+    // dims (chunk 4 * ks + quad) per lane. Values: A operand of the second product, row = dim `col` of a dim
+    // tile, k-slots = keys 4*quad..+3 of tile 0, then of tile 1. Every load is issued, none behind a branch (a
+    // tile that no query sees is read from page 0 and masked like a stale one): only of straight-line code does
+    // the compiler know how many loads are still on their way, and waits for one pair alone while the next flies.
+    auto load_pair = [&](int pair_index, const int (&page)[2], Frag8 (&k_frag)[2][K_STEPS], Frag8 (&v_frag)[HD_TILES]) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const int offset = (key0 + 16 * t) % page_size;
+            const int offset = (pair_index * 32 + 16 * t) % page_size;
             const bf16* k_tile = k_cache + layout.k_tile(max(page[t], 0), kv_head, offset / 16) + col * 8;
             const bf16* v_tile = v_cache + layout.v_tile(max(page[t], 0), kv_head, offset / 16) + (quad * 16 + col) * 4;
 #pragma unroll
             for (int ks = 0; ks < K_STEPS; ++ks) {
                 const int piece = ks * 4 + quad;
-                k_frag[t][ks].raw = make_uint4(0, 0, 0, 0);
-                if (page[t] >= 0 && piece < K_CHUNKS)
+                if (HD % 32 == 0) {
                     k_frag[t][ks].raw = *reinterpret_cast<const uint4*>(k_tile + piece * 128);
+                } else {      // the last 32 dims are not all there: nothing may be read past the tile
+                    k_frag[t][ks].raw = make_uint4(0, 0, 0, 0);
+                    if (piece < K_CHUNKS) k_frag[t][ks].raw = *reinterpret_cast<const uint4*>(k_tile + piece * 128);
+                }
             }
-            if (page[t] >= 0) {
 #pragma unroll
-                for (int d = 0; d < HD_TILES; ++d)
-                    v_frag[d].h[t] = *reinterpret_cast<const bf16x4*>(v_tile + d * 256);
-            }
+            for (int d = 0; d < HD_TILES; ++d) v_frag[d].h[t] = *reinterpret_cast<const bf16x4*>(v_tile + d * 256);
         }
-
+    };
+    auto attend_pair = [&](int pair_index, const Frag8 (&k_frag)[2][K_STEPS], Frag8 (&v_frag)[HD_TILES]) {
+        const int key0 = pair_index * 32;
         // S^T = K . Q^T: lane holds head `col`, keys 4*quad + i of each tile.
         float score[8];
 #pragma unroll
@@ -174,6 +158,47 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
         for (int d = 0; d < HD_TILES; ++d) {
             o_acc[d] *= rescale;
             o_acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_frag[d].v, p_frag.v, o_acc[d], 0, 0, 0);
+        }
+    };
+    // The block table's entry for a tile, read whatever the tile (see load_pair): a tile that no query sees may
+    // have none (the table ends) or a released one (-1); load_pair reads page 0 then.
+    int no_lane = 0;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(no_lane));      // zero, but the compiler cannot tell: the entry stays in a vector
+                                                           // register and is not waited for until a round later
+    auto page_of = [&](int tile_key) -> int { return table[min(tile_key / page_size, table_width - 1) + no_lane]; };
+
+    // The wave's pairs: pair_begin + wave, then every kDecodeWaves-th. While one pair is attended to the next one's
+    // keys and values are on their way into the other set of registers, and the pages of the one after are
+    // looked up. After its last pair a wave asks for that pair again (a place that exists) and drops it.
+    int pair = pair_begin + wave;
+    if (pair < pair_end) {
+        const int last = pair + (pair_end - 1 - pair) / kDecodeWaves * kDecodeWaves;      // this wave's last pair
+        Frag8 k_first[2][K_STEPS], k_second[2][K_STEPS];
+        Frag8 v_first[HD_TILES], v_second[HD_TILES];
+        // Loads arrive in the order they were issued: a look-up is issued before the keys and values of the same
+        // round, so that waiting for it a round later does not wait for them.
+        int page[2] = {page_of(pair * 32), page_of(pair * 32 + 16)};
+        int following = min(pair + kDecodeWaves, last);
+        int next_page[2] = {page_of(following * 32), page_of(following * 32 + 16)};
+        load_pair(pair, page, k_first, v_first);
+        while (true) {
+            int after = min(following + kDecodeWaves, last);
+            page[0] = page_of(after * 32);
+            page[1] = page_of(after * 32 + 16);
+            load_pair(following, next_page, k_second, v_second);
+            attend_pair(pair, k_first, v_first);
+            if (pair == last) break;
+            pair = following;
+            following = after;
+
+            after = min(following + kDecodeWaves, last);
+            next_page[0] = page_of(after * 32);
+            next_page[1] = page_of(after * 32 + 16);
+            load_pair(following, page, k_first, v_first);
+            attend_pair(pair, k_second, v_second);
+            if (pair == last) break;
+            pair = following;
+            following = after;
         }
     }
 

@@ -474,10 +474,14 @@ def gemm_bf16_split(x: torch.Tensor, weight: torch.Tensor, parts: int) -> torch.
 
 
 def decode_splits(n_tokens: int, kv_heads: int, longest: int) -> int:
-    """How many splits of the keys: about one workgroup per compute unit, at least 256 keys each (measured on
-    MI355X: more splits cost more in joining them than they gain)."""
-    wanted = -(-256 // max(1, n_tokens * kv_heads))
-    return max(1, min(wanted, longest // 256, 256))
+    """How many splits of the keys: about one workgroup per compute unit, at least 512 keys each, and 1024 where
+    that alone fills the GPU (measured on MI355X: a wave keeps two pairs of key tiles on their way, so few long
+    splits do as well as many short ones, and joining costs more the more there are)."""
+    rows = max(1, n_tokens * kv_heads)
+    splits = max(1, min(-(-256 // rows), longest // 512, 256))
+    if splits > 1 and rows * splits >= 256 and longest // splits < 1024:
+        splits //= 2
+    return splits
 
 
 def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,

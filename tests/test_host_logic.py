@@ -42,6 +42,12 @@ def test_tiled_splits(m, n, k, splits):
     assert -(-k // 64) // splits >= (kernels.TILED_SPLIT_STAGES if splits > 1 else 0)
 
 
+@pytest.mark.parametrize("tokens,kv_heads,longest,splits", [(1, 4, 4096, 8), (8, 4, 4096, 4), (64, 4, 4096, 1), (32, 4, 16384, 2),
+                                                            (16, 4, 4096, 4), (1, 2, 300, 1), (1, 1, 100000, 195), (3, 8, 1024, 2)])
+def test_decode_splits(tokens, kv_heads, longest, splits):
+    assert kernels.decode_splits(tokens, kv_heads, longest) == splits
+
+
 def test_query_tiles_go_in_twos_that_walk_about_as_many_keys():
     # one prompt of 2048 tokens from position 0 (16 tiles), a portion of 300 from position 1000, one tile alone
     tiles = [(0, offset, 128, offset) for offset in range(0, 2048, 128)]
