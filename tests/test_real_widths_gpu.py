@@ -35,10 +35,10 @@ def model_for(tmp_path_factory, which):
     return _models[which]
 
 
-def run_trace(folder, dtype, steps, out_dir, max_tokens):
+def run_trace(folder, dtype, steps, out_dir, max_tokens, **options):
     from microllm_rocm_amd.engine import Engine
     from microllm_rocm_amd.engine.replay import replay
-    engine = Engine.from_folder(folder, dtype=dtype, max_tokens=max_tokens, max_requests=8)
+    engine = Engine.from_folder(folder, dtype=dtype, max_tokens=max_tokens, max_requests=8, **options)
     replay(engine, io.StringIO(to_lines(steps)), str(out_dir), io.StringIO())
     engine.cache.check()
     assert not engine.cache.requests
@@ -73,3 +73,20 @@ def test_real_widths_match_the_plain_implementation(tmp_path_factory, tmp_path, 
             assert np.array_equal(row, together[key]), f"mixed: {key} differs from the request run whole"
         for key, row in decoded.items():
             assert np.array_equal(row, together[key]), f"decoding: {key} differs from the request run whole"
+
+
+@pytest.mark.parametrize("which", ["7b", "0.5b"])
+def test_real_widths_with_the_packed_weights_alone(tmp_path_factory, tmp_path, which):
+    """No copy of the weights for the library: prompts go through this package's tiled product (the reduction in
+    parts where the result is narrow), mixed steps through the streaming ones."""
+    config = WIDE[which]
+    folder, plain_model = model_for(tmp_path_factory, which)
+    requests = {f"r{index}": random_tokens(60 + index, length, config.vocab_size) for index, length in enumerate([300, 70, 129, 33])}
+    steps = whole(requests)
+    engine = run_trace(folder, "bfloat16", steps, tmp_path / "whole", weight_copies="packed",
+                       max_tokens=round_up(sum(len(t) for t in requests.values()), 64) + 256)
+    assert all(block.ffn.down_weight.tensor is None for block in engine.model.blocks)
+    compare(collect(steps, tmp_path / "whole", config.vocab_size), requests, plain_model, "bfloat16")
+    steps, peak = mixed(requests, seed=9)
+    run_trace(folder, "bfloat16", steps, tmp_path / "mixed", max_tokens=peak, weight_copies="packed")
+    compare(collect(steps, tmp_path / "mixed", config.vocab_size), requests, plain_model, "bfloat16")
