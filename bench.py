@@ -42,6 +42,8 @@ def main() -> int:
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--points", default="1,64", help="other decode batch sizes to report")
     parser.add_argument("--no-prefill", action="store_true")
+    parser.add_argument("--no-library-tuning", action="store_true",
+                        help="leave the choice of the library's algorithm for the prompt's large products to its heuristic")
     parser.add_argument("--no-calibration", action="store_true", help="skip measuring what a read-only and an MFMA-only kernel reach")
     args = parser.parse_args()
     if args.gpus != 1:
@@ -63,7 +65,8 @@ def main() -> int:
     per_request = args.context + args.steps + args.warmup + 2 * page_size
     max_tokens = max(largest * per_request, args.prefill_tokens + page_size)
     engine = Engine.from_random(config, seed=0, dtype=args.dtype, device="cuda:0", on_device=True,
-                                page_size=page_size, max_tokens=max_tokens, max_requests=max(largest, 4))
+                                page_size=page_size, max_tokens=max_tokens, max_requests=max(largest, 4),
+                                tune_library=not args.no_library_tuning and not args.no_prefill)
     peak_flops = BF16_PEAK_FLOPS if args.dtype == "bfloat16" else FP32_PEAK_FLOPS
 
     results = {}
@@ -91,7 +94,8 @@ def main() -> int:
             "hidden_size": config.hidden_size, "heads": config.num_attention_heads,
             "kv_heads": config.num_key_value_heads, "head_dim": config.head_dim,
             "intermediate_size": config.intermediate_size, "vocab_size": config.vocab_size,
-            "tie_word_embeddings": config.tie_word_embeddings, "weight_copies": engine.weight_copies, "global_batch": args.batch, "seq_len": args.context,
+            "tie_word_embeddings": config.tie_word_embeddings, "weight_copies": engine.weight_copies,
+            "library_tuning": not args.no_library_tuning and not args.no_prefill, "global_batch": args.batch, "seq_len": args.context,
             "kv_block_size": page_size, "prefill_tokens": args.prefill_tokens, "parallelism": "single GPU",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

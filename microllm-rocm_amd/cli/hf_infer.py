@@ -29,6 +29,7 @@ OPTIONS: Dict[str, object] = {
     "model": None, "dtype": "bfloat16", "temperature": 0.0, "sample-top-k": 0, "seed": 1, "stop-tokens": "",
     "block-size": 16, "num-blocks": 0, "max-batched-tokens": 2048, "prefill-chunk": 512, "max-requests": 64,
     "random-config": None, "prompt-lengths": "", "prompt-seed": 0, "use-graphs": "true", "weight-copies": "auto",
+    "tune-library": "false",
 }
 
 
@@ -146,7 +147,8 @@ def run(options: Dict[str, object]) -> int:
     engine_options = dict(dtype=dtype, device="cuda:0", page_size=block_size, max_tokens=max_tokens, num_pages=num_blocks,
                           max_requests=max(int(options["max-requests"]), batch),
                           use_graphs=boolean(str(options["use-graphs"]), "--use-graphs"),
-                          weight_copies=str(options["weight-copies"]))
+                          weight_copies=str(options["weight-copies"]),
+                          tune_library=boolean(str(options["tune-library"]), "--tune-library"))
     if model_dir is not None:
         engine = Engine.from_folder(str(model_dir), **engine_options)
     else:

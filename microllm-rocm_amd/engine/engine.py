@@ -17,7 +17,7 @@ import torch
 from ..cache.manager import CacheManager, RequestCache
 from ..cache.pages import OutOfPages
 from ..config.registry import architecture_named, load_config
-from ..ops import library
+from ..ops import kernels, library
 from ..parts import Model, ModelSpec, Runtime
 from ..weights import load_folder, place_all, random_tensors
 from .batch import BatchBuilder, StepContext, StepEntry
@@ -54,14 +54,17 @@ class Engine:
                  device: Union[str, torch.device] = "cuda:0", page_size: int = 16,
                  max_tokens: Optional[int] = None, num_pages: Optional[int] = None, max_requests: int = 64,
                  tensors_placed: bool = False, use_graphs: bool = True, weight_copies: str = "auto",
-                 consume_tensors: bool = False):
+                 consume_tensors: bool = False, tune_library: bool = False):
         """``weight_copies``: a bfloat16 weight is kept ``"both"`` as stored (for the library's product of steps
         with many rows) and packed (for the streaming products), or ``"packed"`` only, where memory is short;
         ``"auto"`` keeps both if two copies and the cache fit the GPU's memory. With ``consume_tensors`` the
-        entries of ``tensors`` (a dict) are taken out as the parts take them."""
+        entries of ``tensors`` (a dict) are taken out as the parts take them. ``tune_library``: the library times
+        its candidates for the large products of prompts (``kernels.set_library_tuning``; global to the process)."""
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU is visible; this engine has no CPU path")
         library.load()  # fail now, and loudly, if the kernels are missing and cannot be built
+        if tune_library and not kernels.library_tuning():
+            kernels.set_library_tuning(True)
         self.dtype = parse_dtype(dtype)
         self.device = torch.device(device)
         torch.cuda.set_device(self.device)

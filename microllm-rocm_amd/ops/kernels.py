@@ -7,6 +7,8 @@ a kernel never sees operands that do not fit what its grid assumes.
 from __future__ import annotations
 
 import ctypes
+import os
+import tempfile
 from typing import List, NamedTuple, Optional, Sequence, Tuple
 
 import torch
@@ -418,6 +420,35 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: Optional[torc
     return out
 
 
+LIBRARY_TUNE_ROWS = 1024     # with library tuning on, bfloat16 products of this many rows or more are tuned
+_library_tuning = {"on": False, "seen": set()}
+
+
+def set_library_tuning(on: bool, results_file: Optional[str] = None) -> None:
+    """Let the library choose the algorithm of a large product by timing its candidates instead of by its
+    heuristic (the reference has --bf16-algorithm-index for that, apps/hf_infer.cpp:73). This is PyTorch's
+    TunableOp, and the switch is global to the process: the first product of a new shape with
+    ``LIBRARY_TUNE_ROWS`` rows or more and a bfloat16 result (gate/up of a prompt) then takes seconds, later ones
+    of the shape run the fastest candidate (7B sizes, 2048 rows: 0.45 instead of 0.52 ms). Results are kept in
+    ``results_file`` (default: a file of this user in the temporary folder) and found again by later processes."""
+    import torch.cuda.tunable as tunable
+    if on:
+        if results_file is None:
+            folder = os.path.join(tempfile.gettempdir(), f"microllm_rocm_amd_{os.getuid()}")
+            os.makedirs(folder, exist_ok=True)
+            results_file = os.path.join(folder, "tunableop_results.csv")
+        tunable.set_filename(results_file)
+        tunable.set_max_tuning_duration(30)
+        tunable.set_max_tuning_iterations(10)
+    tunable.enable(on)
+    tunable.tuning_enable(False)     # switched on around the first product of a shape only
+    _library_tuning["on"] = on
+
+
+def library_tuning() -> bool:
+    return _library_tuning["on"]
+
+
 def gemm_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """``x @ weight.T`` for bfloat16 operands with float32 accumulation.
 
@@ -428,6 +459,16 @@ def gemm_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = to
     _device_tensor(weight, "gemm weight", torch.bfloat16)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "gemm takes [m, k] and [n, k]")
     if out_dtype == torch.bfloat16:
+        shape = (x.shape[0], weight.shape[0], x.shape[1])
+        if _library_tuning["on"] and shape[0] >= LIBRARY_TUNE_ROWS and shape not in _library_tuning["seen"] \
+                and not torch.cuda.is_current_stream_capturing():
+            import torch.cuda.tunable as tunable
+            _library_tuning["seen"].add(shape)
+            tunable.tuning_enable(True)
+            try:
+                return torch.mm(x, weight.t())
+            finally:
+                tunable.tuning_enable(False)
         return torch.mm(x, weight.t())
     return torch.mm(x, weight.t(), out_dtype=out_dtype)
 

@@ -736,3 +736,32 @@ def test_measured_peaks_are_plausible():
     peaks = kernels().measured_peaks(read_bytes=1 << 30)
     assert 2000.0 < peaks["hbm_read_GBps"] <= 8000.0, "a read-only kernel reaches between a quarter of and the published HBM peak"
     assert 500.0 < peaks["mfma_bf16_TFLOPs"] <= 2500.0, "an MFMA-only kernel reaches at most the published dense bfloat16 peak"
+
+
+def test_library_tuning_keeps_the_product_and_is_switched_per_shape(tmp_path):
+    """With tuning on, a large bfloat16 product is tuned once per shape (PyTorch's TunableOp) and still the product;
+    small ones and float32 results go the usual way."""
+    import torch.cuda.tunable as tunable
+    ka = kernels()
+    rng = np.random.default_rng(3)
+    a_ref, a = to_bf16_exact(rng.normal(size=(ka.LIBRARY_TUNE_ROWS, 64)))
+    w_ref, w = to_bf16_exact(rng.normal(size=(48, 64)) * 0.1)
+    expected = a_ref @ w_ref.T
+    before = ka.gemm_bf16(a, w)
+    ka.set_library_tuning(True, results_file=str(tmp_path / "results.csv"))
+    try:
+        assert ka.library_tuning() and tunable.is_enabled() and not tunable.tuning_is_enabled()
+        tuned = ka.gemm_bf16(a, w)
+        assert (ka.LIBRARY_TUNE_ROWS, 48, 64) in ka._library_tuning["seen"] and not tunable.tuning_is_enabled()
+        again = ka.gemm_bf16(a, w)
+        assert torch.equal(tuned, again)
+        for out in (before, tuned):
+            assert np.abs(out.float().cpu().numpy() - expected).max() <= 5e-3 * np.abs(expected).max()
+        small = ka.gemm_bf16(a[:100].contiguous(), w)
+        assert (100, 48, 64) not in ka._library_tuning["seen"]
+        assert np.abs(small.float().cpu().numpy() - expected[:100]).max() <= 5e-3 * np.abs(expected).max()
+        wide = ka.gemm_bf16(a, w, torch.float32)
+        assert np.abs(wide.double().cpu().numpy() - expected).max() <= 1e-5 * np.abs(expected).max()
+    finally:
+        ka.set_library_tuning(False)
+    assert not ka.library_tuning() and not tunable.is_enabled()
