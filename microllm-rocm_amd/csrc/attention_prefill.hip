@@ -141,6 +141,7 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
 
     floatx4 o_acc[2][HD_TILES];
     float running_max[2] = {-INFINITY, -INFINITY}, running_sum[2] = {0.0f, 0.0f};
+    float running_offset[2] = {0.0f, 0.0f};      // -(running maximum) in units of log 2; 0 while the maximum is -inf
 #pragma unroll
     for (int c = 0; c < 2; ++c)
 #pragma unroll
@@ -282,12 +283,21 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
             float tile_max = score[0];
 #pragma unroll
             for (int j = 1; j < 8; ++j) tile_max = fmaxf(tile_max, score[j]);
-            tile_max = max_lanes_16_apart(tile_max);
-            const float new_max = fmaxf(running_max[c], tile_max);
-            // A query may see nothing of a pair that others see (the window's edge): its maximum stays -inf.
-            const float safe_max = (MASKED && new_max == -INFINITY) ? 0.0f : new_max;
-            const float offset = -safe_max * scale_log2;
-            rescale[c] = __builtin_amdgcn_exp2f(fmaf(running_max[c], scale_log2, offset));
+            // Far into a prompt a pair rarely holds a new maximum for any of the wave's tokens: then the four
+            // lanes of a token need not compare notes, and nothing is rescaled (the same numbers either way).
+            rescale[c] = 1.0f;
+            if (__any(tile_max > running_max[c])) {
+                tile_max = max_lanes_16_apart(tile_max);
+                const float new_max = fmaxf(running_max[c], tile_max);
+                // A query may see nothing of a pair that others see (the window's edge): its maximum stays -inf.
+                const float safe_max = (MASKED && new_max == -INFINITY) ? 0.0f : new_max;
+                running_offset[c] = -safe_max * scale_log2;
+                // exactly 1 for a token whose maximum stays (the rounding of maximum * scale would else leave a factor
+                // of 1 +- 1e-7, and every sum would be multiplied by it)
+                rescale[c] = new_max == running_max[c] ? 1.0f : __builtin_amdgcn_exp2f(fmaf(running_max[c], scale_log2, running_offset[c]));
+                running_max[c] = new_max;
+            }
+            const float offset = running_offset[c];
             float tile_sum = 0.0f;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
@@ -297,7 +307,6 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
             }
             tile_sum = sum_lanes_16_apart(tile_sum);
             running_sum[c] = running_sum[c] * rescale[c] + tile_sum;
-            running_max[c] = new_max;
         }
         // Once the running maxima have settled, no column's sum needs rescaling: one branch for the whole wave.
         if (__any(rescale[0] != 1.0f || rescale[1] != 1.0f)) {
