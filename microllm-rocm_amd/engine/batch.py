@@ -92,6 +92,17 @@ class BatchBuilder:
             self._copied.synchronize()  # the last step's copy has left the staging buffer
         return self._staging, self._device_buffer
 
+    def fill_tokens(self, tokens: Sequence[int]) -> None:
+        """Put the tokens of a step of single tokens into the buffers that ``build`` filled for it ahead of time
+        (with any tokens): they lie first in the packed buffer."""
+        count = len(tokens)
+        if self._copied is not None:
+            self._copied.synchronize()
+        self._staging.numpy()[:count] = tokens
+        self._device_buffer[:count].copy_(self._staging[:count], non_blocking=True)
+        self._copied = torch.cuda.Event()
+        self._copied.record()
+
     def build(self, requests: Sequence[RequestCache], token_lists: Sequence[Sequence[int]],
               wants: Sequence[Sequence[int]], fixed_width: Optional[int] = None) -> StepContext:
         page_size = self.cache.page_size

@@ -49,6 +49,22 @@ class _DecodeGraph:
         self.logits: Optional[torch.Tensor] = None
 
 
+class _BuiltAhead:
+    """The metadata of the decode step that is likely to come next, built while the GPU runs this one: the same
+    requests, one more token each. What it was built from is kept, to tell whether it still holds."""
+
+    def __init__(self, state: _DecodeGraph, ctx: StepContext, requests: List[RequestCache]):
+        self.state, self.ctx, self.requests = state, ctx, requests
+        self.num_tokens = [request.num_tokens for request in requests]
+        self.page_counts = [[len(pages) for pages in request.pages] for request in requests]
+
+    def holds_for(self, state: _DecodeGraph, requests: List[RequestCache]) -> bool:
+        return (state is self.state and len(requests) == len(self.requests)
+                and all(now is then for now, then in zip(requests, self.requests))
+                and all(request.num_tokens == count for request, count in zip(requests, self.num_tokens))
+                and all([len(pages) for pages in request.pages] == counts for request, counts in zip(requests, self.page_counts)))
+
+
 class Engine:
     def __init__(self, spec: ModelSpec, tensors: Mapping[str, torch.Tensor], dtype: Union[str, torch.dtype] = "bfloat16",
                  device: Union[str, torch.device] = "cuda:0", page_size: int = 16,
@@ -63,6 +79,9 @@ class Engine:
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU is visible; this engine has no CPU path")
         library.load()  # fail now, and loudly, if the kernels are missing and cannot be built
+        self._ahead: Optional[_BuiltAhead] = None
+        self.steps_built_ahead = 0      # decode steps whose metadata was ready when they came
+        self._last_graph: Optional[_DecodeGraph] = None
         if tune_library and not kernels.library_tuning():
             kernels.set_library_tuning(True)
         self.dtype = parse_dtype(dtype)
@@ -158,9 +177,15 @@ class Engine:
         state = self._graphs.get(key)
         if state is None:
             state = self._graphs[key] = _DecodeGraph(self, width)
-        tokens = [entry.tokens for entry in entries]
         every_row = [[0]] * n   # the graph computes the logits of every row; the wanted ones are picked after
-        ctx = state.builder.build(requests, tokens, every_row, fixed_width=width)
+        ahead, self._ahead = self._ahead, None
+        if ahead is not None and state.graph is not None and ahead.holds_for(state, requests):
+            state.builder.fill_tokens([entry.tokens[0] for entry in entries])
+            ctx = ahead.ctx
+            self.steps_built_ahead += 1
+        else:
+            ctx = state.builder.build(requests, [entry.tokens for entry in entries], every_row, fixed_width=width)
+        self._last_graph = state
         if state.graph is None:
             # Once eagerly (libraries create their handles and workspaces), then the capture. The step writes
             # the same keys and values to the same slots each time, so running it twice changes nothing.
@@ -225,9 +250,26 @@ class Engine:
         if self.use_graphs and len(entries) <= MAX_GRAPH_REQUESTS and all(len(entry.tokens) == 1 for entry in entries):
             logits = self._graph_step(requests, entries)
         else:
+            self._last_graph = None
             ctx = self._builder.build(requests, [entry.tokens for entry in entries], [entry.want for entry in entries])
             logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
         for request, entry in zip(requests, entries):
             self.cache.commit(request, len(entry.tokens))
         self.steps_run += 1
+        if self._last_graph is not None:
+            self._build_ahead(self._last_graph, requests)
         return logits
+
+    def _build_ahead(self, state: _DecodeGraph, requests: List[RequestCache]) -> None:
+        """After a decode step from a graph: the next one's metadata (positions, slots, block tables), while the
+        GPU is busy with this one. Only where every request has room for one more position in the pages it holds
+        and the block tables keep their width; the tokens are filled in when the step comes."""
+        self._last_graph = None
+        if state.graph is None or any(need for request in requests for need in self.cache.pages_needed(request, 1)):
+            return
+        widest = -(-(max(request.num_tokens for request in requests) + 1) // self.cache.page_size)
+        if max(MIN_GRAPH_WIDTH, 1 << (max(widest, 1) - 1).bit_length()) != state.width:
+            return
+        count = len(requests)
+        ctx = state.builder.build(requests, [[0]] * count, [[0]] * count, fixed_width=state.width)
+        self._ahead = _BuiltAhead(state, ctx, list(requests))

@@ -107,11 +107,19 @@ def test_every_replay_of_a_decode_graph_equals_the_eager_step(tmp_path, dtype):
         if step == 25:      # a request leaves: the graph for two requests again
             for engine in (graphs, eager):
                 engine.close("b")
+        if step == 31:      # a request ends and another comes under its name, as long as the old one was
+            for engine in (graphs, eager):
+                length = engine.cache.get("a").num_tokens
+                engine.close("a"), engine.open("a")
+            both([("a", random_tokens(99, length, config.vocab_size), [])])
         live = [name for name in ("a", "b", "c") if graphs.is_open(name)]
         wanted = [[0], [], [0]] if step % 7 == 3 else [[0]] * 3        # logits of some requests only
         both([(name, [token], want) for name, token, want in zip(live, tokens, wanted)])
         replays += 1
     assert graphs.graph_replays == replays and eager.graph_replays == 0
+    # most replays found their metadata built while the step before ran (not the first of a graph, not those at a
+    # page's edge or after another kind of step), and none took what was built for other requests
+    assert replays // 2 < graphs.steps_built_ahead < replays
     assert len(graphs._graphs) >= 2, "more than one graph was captured (two and three requests)"
     for engine in (graphs, eager):
         engine.cache.check()
