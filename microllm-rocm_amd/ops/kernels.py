@@ -420,17 +420,21 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: Optional[torc
     return out
 
 
-LIBRARY_TUNE_ROWS = 1024     # with library tuning on, bfloat16 products of this many rows or more are tuned
-_library_tuning = {"on": False, "seen": set()}
+LIBRARY_TUNE_ROWS = 1024     # with library tuning on, bfloat16 products of this many rows or more are tuned,
+LIBRARY_TUNE_DECODE_ROWS = 64     # and those of up to this many (the gate/up product of large decode batches); between
+                                  # the two a serving engine meets too many shapes, and short tuning runs mislead
+_library_tuning = {"on": False, "seen": set(), "plain": set()}
 
 
 def set_library_tuning(on: bool, results_file: Optional[str] = None) -> None:
     """Let the library choose the algorithm of a large product by timing its candidates instead of by its
     heuristic (the reference has --bf16-algorithm-index for that, apps/hf_infer.cpp:73). This is PyTorch's
-    TunableOp, and the switch is global to the process: the first product of a new shape with
-    ``LIBRARY_TUNE_ROWS`` rows or more and a bfloat16 result (gate/up of a prompt) then takes seconds, later ones
-    of the shape run the fastest candidate (7B sizes, 2048 rows: 0.45 instead of 0.52 ms). Results are kept in
-    ``results_file`` (default: a file of this user in the temporary folder) and found again by later processes."""
+    TunableOp, and the switch is global to the process: the first bfloat16-result product of a new shape with
+    ``LIBRARY_TUNE_ROWS`` rows or more (gate/up of a prompt), or with at most ``LIBRARY_TUNE_DECODE_ROWS``, then
+    takes seconds; later ones of the shape run the fastest candidate (7B sizes, 2048 rows: 0.45 instead of
+    0.52 ms), or the heuristic's choice where that proves faster when the two are timed by turns. Results are
+    kept in ``results_file`` (default: a file of this user in the temporary folder) and found again by later
+    processes."""
     import torch.cuda.tunable as tunable
     if on:
         if results_file is None:
@@ -449,6 +453,34 @@ def library_tuning() -> bool:
     return _library_tuning["on"]
 
 
+def _tune_product(x: torch.Tensor, transposed_weight: torch.Tensor, shape: Tuple[int, int, int]) -> None:
+    """Tune one shape, then time the tuned choice and the heuristic's by turns: the tuner's own runs are short."""
+    import torch.cuda.tunable as tunable
+    _library_tuning["seen"].add(shape)
+    tunable.tuning_enable(True)
+    try:
+        torch.mm(x, transposed_weight)
+    finally:
+        tunable.tuning_enable(False)
+    times = {True: 0.0, False: 0.0}
+    try:
+        for _ in range(3):
+            for tuned in (True, False):
+                tunable.enable(tuned)
+                torch.mm(x, transposed_weight)
+                start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record()
+                for _ in range(10):
+                    torch.mm(x, transposed_weight)
+                stop.record()
+                stop.synchronize()
+                times[tuned] += start.elapsed_time(stop)
+    finally:
+        tunable.enable(True)
+    if times[False] < times[True]:
+        _library_tuning["plain"].add(shape)
+
+
 def gemm_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """``x @ weight.T`` for bfloat16 operands with float32 accumulation.
 
@@ -458,19 +490,21 @@ def gemm_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = to
     _device_tensor(x, "gemm input", torch.bfloat16)
     _device_tensor(weight, "gemm weight", torch.bfloat16)
     _need(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1], "gemm takes [m, k] and [n, k]")
-    if out_dtype == torch.bfloat16:
+    if out_dtype != torch.bfloat16:
+        return torch.mm(x, weight.t(), out_dtype=out_dtype)
+    if _library_tuning["on"]:
         shape = (x.shape[0], weight.shape[0], x.shape[1])
-        if _library_tuning["on"] and shape[0] >= LIBRARY_TUNE_ROWS and shape not in _library_tuning["seen"] \
-                and not torch.cuda.is_current_stream_capturing():
+        tuned_rows = shape[0] >= LIBRARY_TUNE_ROWS or 0 < shape[0] <= LIBRARY_TUNE_DECODE_ROWS
+        if tuned_rows and shape not in _library_tuning["seen"] and not torch.cuda.is_current_stream_capturing():
+            _tune_product(x, weight.t(), shape)
+        if shape in _library_tuning["plain"]:
             import torch.cuda.tunable as tunable
-            _library_tuning["seen"].add(shape)
-            tunable.tuning_enable(True)
+            tunable.enable(False)
             try:
                 return torch.mm(x, weight.t())
             finally:
-                tunable.tuning_enable(False)
-        return torch.mm(x, weight.t())
-    return torch.mm(x, weight.t(), out_dtype=out_dtype)
+                tunable.enable(True)
+    return torch.mm(x, weight.t())
 
 
 LIBRARY_TILE = 256          # the library's products of many rows work in tiles of about 256 x 256
