@@ -178,21 +178,38 @@ def run(options: Dict[str, object]) -> int:
                                         seed=params.seed + index, stop_tokens=stop_tokens)
                        for index, new in enumerate(new_lengths)]
         slots = int(options["continuous-slots"]) or None
+
+        def run_once():
+            return generate(engine, prompts, per_request, max_batched_tokens=int(options["max-batched-tokens"]),
+                            prefill_chunk=int(options["prefill-chunk"]), max_requests=slots,
+                            arrival_steps=arrivals, return_scheduler=True)
+
+        # The whole workload runs --warmup times untimed and --steps times timed; every timed run must generate the
+        # same tokens (apps/hf_infer.cpp:862-900).
         torch.cuda.synchronize()
         begun = time.perf_counter()
-        outputs, scheduler = generate(engine, prompts, per_request, max_batched_tokens=int(options["max-batched-tokens"]),
-                                      prefill_chunk=int(options["prefill-chunk"]), max_requests=slots,
-                                      arrival_steps=arrivals, return_scheduler=True)
+        for _ in range(int(options["warmup"])):
+            run_once()
         torch.cuda.synchronize()
-        elapsed = time.perf_counter() - begun
+        warmup_ms = (time.perf_counter() - begun) * 1e3
+        elapsed, outputs, scheduler = 0.0, None, None
+        for _ in range(max(1, int(options["steps"]))):
+            begun = time.perf_counter()
+            current, scheduler = run_once()
+            torch.cuda.synchronize()
+            elapsed += time.perf_counter() - begun
+            if outputs is not None and current != outputs:
+                raise RuntimeError("continuous generation changed across measured runs")
+            outputs = current
         generated = [output[len(prompt):] for output, prompt in zip(outputs, prompts)]
         metrics = scheduler.metrics
         requests = [scheduler.request(index) for index in range(len(prompts))]
         report.update({
             "request_count": len(prompts), "continuous_slots": slots or engine.cache.max_requests,
             "prompt_lengths": lengths, "new_token_lengths": new_lengths, "arrival_steps": arrivals, "prompt_offsets": offsets,
-            "measured_ms": round(elapsed * 1e3, 3), "measured_tokens": sum(len(g) for g in generated),
-            "tokens_per_second": round(sum(len(g) for g in generated) / elapsed, 3),
+            "warmup": int(options["warmup"]), "steps": max(1, int(options["steps"])), "warmup_ms": round(warmup_ms, 3),
+            "measured_ms": round(elapsed * 1e3, 3), "measured_tokens": sum(len(g) for g in generated) * max(1, int(options["steps"])),
+            "tokens_per_second": round(sum(len(g) for g in generated) * max(1, int(options["steps"])) / elapsed, 3),
             "scheduler_steps": metrics.scheduler_steps, "slot_admissions": metrics.admissions,
             "preemptions": metrics.preemptions, "prefill_tokens": metrics.prefill_tokens, "decode_tokens": metrics.decode_tokens,
             "completed_requests": metrics.completed_requests, "peak_active_requests": metrics.peak_active_requests,

@@ -45,7 +45,7 @@ class CompletionReason(enum.Enum):
     CANCELLED = "cancelled"
 
 
-@dataclass
+@dataclass(eq=False)      # a request is itself: membership and removal go by identity, not by comparing prompts
 class Request:
     id: int
     prompt: List[int]
@@ -92,7 +92,7 @@ class SchedulerMetrics:
     peak_held_pages: int = 0
 
 
-@dataclass
+@dataclass(eq=False)
 class Portion:
     """What one request brings to a step."""
     request: Request

@@ -174,10 +174,13 @@ def test_command_line(tmp_path):
     continuous = subprocess.run(command[:6] + ["--tokens", ",".join(map(str, prompt)), "--device", "hip", "--dtype", "float32",
                                                "--workload", "continuous", "--continuous-prompt-lengths", "5,9,7",
                                                "--continuous-new-token-lengths", "4,6,3", "--continuous-arrival-steps", "0,1,1",
-                                               "--continuous-slots", "2"], capture_output=True, text=True, timeout=300)
+                                               "--continuous-slots", "2", "--warmup", "1", "--steps", "2"],
+                                capture_output=True, text=True, timeout=300)
     assert continuous.returncode == 0, continuous.stderr
     report = json.loads(continuous.stdout.strip().splitlines()[-1])
     assert report["completed_requests"] == 3 and [len(r) for r in report["generated"]] == [4, 6, 3]
+    # the workload ran once untimed and twice timed, with the same tokens both times
+    assert report["warmup"] == 1 and report["steps"] == 2 and report["measured_tokens"] == 2 * 13 and report["warmup_ms"] > 0
     for generated, length, new in zip(report["generated"], (5, 9, 7), (4, 6, 3)):
         cyclic = [prompt[i % len(prompt)] for i in range(length)]
         assert generated == plain.generate_greedy(model.config, model.weights, cyclic, new)
