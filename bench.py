@@ -42,6 +42,8 @@ def main() -> int:
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--points", default="1,64", help="other decode batch sizes to report")
     parser.add_argument("--no-prefill", action="store_true")
+    parser.add_argument("--weight-copies", default="auto", choices=["auto", "both", "packed"],
+                        help="packed: one copy of every weight, and this package's own matrix kernels for every product")
     parser.add_argument("--no-library-tuning", action="store_true",
                         help="leave the choice of the library's algorithm for the prompt's large products to its heuristic")
     parser.add_argument("--no-calibration", action="store_true", help="skip measuring what a read-only and an MFMA-only kernel reach")
@@ -66,6 +68,7 @@ def main() -> int:
     max_tokens = max(largest * per_request, args.prefill_tokens + page_size)
     engine = Engine.from_random(config, seed=0, dtype=args.dtype, device="cuda:0", on_device=True,
                                 page_size=page_size, max_tokens=max_tokens, max_requests=max(largest, 4),
+                                weight_copies=args.weight_copies,
                                 tune_library=not args.no_library_tuning and not args.no_prefill)
     peak_flops = BF16_PEAK_FLOPS if args.dtype == "bfloat16" else FP32_PEAK_FLOPS
 
