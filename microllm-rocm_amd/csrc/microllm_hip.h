@@ -164,8 +164,12 @@ int mll_argmax_slices(int vocab);
 // Draws one token per row from softmax(logits / temperature) restricted to the top_k largest
 // logits (top_k <= 0: all; ties at the k-th value go to the lower token ids), by inverse CDF in
 // token order with the given uniform in [0, 1). temperature == 0 or top_k == 1 gives the
-// argmax. A non-finite logit gives -1. top_k may be null.
+// argmax. A non-finite logit gives -1. top_k may be null (no row is restricted: the search for the
+// k-th value is left out). `workspace`: mll_sample_workspace(n_rows, vocab) bytes of device scratch,
+// 4-byte aligned; its contents need not be cleared.
 int mll_sample(const float* logits, const float* temperature, const int32_t* top_k,
-               const float* uniform, int32_t* out, int n_rows, int vocab, hipStream_t stream);
+               const float* uniform, int32_t* out, void* workspace, int n_rows, int vocab,
+               hipStream_t stream);
+int64_t mll_sample_workspace(int n_rows, int vocab);
 
 }  // extern "C"

@@ -415,7 +415,8 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: Optional[torc
         _device_tensor(top_k, "top_k", torch.int32)
         _need(top_k.shape[0] == rows, "one top_k per row")
     out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
-    _check(lib.mll_sample(_ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(uniform), _ptr(out),
+    workspace = torch.empty((lib.mll_sample_workspace(rows, logits.shape[1]) // 4,), dtype=torch.int32, device=logits.device)
+    _check(lib.mll_sample(_ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(uniform), _ptr(out), _ptr(workspace),
                           rows, logits.shape[1], _stream()), lib)
     return out
 

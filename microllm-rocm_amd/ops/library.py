@@ -150,6 +150,7 @@ def load() -> ctypes.CDLL:
     except OSError as error:
         raise KernelLibraryError(f"cannot load {path}: {error}") from error
     _library.mll_last_error.restype = ctypes.c_char_p
+    _library.mll_sample_workspace.restype = ctypes.c_int64
     return _library
 
 

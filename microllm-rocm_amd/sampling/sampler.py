@@ -16,6 +16,7 @@ import math
 from dataclasses import dataclass, field
 from typing import List, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from ..ops import kernels
@@ -72,10 +73,15 @@ class Sampler:
         if all(p.greedy for p in params):
             chosen = kernels.argmax(logits)
         else:
-            device = logits.device
-            temperature = torch.tensor([0.0 if p.greedy else p.temperature for p in params], dtype=torch.float32, device=device)
-            top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32, device=device)
-            uniform = torch.tensor([uniform_for(p.seed, d) for p, d in zip(params, draws)], dtype=torch.float32, device=device)
+            # one transfer for the three per-row values: temperatures, top-k counts (as int32 bits) and uniforms
+            packed = np.empty((3, len(params)), dtype=np.float32)
+            packed[0] = [0.0 if p.greedy else p.temperature for p in params]
+            packed[1].view(np.int32)[:] = [p.top_k for p in params]
+            packed[2] = [uniform_for(p.seed, d) for p, d in zip(params, draws)]
+            on_device = torch.from_numpy(packed).to(logits.device)
+            temperature, top_k, uniform = on_device[0], on_device[1].view(torch.int32), on_device[2]
+            if all(p.top_k == 0 for p in params):
+                top_k = None      # no row is restricted: the kernel leaves its search for the k-th value out
             chosen = kernels.sample(logits, temperature, top_k, uniform)
         tokens = chosen.tolist()
         for row, token in enumerate(tokens):

@@ -410,7 +410,8 @@ def test_argmax_rules():
     assert k.argmax(torch.from_numpy(big[:, :331].copy()).to(DEVICE)).tolist() == np.argmax(big[:, :331], axis=1).tolist()
 
 
-@pytest.mark.parametrize("vocab,top_k", [(331, 0), (331, 5), (5000, 50), (152064, 0), (152064, 40), (40, 40), (40, 39)])
+@pytest.mark.parametrize("vocab,top_k", [(331, 0), (331, 5), (5000, 50), (152064, 0), (152064, 40), (40, 40), (40, 39),
+                                         (9001, 3000), (152064, 100000), (2049, 2)])
 def test_sampling_follows_the_plain_rule(vocab, top_k):
     rng = np.random.default_rng(vocab + top_k)
     rows = 24
@@ -440,6 +441,33 @@ def test_sampling_follows_the_plain_rule(vocab, top_k):
     out = kernels().sample(torch.from_numpy(bad).to(DEVICE), torch.from_numpy(temperature).to(DEVICE), None,
                            torch.from_numpy(uniform).to(DEVICE)).tolist()
     assert out[4] == -1 and all(token >= 0 for index, token in enumerate(out) if index != 4)
+
+
+def test_sampling_with_a_rule_per_row_and_draws_at_both_ends():
+    """Rows of one call differ in top_k and temperature; uniforms near 0 and near 1 fall into the first and the
+    last selected tokens, which lie in different slices of the row."""
+    rng = np.random.default_rng(11)
+    vocab, rows = 50021, 12
+    logits = (rng.normal(size=(rows, vocab)) * 1.5).astype(np.float32)
+    top_k = np.array([0, 1, 7, 300, 0, 50020, 2, 0, 9, 9, 0, 1000], dtype=np.int32)
+    temperature = np.array([0.9, 1.0, 1.1, 0.6, 0.0, 1.0, 0.8, 2.0, 0.7, 0.7, 1.0, 1.4], dtype=np.float32)
+    uniform = np.array([0.0, 0.5, 0.999999, 0.0, 0.3, 0.999999, 0.5, 0.999999, 0.0, 0.999999, 1e-7, 0.25], dtype=np.float32)
+    chosen = kernels().sample(torch.from_numpy(logits).to(DEVICE), torch.from_numpy(temperature).to(DEVICE),
+                              torch.from_numpy(top_k).to(DEVICE), torch.from_numpy(uniform).to(DEVICE)).tolist()
+    for row in range(rows):
+        row_logits = logits[row].astype(np.float64)
+        if temperature[row] == 0.0 or top_k[row] == 1:
+            assert chosen[row] == plain.greedy(row_logits)
+            continue
+        weights = plain.sampling_weights(row_logits, float(temperature[row]), int(top_k[row]))
+        assert weights[chosen[row]] > 0.0
+        cumulative = np.cumsum(weights)
+        target = float(uniform[row]) * cumulative[-1]
+        slack = 2e-4 * cumulative[-1]
+        assert cumulative[chosen[row]] - weights[chosen[row]] - slack <= target <= cumulative[chosen[row]] + slack, row
+    selected = np.flatnonzero(plain.sampling_weights(logits[2].astype(np.float64), 1.1, 7))
+    assert chosen[0] == 0 and chosen[2] == selected[-1] and chosen[8] == np.flatnonzero(
+        plain.sampling_weights(logits[8].astype(np.float64), 0.7, 9))[0]
 
 
 def test_sampling_frequencies():
