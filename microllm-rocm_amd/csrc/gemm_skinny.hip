@@ -39,7 +39,7 @@ __device__ inline float silu_f(float value) {
 // if one is given (at most 16 rows).
 // TEMPORAL: W is read with ordinary loads instead of non-temporal ones (measured on MI355X: better for weights
 // of a few tens of MB, worse for the large ones).
-template <int MT, int NT, int EPILOGUE, bool TEMPORAL, bool SCALED>
+template <int MT, int NT, int EPILOGUE, bool TEMPORAL, bool SCALED, bool PAIRED>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w_packed, void* __restrict__ out,
     int m, int n, int k, int n_tiles, int k_steps, MllSkinnyExtras extras) {
@@ -122,6 +122,13 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
         a_live[mt] = row < m;
         a_ptr[mt] = a + static_cast<int64_t>(a_live[mt] ? row : 0) * k + quad * 8;
     }
+    // PAIRED (one tile of rows, more than two rows): the activations are read two k steps at a time: lanes 0..7 of every 16 read rows
+    // 0..7 (then 8..15) at one step and lanes 8..15 the same rows at the next, so that a load touches whole 128-byte
+    // lines of 8 rows instead of half lines of 16; lanes 8 apart then exchange what the other needs.
+    const bool upper = col >= 8;
+    const bool low_live = (col & 7) < m, high_live = (col & 7) + 8 < m;
+    const bf16* a_low = a + static_cast<int64_t>(low_live ? (col & 7) : 0) * k + quad * 8;
+    const bf16* a_high = a + static_cast<int64_t>(high_live ? (col & 7) + 8 : 0) * k + quad * 8;
 
     // A wave takes kChunk consecutive k steps at a time, then skips what the other waves take (the last wave
     // begins, so that wave 0, which also writes the result, never has more chunks than another); which k steps a
@@ -146,12 +153,40 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
                                      : __builtin_nontemporal_load(
                                            reinterpret_cast<const uintx4*>(w_ptr[nt] + static_cast<int64_t>(ks) * 512));
                 }
-                const int k_offset = ks * 32;
-                const bool in_k = live && k_offset + quad * 8 < k;
+                if constexpr (PAIRED) {
+                    // a_piece[u] of an even u: rows 0..7 (both steps of the pair); of the odd u after it: rows 8..15
+                    const int own = (ks & ~1) + (upper ? 1 : 0);
+                    const int k_offset = own * 32;
+                    const bool in_k = own < k_steps && k_offset + quad * 8 < k;
+                    const bool rows_live = (u & 1) ? high_live : low_live;
+                    a_piece[u][0].raw = uintx4{0u, 0u, 0u, 0u};
+                    if (rows_live && in_k)
+                        a_piece[u][0].raw = *reinterpret_cast<const uintx4*>(((u & 1) ? a_high : a_low) + k_offset);
+                } else {
+                    const int k_offset = ks * 32;
+                    const bool in_k = live && k_offset + quad * 8 < k;
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) {
-                    a_piece[u][mt].raw = uintx4{0u, 0u, 0u, 0u};
-                    if (a_live[mt] && in_k) a_piece[u][mt].raw = *reinterpret_cast<const uintx4*>(a_ptr[mt] + k_offset);
+                    for (int mt = 0; mt < MT; ++mt) {
+                        a_piece[u][mt].raw = uintx4{0u, 0u, 0u, 0u};
+                        if (a_live[mt] && in_k) a_piece[u][mt].raw = *reinterpret_cast<const uintx4*>(a_ptr[mt] + k_offset);
+                    }
+                }
+            }
+            if constexpr (PAIRED) {
+                // low = rows 0..7 at the pair's first step (lanes 0..7) and its second (lanes 8..15), high = rows
+                // 8..15 likewise. The first step's operand: own low | the partner's high; the second's: the partner's
+                // low | own high.
+#pragma unroll
+                for (int u = 0; u < DEPTH; u += 2) {
+                    const uintx4 low = a_piece[u][0].raw, high = a_piece[u + 1][0].raw;
+                    uintx4 low_swapped, high_swapped;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        low_swapped[i] = static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(low[i]), 0x128, 0xf, 0xf, false));
+                        high_swapped[i] = static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(high[i]), 0x128, 0xf, 0xf, false));
+                    }
+                    a_piece[u][0].raw = upper ? high_swapped : low;
+                    a_piece[u + 1][0].raw = upper ? high : low_swapped;
                 }
             }
 #pragma unroll
@@ -309,20 +344,29 @@ static void launch_one(const bf16* a, const bf16* w, void* out, int m, int n, in
     size_t lds = waves > 1 ? static_cast<size_t>(waves - 1) * NT * MT * kWave * sizeof(floatx4) : 0;
     const bool temporal = static_cast<int64_t>(n_tiles) * k_steps * 1024 < (64ll << 20);   // bytes of the packed weight
     const bool scaled = extras.scale.sumsq != nullptr;
+    // PAIRED pays from three rows on (measured on MI355X: 18944 x 3584 at 8 rows 27 -> 25.6 us, at 16 rows 34 -> 30.7;
+    // at one row 22.8 -> 24.4).
+#define MLL_SKINNY_LAUNCH(TEMPORAL_, SCALED_, PAIRED_)                                                                 \
+    gemm_skinny_kernel<MT, NT, EPILOGUE, TEMPORAL_, SCALED_, PAIRED_><<<groups, waves * kWave, lds, stream>>>(         \
+        a, w, out, m, n, k, n_tiles, k_steps, extras)
     if constexpr (MT == 1) {
+        const bool paired = m > 2;
         if (scaled) {
             lds += (static_cast<size_t>(m) * extras.scale.stride * sizeof(float) + 1023) / 1024 * 1024;
-            if (temporal)
-                gemm_skinny_kernel<MT, NT, EPILOGUE, true, true><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps, extras);
-            else
-                gemm_skinny_kernel<MT, NT, EPILOGUE, false, true><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps, extras);
-            return;
+            if (temporal) {
+                if (paired) MLL_SKINNY_LAUNCH(true, true, true); else MLL_SKINNY_LAUNCH(true, true, false);
+            } else {
+                if (paired) MLL_SKINNY_LAUNCH(false, true, true); else MLL_SKINNY_LAUNCH(false, true, false);
+            }
+        } else if (temporal) {
+            if (paired) MLL_SKINNY_LAUNCH(true, false, true); else MLL_SKINNY_LAUNCH(true, false, false);
+        } else {
+            if (paired) MLL_SKINNY_LAUNCH(false, false, true); else MLL_SKINNY_LAUNCH(false, false, false);
         }
+    } else {
+        if (temporal) MLL_SKINNY_LAUNCH(true, false, false); else MLL_SKINNY_LAUNCH(false, false, false);
     }
-    if (temporal)
-        gemm_skinny_kernel<MT, NT, EPILOGUE, true, false><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps, extras);
-    else
-        gemm_skinny_kernel<MT, NT, EPILOGUE, false, false><<<groups, waves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps, extras);
+#undef MLL_SKINNY_LAUNCH
 }
 
 // Tiles of W a workgroup takes. Few tiles of W: one, so that the GPU is filled. Many tiles of W, or several rows of
