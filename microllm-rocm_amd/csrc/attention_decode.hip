@@ -272,17 +272,34 @@ __global__ void paged_attention_join_kernel(const float* __restrict__ part_o, co
     const int token = token_ids ? token_ids[blockIdx.x / heads] : blockIdx.x / heads;
     const int64_t row = static_cast<int64_t>(token) * heads + blockIdx.x % heads;
     const int64_t part_row = blockIdx.x;
-    const float* ml = part_ml + part_row * n_splits * 2;
+    // Eight splits at a time: their loads are asked for together, then used in the order of the splits.
+    const float2* ml = reinterpret_cast<const float2*>(part_ml) + part_row * n_splits;
     float top = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) top = fmaxf(top, ml[2 * s]);
+    for (int base = 0; base < n_splits; base += 8) {
+        float2 pair[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pair[j] = ml[min(base + j, n_splits - 1)];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) top = fmaxf(top, pair[j].x);
+    }
     for (int dim = threadIdx.x; dim < head_dim; dim += blockDim.x) {
         float total = 0.0f, weight_sum = 0.0f;
-        for (int s = 0; s < n_splits; ++s) {
-            const float m = ml[2 * s];
-            if (m == -INFINITY) continue;   // a split without keys
-            const float weight = __expf(m - top);
-            total += weight * part_o[(part_row * n_splits + s) * head_dim + dim];
-            weight_sum += weight * ml[2 * s + 1];
+        for (int base = 0; base < n_splits; base += 8) {
+            float2 pair[8];
+            float part[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int split = min(base + j, n_splits - 1);
+                pair[j] = ml[split];
+                part[j] = part_o[(part_row * n_splits + split) * head_dim + dim];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                if (base + j >= n_splits || pair[j].x == -INFINITY) continue;   // past the end, or a split without keys
+                const float weight = __expf(pair[j].x - top);
+                total += weight * part[j];
+                weight_sum += weight * pair[j].y;
+            }
         }
         out[row * head_dim + dim] = from_float<bf16>(total / weight_sum);
     }
