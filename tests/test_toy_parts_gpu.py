@@ -205,3 +205,89 @@ def test_toy_position_and_routed_feed_forward_in_one_model(toys_registered, dtyp
     # the routed feed-forward really routes: every expert is chosen by some token
     w = {name: value.double().numpy() for name, value in tensors.items()}
     assert len(set(np.argmax(np.random.default_rng(0).normal(size=(200, HIDDEN)) @ w["layers.1.ffn.router"].T, axis=1))) == EXPERTS
+
+
+# ---- a toy arrangement ---------------------------------------------------------------------------------------------
+def parallel_block_class():
+    """A toy arrangement from the package's ``Block``: mixer and feed-forward both read the first norm's output and
+    their results are added to the stream together (the second norm is declared, since a layer's spec names two, and
+    not used). It takes no part in the fusing of sums and norms across blocks."""
+    from microllm_rocm_amd.parts import Block
+
+    class Parallel(Block):
+        def first_norm_after(self, producer, rows, h):
+            return None       # the block before hands its delta on as it is
+
+        def forward(self, h, pending, ctx, cache, next_block=None):
+            x = self.mixer_norm.forward(h, delta=pending, write_h=True)
+            deltas = (self.mixer.forward(x, ctx, cache), self.ffn.forward(x, ctx))
+            # a delta is [rows, width] or partial sums [parts, rows, width]: all of them go on as partial sums
+            return torch.cat([delta.float().reshape(-1, *h.shape) for delta in deltas])
+
+    return Parallel
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_arrangement_beside_the_packages_own(dtype):
+    from microllm_rocm_amd.parts import register_arrangement
+    register_arrangement("toy_parallel", parallel_block_class(), replace=True)
+    layers = []
+    for index, arrangement in enumerate(("toy_parallel", "pre_norm", "toy_parallel")):
+        prefix = f"layers.{index}"
+        names = {f"{role}_proj.{kind}": f"{prefix}.attn.{role}.{kind}" for role in ("q", "k", "v") for kind in ("weight", "bias")}
+        names["o_proj.weight"] = f"{prefix}.attn.o.weight"
+        position = PartSpec("rope_split_half", {"theta": THETA, "head_dim": HEAD_DIM})
+        mixer = PartSpec("paged_attention", {"hidden_size": HIDDEN, "num_heads": HEADS, "num_kv_heads": KV_HEADS, "head_dim": HEAD_DIM,
+                                             "qkv_bias": True, "window": None, "position": position}, names)
+        ffn = PartSpec("swiglu", {"hidden_size": HIDDEN, "intermediate_size": INTER},
+                       {f"{r}_proj.weight": f"{prefix}.ffn.{r}" for r in ("gate", "up", "down")})
+        layers.append(LayerSpec(arrangement, PartSpec("rms_norm", {"size": HIDDEN, "eps": EPS}, {"weight": f"{prefix}.norm1"}),
+                                mixer, PartSpec("rms_norm", {"size": HIDDEN, "eps": EPS}, {"weight": f"{prefix}.norm2"}), ffn))
+    sizes = {"vocab_size": VOCAB, "hidden_size": HIDDEN}
+    spec = ModelSpec("ToyArrangement", VOCAB, HIDDEN, 512, PartSpec("token_embedding", sizes, {"weight": "embed"}), tuple(layers),
+                     tuple(RunEntry(index) for index in range(3)), PartSpec("rms_norm", {"size": HIDDEN, "eps": EPS}, {"weight": "norm"}),
+                     PartSpec("lm_head", sizes, {"weight": "head"}))
+    tensors = toy_tensors(spec)
+    engine = Engine(spec, tensors, dtype=dtype, max_tokens=512)
+    tokens = np.random.default_rng(4).integers(0, VOCAB, size=70).tolist()
+
+    w = {name: value.double().numpy() for name, value in tensors.items()}
+    h = plain.embedding(w["embed"], tokens)
+    count, positions = len(tokens), np.arange(len(tokens))
+    for index, arrangement in enumerate(("toy_parallel", "pre_norm", "toy_parallel")):
+        p = f"layers.{index}"
+
+        def attention(x):
+            q = plain.linear(x, w[f"{p}.attn.q.weight"], w[f"{p}.attn.q.bias"]).reshape(count, HEADS, HEAD_DIM)
+            k = plain.linear(x, w[f"{p}.attn.k.weight"], w[f"{p}.attn.k.bias"]).reshape(count, KV_HEADS, HEAD_DIM)
+            v = plain.linear(x, w[f"{p}.attn.v.weight"], w[f"{p}.attn.v.bias"]).reshape(count, KV_HEADS, HEAD_DIM)
+            q, k = plain.rope_split_half(q, positions, THETA), plain.rope_split_half(k, positions, THETA)
+            o = plain.causal_gqa_attention(q, k, v, 1.0 / math.sqrt(HEAD_DIM), None).reshape(count, HEADS * HEAD_DIM)
+            return plain.linear(o, w[f"{p}.attn.o.weight"])
+
+        def feed_forward(x):
+            return plain.swiglu_ffn(x, w[f"{p}.ffn.gate"], w[f"{p}.ffn.up"], w[f"{p}.ffn.down"])
+
+        x = plain.rms_norm(h, w[f"{p}.norm1"], EPS)
+        if arrangement == "toy_parallel":
+            h = h + attention(x) + feed_forward(x)
+        else:
+            h = h + attention(x)
+            h = h + feed_forward(plain.rms_norm(h, w[f"{p}.norm2"], EPS))
+    expected = plain.rms_norm(h, w["norm"], EPS) @ w["head"].T
+    tolerance = 2e-5 if dtype == "float32" else 4e-2
+
+    engine.open("whole")
+    whole = engine.step([StepEntry("whole", tokens, list(range(count)))]).double().cpu().numpy()
+    engine.close("whole")
+    assert np.abs(whole - expected).max() <= tolerance * np.abs(expected).max()
+    # in portions and then token by token (few rows: the package's blocks fuse sums and norms around the toy block)
+    engine.open("cut")
+    rows, position = [], 0
+    for size in (33, 2, 20):
+        rows.append(engine.step([StepEntry("cut", tokens[position:position + size], list(range(size)))]).double().cpu().numpy())
+        position += size
+    for token in tokens[position:]:
+        rows.append(engine.step([StepEntry("cut", [token], [0])]).double().cpu().numpy())
+    assert np.abs(np.concatenate(rows) - expected).max() <= tolerance * np.abs(expected).max()
+    engine.cache.check()
