@@ -6,6 +6,12 @@ standard output. Options the reference has keep their names and meanings; what t
     microllm_hf_infer --config DIR/config.json --weights DIR/model.safetensors --tokens 1,2,3 \\
                       --device hip --new-tokens 16
 
+``--use-cache false`` generates by running every sequence whole for each new token (the reference's oracle for
+its cached path), ``--cache-prefill-mode token`` feeds the prompt one token a step, ``--prefill-logits full`` computes
+the logits of every prompt position, ``--batch-argmax-mode host`` picks tokens from logits copied to the host,
+``--cache-logits-output`` writes the last decode step's logits, and ``--bf16-ffn`` with ``--bf16-attention``
+choose the precision as ``--dtype`` does (apps/hf_infer.cpp:52-57, 1121-1123, 1238-1305).
+
 Workloads (``--workload``): ``prefill`` times the prompt alone, ``decode`` times steady decoding after it,
 ``both`` (default) generates ``--new-tokens`` tokens after the prompt, ``continuous`` serves several requests
 whose prompts are cyclic slices of the given token ids (apps/hf_infer.cpp:845-861), arriving at given steps.
@@ -25,6 +31,8 @@ OPTIONS: Dict[str, object] = {
     "batch": 1, "decode-mode": "generation", "kv-cache-dtype": None, "cache-capacity": 0,
     "continuous-slots": 0, "continuous-prompt-lengths": "", "continuous-new-token-lengths": "",
     "continuous-prompt-offsets": "", "continuous-arrival-steps": "",
+    "use-cache": "true", "cache-prefill-mode": "full", "prefill-logits": "last", "batch-argmax-mode": "device",
+    "cache-logits-output": None, "bf16-ffn": None, "bf16-attention": None,
     # this engine's own
     "model": None, "dtype": "bfloat16", "temperature": 0.0, "sample-top-k": 0, "seed": 1, "stop-tokens": "",
     "block-size": 16, "num-blocks": 0, "max-batched-tokens": 2048, "prefill-chunk": 512, "max-requests": 64,
@@ -106,6 +114,23 @@ def run(options: Dict[str, object]) -> int:
     if model_dir is None and options["random-config"] is None:
         raise UsageError("give --model DIR, --config and --weights, or --random-config FILE")
     dtype = str(options["dtype"])
+    # The reference keeps its weights in 32-bit unless --bf16-ffn and --bf16-attention say otherwise
+    # (apps/hf_infer.cpp:52-53); this engine has one precision for all: both switches together choose it.
+    switches = {name: boolean(str(options[name]), f"--{name}") for name in ("bf16-ffn", "bf16-attention") if options[name] is not None}
+    if switches:
+        if len(switches) != 2 or len(set(switches.values())) != 1:
+            raise UsageError("this engine has one precision: give --bf16-ffn and --bf16-attention the same value, or use --dtype")
+        dtype = "bfloat16" if switches["bf16-ffn"] else "float32"
+    use_cache = boolean(str(options["use-cache"]), "--use-cache")
+    for name, allowed in (("cache-prefill-mode", ("full", "token")), ("prefill-logits", ("last", "full")),
+                          ("batch-argmax-mode", ("device", "host"))):
+        if options[name] not in allowed:
+            raise UsageError(f"--{name} must be {' or '.join(allowed)}")      # apps/hf_infer.cpp:194-202
+    if options["workload"] == "continuous" and not use_cache:
+        raise UsageError("the continuous workload needs --use-cache true")      # apps/hf_infer.cpp:241
+    if options["cache-logits-output"] and (not use_cache or options["workload"] == "prefill" or int(options["new-tokens"]) < 2):
+        raise UsageError("--cache-logits-output needs --use-cache true, a workload with decoding and "
+                         "--new-tokens of at least 2")                          # apps/hf_infer.cpp:280-284
     if options["kv-cache-dtype"] is not None and options["kv-cache-dtype"] not in ("fp32", "bf16"):
         raise UsageError("--kv-cache-dtype must be fp32 or bf16")
     if dtype in ("fp32",):
@@ -231,7 +256,13 @@ def run(options: Dict[str, object]) -> int:
                 engine.open(request_id)
             torch.cuda.synchronize()
             begun = time.perf_counter()
-            logits = engine.step([StepEntry(request_id, prompt, [len(prompt) - 1]) for request_id, prompt in zip(ids, prompts)])
+            # --prefill-logits full: the logits of every position are computed, last: of the last alone; the
+            # report and --logits-output take the last row either way (apps/hf_infer.cpp:1121-1123, 1166-1181)
+            every = options["prefill-logits"] == "full"
+            logits = engine.step([StepEntry(request_id, prompt, list(range(len(prompt))) if every else [len(prompt) - 1])
+                                  for request_id, prompt in zip(ids, prompts)])
+            if every:
+                logits = logits.view(batch, len(tokens), -1)[:, -1]
             torch.cuda.synchronize()
             if iteration >= int(options["prefill-warmup"]):
                 timings.append(time.perf_counter() - begun)
@@ -250,15 +281,92 @@ def run(options: Dict[str, object]) -> int:
         report["decode_tokens_per_second"] = round(steady["tokens_per_second"], 3)
         report["decode_ms_per_step"] = round(steady["ms_per_step"], 4)
     if options["workload"] == "both" and new_tokens > 0:
-        torch.cuda.synchronize()
-        begun = time.perf_counter()
-        outputs = generate(engine, prompts, params, max_batched_tokens=int(options["max-batched-tokens"]),
-                           prefill_chunk=int(options["prefill-chunk"]))
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - begun
+        from ..ops import kernels
+        on_host = options["batch-argmax-mode"] == "host"
+
+        def engine_argmax(logits):
+            chosen = kernels.argmax(logits).tolist()
+            if min(chosen) < 0:
+                raise RuntimeError("a row of the logits is not finite")
+            return chosen
+
+        def first_maximum(logits):
+            """Greedy choice per row, on the device or (--batch-argmax-mode host) from the rows copied out."""
+            if not on_host:
+                return engine_argmax(logits)
+            rows = logits.cpu().numpy()
+            if not np.isfinite(rows).all():
+                raise RuntimeError("a row of the logits is not finite")
+            return [int(np.argmax(row)) for row in rows]
+
+        def without_cache():
+            """Every new token runs its whole sequence again through an empty cache: the reference's
+            generate_uncached (apps/hf_infer.cpp:1262-1283), an oracle for the cached path."""
+            sequences = [list(prompt) for prompt in prompts]
+            for produced in range(new_tokens):
+                ids = [("uncached", produced, row) for row in range(batch)]
+                for request_id in ids:
+                    engine.open(request_id)
+                logits = engine.step([StepEntry(request_id, sequence, [len(sequence) - 1]) for request_id, sequence in zip(ids, sequences)])
+                for request_id in ids:
+                    engine.close(request_id)
+                for sequence, token in zip(sequences, first_maximum(logits)):
+                    sequence.append(token)
+            return sequences, None
+
+        def with_cache_step_by_step():
+            """The prompt whole or token by token (--cache-prefill-mode), then one token a step for all rows; keeps
+            the last step's logits for --cache-logits-output (apps/hf_infer.cpp:1238-1260)."""
+            ids = [("cached", row) for row in range(batch)]
+            for request_id in ids:
+                engine.open(request_id)
+            sequences = [list(prompt) for prompt in prompts]
+            portion = len(tokens) if options["cache-prefill-mode"] == "full" else 1
+            logits = None
+            for start in range(0, len(tokens), portion):
+                last = start + portion >= len(tokens)
+                logits = engine.step([StepEntry(request_id, prompt[start:start + portion], [min(portion, len(prompt) - start) - 1] if last else [])
+                                      for request_id, prompt in zip(ids, prompts)])
+            for produced in range(new_tokens):
+                chosen = first_maximum(logits)
+                for sequence, token in zip(sequences, chosen):
+                    sequence.append(token)
+                if produced + 1 < new_tokens:
+                    logits = engine.step([StepEntry(request_id, [token], [0]) for request_id, token in zip(ids, chosen)])
+            for request_id in ids:
+                engine.close(request_id)
+            return sequences, logits
+
+        greedy = params.temperature == 0.0 or params.top_k == 1
+        explicit = not use_cache or options["cache-prefill-mode"] == "token" or options["cache-logits-output"] or on_host
+        if explicit and not greedy:
+            raise UsageError("--use-cache false, --cache-prefill-mode token, --batch-argmax-mode host and "
+                             "--cache-logits-output are for greedy generation (--temperature 0)")
+        outputs, elapsed = None, 0.0
+        for _ in range(max(1, int(options["steps"])) if options["decode-mode"] == "generation" else 1):
+            torch.cuda.synchronize()
+            begun = time.perf_counter()
+            if not use_cache:
+                current, last_logits = without_cache()
+            elif explicit:
+                current, last_logits = with_cache_step_by_step()
+            else:
+                current, last_logits = generate(engine, prompts, params, max_batched_tokens=int(options["max-batched-tokens"]),
+                                                prefill_chunk=int(options["prefill-chunk"])), None
+            torch.cuda.synchronize()
+            elapsed += time.perf_counter() - begun
+            if outputs is not None and current != outputs:
+                raise RuntimeError("deterministic generation changed across steps")      # apps/hf_infer.cpp:1285-1287
+            outputs = current
+            if options["cache-logits-output"] and last_logits is not None:
+                last_logits.cpu().numpy().astype("<f4").tofile(str(options["cache-logits-output"]))   # apps/hf_infer.cpp:1297-1305
+        runs = max(1, int(options["steps"])) if options["decode-mode"] == "generation" else 1
         report["generated_tokens"] = outputs[0][len(tokens):]
         report["generation_ms"] = round(elapsed * 1e3, 3)
-        report["generation_tokens_per_second"] = round(sum(len(o) - len(tokens) for o in outputs) / elapsed, 3)
+        report["generation_tokens_per_second"] = round(runs * sum(len(o) - len(tokens) for o in outputs) / elapsed, 3)
+        report.update({"use_cache": use_cache, "cache_prefill_mode": options["cache-prefill-mode"],
+                       "batch_argmax_mode": options["batch-argmax-mode"]})
+    report["prefill_logits_mode"] = options["prefill-logits"]
     report["prompt_tokens"] = len(tokens)
     print(json.dumps(report), flush=True)
     return 0

@@ -186,6 +186,41 @@ def test_command_line(tmp_path):
         assert generated == plain.generate_greedy(model.config, model.weights, cyclic, new)
 
 
+def test_command_line_ways_of_generating(tmp_path, capsys):
+    """The reference's switches for how tokens are generated: without the cache, the prompt token by token, argmax on
+    the host, every prompt position's logits, the weights' precision by --bf16-ffn and --bf16-attention. All give
+    the plain implementation's tokens; the cached run's last logits are those of the last generated position."""
+    from microllm_rocm_amd.cli import hf_infer
+    folder = make_folder(tmp_path, "A", SHARP)
+    model = PlainModel(folder)
+    prompt = random_tokens(5, 11, CONFIGS["A"].vocab_size)
+    expected = plain.generate_greedy(model.config, model.weights, prompt, 5)
+    base = ["--model", folder, "--tokens", ",".join(map(str, prompt)), "--new-tokens", "5", "--batch", "2"]
+    cache_logits = tmp_path / "cache.f32"
+
+    def run(*more):
+        capsys.readouterr()
+        assert hf_infer.main(base + list(more)) == 0
+        return json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+
+    for more in (["--bf16-ffn", "false", "--bf16-attention", "false", "--use-cache", "false"],
+                 ["--dtype", "float32", "--use-cache", "false", "--batch-argmax-mode", "host"],
+                 ["--dtype", "float32", "--cache-prefill-mode", "token", "--cache-logits-output", str(cache_logits), "--steps", "2"],
+                 ["--dtype", "float32", "--prefill-logits", "full", "--batch-argmax-mode", "host"]):
+        report = run(*more)
+        assert report["compute_dtype"] == "float32" and report["generated_tokens"] == expected, more
+    # the logits that chose the last token: position prompt + 4 of the sequence, for both rows of the batch
+    written = np.fromfile(cache_logits, dtype="<f4").reshape(2, -1)
+    reference = model.logits(prompt + expected[:4])[-1]
+    assert np.abs(written - reference[None, :]).max() <= 2e-5 * np.abs(reference).max()
+    assert run("--bf16-ffn", "true", "--bf16-attention", "true")["compute_dtype"] == "bfloat16"
+    for bad in (["--bf16-ffn", "true", "--bf16-attention", "false"], ["--bf16-ffn", "true"], ["--prefill-logits", "some"],
+                ["--use-cache", "false", "--cache-logits-output", str(cache_logits)],
+                ["--use-cache", "false", "--temperature", "0.7"]):
+        assert hf_infer.main(base + bad) == 2, bad
+        assert "microllm_hf_infer:" in capsys.readouterr().err
+
+
 def test_step_refuses_bad_batches_and_leaves_the_cache_as_it_was(tmp_path):
     from microllm_rocm_amd import StepEntry
     from microllm_rocm_amd.cache import OutOfPages
