@@ -337,10 +337,12 @@ template <int MT, int NT, int EPILOGUE>
 static void launch_one(const bf16* a, const bf16* w, void* out, int m, int n, int k, int n_tiles,
                        int k_steps, const MllSkinnyExtras& extras, hipStream_t stream) {
     const int groups = (n_tiles + NT - 1) / NT;
-    // Waves per workgroup: enough that about eight thousand waves would stream W one tile each, at most 16, and
-    // no more than there are chunks of k for them. A function of (n, k) alone, like the split of k it implies.
+    // Waves per workgroup: enough that about sixteen thousand waves would stream W one tile each (timed inside the
+    // decode step of 7B sizes: 1 % faster than eight thousand at 8 and 16 rows, the same at one; thirty-two thousand
+    // lose at one row), at most 16, and no more than there are chunks of k for them. A function of (n, k) alone,
+    // like the split of k it implies.
     int waves = 1;
-    while (waves < 16 && n_tiles * waves * 2 <= 8192 && waves * 2 * kChunk <= k_steps) waves *= 2;
+    while (waves < 16 && n_tiles * waves * 2 <= 16384 && waves * 2 * kChunk <= k_steps) waves *= 2;
     size_t lds = waves > 1 ? static_cast<size_t>(waves - 1) * NT * MT * kWave * sizeof(floatx4) : 0;
     const bool temporal = static_cast<int64_t>(n_tiles) * k_steps * 1024 < (64ll << 20);   // bytes of the packed weight
     const bool scaled = extras.scale.sumsq != nullptr;
