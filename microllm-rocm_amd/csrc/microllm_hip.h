@@ -161,6 +161,18 @@ int mll_measure_mfma(int iterations, void* sink, int blocks, hipStream_t stream)
 int mll_argmax(const float* logits, int32_t* out, void* parts, int n_rows, int vocab, hipStream_t stream);
 int mll_argmax_slices(int vocab);
 
+// mll_argmax for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+// harnesses that forbid hipMalloc). It has no counterpart in the reference. The slices' scratch is a static
+// array in device memory of MLL_ARGMAX_STATIC_MAX_PARTS * 16 bytes (1 MiB), one per GPU, held until the process
+// ends; the call allocates and frees nothing. It refuses n_rows * mll_argmax_slices(vocab) beyond
+// MLL_ARGMAX_STATIC_MAX_PARTS (at 64 slices, vocabularies from 129 025 tokens on: 1024 rows). The GPU whose
+// scratch is used is the current one, which must be the stream's; the first call on a GPU looks the array's
+// address up (make that call outside a graph capture). All calls on one GPU share the array: calls that overlap
+// on one GPU (two streams, two threads) race; calls on one stream do not. The array keeps the last call's
+// contents and needs no clearing: each call writes every entry it reads.
+#define MLL_ARGMAX_STATIC_MAX_PARTS 65536
+int mll_argmax_static(const float* logits, int32_t* out, int n_rows, int vocab, hipStream_t stream);
+
 // Draws one token per row from softmax(logits / temperature) restricted to the top_k largest
 // logits (top_k <= 0: all; ties at the k-th value go to the lower token ids), by inverse CDF in
 // token order with the given uniform in [0, 1). temperature == 0 or top_k == 1 gives the

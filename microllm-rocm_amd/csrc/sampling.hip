@@ -3,6 +3,8 @@
 #include "common.h"
 #include "microllm_hip.h"
 
+#include <mutex>
+
 namespace mll {
 
 // Monotone map from float to unsigned: a larger float gives a larger key.
@@ -524,6 +526,54 @@ extern "C" int mll_argmax(const float* logits, int32_t* out, void* parts, int n_
     argmax_slices_kernel<<<dim3(n_rows, slices), kArgmaxThreads, 0, stream>>>(logits, static_cast<ArgmaxPart*>(parts), vocab, slice);
     argmax_pick_kernel<<<n_rows, kWave, 0, stream>>>(static_cast<const ArgmaxPart*>(parts), out, slices);
     return check_launch("argmax");
+}
+
+// The scratch of mll_argmax_static: the slices' results of its last call. One copy per GPU, held until the
+// process ends. In host code this name is a stand-in for the symbol, not a device address: the address on a GPU
+// comes from hipGetSymbolAddress with that GPU current, and only that address is handed to kernels.
+static __device__ __align__(256) unsigned char argmax_static_scratch[MLL_ARGMAX_STATIC_MAX_PARTS * sizeof(mll::ArgmaxPart)];
+
+namespace {
+
+constexpr int kStaticMaxDevices = 64;
+std::mutex static_scratch_mutex;
+void* static_scratch_of_device[kStaticMaxDevices] = {};
+
+// The address of argmax_static_scratch on the current GPU, asked for once per GPU; null after fail().
+void* argmax_static_scratch_here() {
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kStaticMaxDevices) {
+        fail("argmax_static: no current GPU, or its index is beyond 63");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> guard(static_scratch_mutex);
+    if (static_scratch_of_device[device] == nullptr) {
+        void* address = nullptr;
+        const hipError_t status = hipGetSymbolAddress(&address, HIP_SYMBOL(argmax_static_scratch));
+        if (status != hipSuccess || address == nullptr) {
+            fail(std::string("argmax_static: hipGetSymbolAddress: ") + hipGetErrorString(status));
+            return nullptr;
+        }
+        static_scratch_of_device[device] = address;
+    }
+    return static_scratch_of_device[device];
+}
+
+}  // namespace
+
+extern "C" int mll_argmax_static(const float* logits, int32_t* out, int n_rows, int vocab, hipStream_t stream) {
+    MLL_REQUIRE(n_rows >= 0 && vocab > 0, "argmax_static: sizes must be positive");
+    MLL_REQUIRE(logits != nullptr && out != nullptr, "argmax_static: logits and out are required");
+    const int64_t parts_needed = static_cast<int64_t>(n_rows) * mll_argmax_slices(vocab);
+    MLL_REQUIRE(n_rows <= 65535 && parts_needed <= MLL_ARGMAX_STATIC_MAX_PARTS,
+                "argmax_static: rows x slices is " + std::to_string(parts_needed) + ", beyond the static scratch of " +
+                    std::to_string(MLL_ARGMAX_STATIC_MAX_PARTS) + " (use mll_argmax with a scratch of the caller's)");
+    if (n_rows == 0) return 0;
+    void* parts = argmax_static_scratch_here();
+    if (parts == nullptr) return 1;
+    // Every slice of every row of this call is written by the first kernel before the second reads it: nothing
+    // of an earlier call's contents is read, so nothing has to be cleared.
+    return mll_argmax(logits, out, parts, n_rows, vocab, stream);
 }
 
 extern "C" int64_t mll_sample_workspace(int n_rows, int vocab) {
