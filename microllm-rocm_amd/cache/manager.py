@@ -52,6 +52,7 @@ class RequestCache:
     reserved: int = 0                        # positions beyond num_tokens that already have pages
     pages: List[List[int]] = field(default_factory=list)  # per group: page of every block, RELEASED if given back
     closed: bool = False
+    broken: bool = False                     # its state may hold part of a step that failed: only closing is left
 
 
 class CacheGroup:
@@ -131,6 +132,12 @@ class CacheManager:
                 self._bindings[entry] = StateBinding(binding.need, binding.state, owned=False)
 
     # ---- what the model sees -------------------------------------------------------------
+    @property
+    def has_state(self) -> bool:
+        """Whether any run entry keeps per-request state of fixed size (which, unlike pages, a failed step cannot
+        simply leave behind)."""
+        return any(isinstance(binding, StateBinding) and binding.owned for binding in self._bindings)
+
     def bindings(self) -> List[object]:
         return list(self._bindings)
 

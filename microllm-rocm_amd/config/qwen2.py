@@ -126,6 +126,12 @@ class Qwen2Config:
             for kind in self.layer_types:
                 if kind not in (FULL_ATTENTION, SLIDING_ATTENTION):
                     raise ConfigError(f"unknown layer type {kind!r}")
+            if SLIDING_ATTENTION in self.layer_types and not self.use_sliding_window:
+                # The two keys contradict each other, and implementations differ in which one wins (one that
+                # drops sliding_window when use_sliding_window is false attends to every key in every layer):
+                # refused rather than guessed.
+                raise ConfigError("layer_types names sliding_attention layers but use_sliding_window is false; "
+                                  "set use_sliding_window to true or make every layer full_attention")
         windowed = any(window is not None for window in self.layer_windows())
         if windowed or self.use_sliding_window:
             if self.sliding_window is None or self.sliding_window <= 0:
@@ -138,14 +144,14 @@ class Qwen2Config:
     def layer_windows(self) -> Tuple[Optional[int], ...]:
         """The window of every layer, ``None`` for a layer that sees all keys.
 
-        ``layer_types`` decides where it is given; otherwise layers with index
-        ``>= max_window_layers`` use the window when ``use_sliding_window`` is true.
+        Without ``use_sliding_window`` no layer has one. With it, ``layer_types`` decides where it is given if
+        present; otherwise layers with index ``>= max_window_layers`` use it.
         """
+        if not self.use_sliding_window:
+            return tuple(None for _ in range(self.num_hidden_layers))
         if self.layer_types is not None:
             return tuple(self.sliding_window if kind == SLIDING_ATTENTION else None
                          for kind in self.layer_types)
-        if not self.use_sliding_window:
-            return tuple(None for _ in range(self.num_hidden_layers))
         first = self.max_window_layers if self.max_window_layers is not None else self.num_hidden_layers
         return tuple(self.sliding_window if index >= first else None
                      for index in range(self.num_hidden_layers))

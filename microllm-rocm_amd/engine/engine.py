@@ -221,6 +221,9 @@ class Engine:
                 raise ValueError(f"request {entry.request_id!r} appears twice in one step")
             seen.add(entry.request_id)
             request = self.cache.get(entry.request_id)
+            if request.broken:
+                raise ValueError(f"request {entry.request_id!r} was in a step that failed after its state may have "
+                                 "changed; close it and run it again from its first token")
             count = len(entry.tokens)
             if count == 0:
                 raise ValueError(f"request {entry.request_id!r} brings no tokens")
@@ -247,18 +250,40 @@ class Engine:
                 for request in taken:
                     self.cache.cancel_reservation(request)
                 raise
-        if self.use_graphs and len(entries) <= MAX_GRAPH_REQUESTS and all(len(entry.tokens) == 1 for entry in entries):
-            logits = self._graph_step(requests, entries)
-        else:
-            self._last_graph = None
-            ctx = self._builder.build(requests, [entry.tokens for entry in entries], [entry.want for entry in entries])
-            logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
+        try:
+            if self.use_graphs and len(entries) <= MAX_GRAPH_REQUESTS and all(len(entry.tokens) == 1 for entry in entries):
+                logits = self._graph_step(requests, entries)
+            else:
+                self._last_graph = None
+                ctx = self._builder.build(requests, [entry.tokens for entry in entries], [entry.want for entry in entries])
+                logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
+        except BaseException:
+            self._roll_back(requests)
+            raise
         for request, entry in zip(requests, entries):
             self.cache.commit(request, len(entry.tokens))
         self.steps_run += 1
         if self._last_graph is not None:
             self._build_ahead(self._last_graph, requests)
         return logits
+
+    def _roll_back(self, requests: List[RequestCache]) -> None:
+        """A step failed inside the model (a kernel refused its arguments, a part raised): nothing of it counts.
+
+        Every request of the step gives back the pages that only this step needed, whoever reserved them, and
+        keeps the positions it had; keys and values that the step wrote beyond them are never read, since
+        lengths, not contents, say what is valid. Per-request state has no such rule: a part may have changed it
+        before the failure, so with state in the model the step's requests are marked broken and refused from
+        then on; whoever runs them closes them and runs them again from their first token (the scheduler does).
+        The reference resets the cache on any failure of a forward (src/model/model.cpp:1131-1134)."""
+        self._ahead = None
+        self._last_graph = None
+        for request in requests:
+            if request.closed:
+                continue
+            self.cache.cancel_reservation(request)
+            if self.cache.has_state:
+                request.broken = True
 
     def _build_ahead(self, state: _DecodeGraph, requests: List[RequestCache]) -> None:
         """After a decode step from a graph: the next one's metadata (positions, slots, block tables), while the

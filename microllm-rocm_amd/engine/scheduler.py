@@ -90,6 +90,7 @@ class SchedulerMetrics:
     engine_steps: int = 0
     peak_active_requests: int = 0
     peak_held_pages: int = 0
+    failed_steps: int = 0
 
 
 @dataclass(eq=False)
@@ -177,6 +178,7 @@ class Scheduler:
         """Decide what this step runs. Takes pages (a reservation per portion); may preempt."""
         budget = self.max_batched_tokens
         portions: List[Portion] = []
+        preempted_now = False
 
         def portion_of(request: Request, budget_left: int) -> int:
             remaining = request.known - request.computed
@@ -201,6 +203,7 @@ class Scheduler:
                         portions.remove(planned)
                         budget += planned.count
                     self._preempt(victim)
+                    preempted_now = True
                     if victim is request:
                         count = 0
                         break
@@ -208,12 +211,17 @@ class Scheduler:
                 portions.append(Portion(request, request.computed, count, request.computed + count == request.known))
                 budget -= count
 
-        # Then admissions, first come first served; a request that does not fit stops the queue.
-        while self.waiting and budget > 0 and len(self.running) < self.max_requests:
+        # Then admissions, first come first served; a request that does not fit stops the queue. None in a step
+        # that had to preempt: the victim is first in the queue, and a small portion of it would fit the pages it
+        # has just given back, only for the next page an older request needs to throw it out again, its prompt
+        # recomputed from the first token each time. It waits for a step in which the running ones find room.
+        while self.waiting and budget > 0 and len(self.running) < self.max_requests and not preempted_now:
             request = self.waiting[0]
             if request.arrival_step > self.current_step:
                 break
             count = portion_of(request, budget)
+            if request.preemptions > 0 and not self._room_for_all_of(request):
+                break
             handle = self.cache.open(request.id)
             try:
                 self.cache.reserve(handle, count)
@@ -230,6 +238,15 @@ class Scheduler:
             budget -= count
         return portions
 
+    def _room_for_all_of(self, request: Request) -> bool:
+        """Whether the free pages hold everything the request has to run again and its next token. A request that
+        was preempted comes back only then: admitted into less, it would recompute a part of its prompt and be
+        thrown out again by the next page an older request needs."""
+        if not self.running:
+            return True      # alone it fits: submit saw to that
+        blocks = self.cache.blocks_for(request.known + 1)
+        return all(blocks <= group.pool.num_free for group in self.cache.groups)
+
     def step(self) -> List[int]:
         """Run one batch; returns the ids of requests that got a token in this step."""
         portions = self.plan()
@@ -244,12 +261,17 @@ class Scheduler:
                 request = portion.request
                 tokens = [request.token_at(index) for index in range(portion.start, portion.start + portion.count)]
                 entries.append(StepEntry(request.id, tokens, [portion.count - 1] if portion.wants_logits else []))
-                if portion.count == 1 and request.state == RequestState.DECODING:
+            try:
+                logits = self.engine.step(entries, reserved=True)
+            except Exception:
+                self._step_failed(portions)
+                raise
+            for portion in portions:
+                if portion.count == 1 and portion.request.state == RequestState.DECODING:
                     self.metrics.decode_tokens += 1
                 else:
                     self.metrics.prefill_tokens += portion.count
                 self.metrics.batched_tokens += portion.count
-            logits = self.engine.step(entries, reserved=True)
             self.metrics.engine_steps += 1
             for portion in portions:
                 portion.request.computed += portion.count
@@ -285,14 +307,31 @@ class Scheduler:
         if self.cache.requests.get(request.id) is not None:
             self.cache.close(request.id)
 
-    def _preempt(self, request: Request) -> None:
+    def _step_failed(self, portions: List[Portion]) -> None:
+        """The engine raised inside a step: nothing of the step counts. The engine has given back the pages the
+        step took; the requests keep the positions they had and go on from there in the next step. Where the
+        model keeps per-request state, which the failed step may have changed, every request of the step starts
+        again from its first token instead, as after a preemption (the engine refuses to go on with them). The
+        reference resets the rows of a failed prefill (src/inference/scheduler.cpp:763-766)."""
+        self.metrics.failed_steps += 1
+        if getattr(self.cache, "has_state", False):
+            for portion in reversed(portions):
+                if portion.request in self.running:
+                    self._preempt(portion.request, failed=True)
+        for portion in portions:      # reservations that the engine did not see (it raised before it came to them)
+            handle = self.cache.requests.get(portion.request.id)
+            if handle is not None and handle.reserved:
+                self.cache.cancel_reservation(handle)
+
+    def _preempt(self, request: Request, failed: bool = False) -> None:
         self.running.remove(request)
         self._release(request)
         request.computed = 0
         request.admitted = False
-        request.preemptions += 1
         request.state = RequestState.PENDING_PREFILL
-        self.metrics.preemptions += 1
+        if not failed:
+            request.preemptions += 1
+            self.metrics.preemptions += 1
         self.waiting.appendleft(request)
 
     def _complete(self, request: Request, reason: CompletionReason) -> None:

@@ -150,10 +150,12 @@ def head_dim_of(config: dict) -> int:
 def layer_windows(config: dict) -> List[Optional[int]]:
     """Layers with index >= max_window_layers use the window when use_sliding_window is true."""
     layers = config["num_hidden_layers"]
+    if not config.get("use_sliding_window", False):
+        if "sliding_attention" in (config.get("layer_types") or []):
+            raise ValueError("layer_types names sliding_attention layers but use_sliding_window is false")
+        return [None] * layers
     if config.get("layer_types"):
         return [config["sliding_window"] if kind == "sliding_attention" else None for kind in config["layer_types"]]
-    if not config.get("use_sliding_window", False):
-        return [None] * layers
     return [config["sliding_window"] if index >= config["max_window_layers"] else None for index in range(layers)]
 
 

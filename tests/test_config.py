@@ -77,11 +77,18 @@ def test_windows_by_layer():
     config = Qwen2Config.from_dict(dict(QWEN25_05B, use_sliding_window=True, sliding_window=100, max_window_layers=20))
     windows = config.layer_windows()
     assert windows[:20] == tuple([None] * 20) and windows[20:] == (100, 100, 100, 100)
-    typed = Qwen2Config.from_dict(dict(QWEN25_05B, num_hidden_layers=3, sliding_window=7,
+    typed = Qwen2Config.from_dict(dict(QWEN25_05B, num_hidden_layers=3, sliding_window=7, use_sliding_window=True,
                                        layer_types=["sliding_attention", "full_attention", "sliding_attention"]))
     assert typed.layer_windows() == (7, None, 7)
     spec = build_spec(typed)
     assert [layer.mixer.params["window"] for layer in spec.layers] == [7, None, 7]
+    # layer_types that ask for a window while use_sliding_window is false contradict: refused, not guessed.
+    with pytest.raises(ConfigError, match="use_sliding_window is false"):
+        Qwen2Config.from_dict(dict(QWEN25_05B, num_hidden_layers=2, sliding_window=7, use_sliding_window=False,
+                                   layer_types=["sliding_attention", "full_attention"]))
+    plain_only_full = Qwen2Config.from_dict(dict(QWEN25_05B, num_hidden_layers=2, sliding_window=7, use_sliding_window=False,
+                                                 layer_types=["full_attention", "full_attention"]))
+    assert plain_only_full.layer_windows() == (None, None)
 
 
 def test_spec_holds_every_size_of_the_configuration():

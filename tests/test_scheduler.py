@@ -183,6 +183,75 @@ def test_running_out_of_pages_preempts_the_latest_and_recomputes():
     assert again
 
 
+def test_a_preempted_request_waits_for_room_instead_of_being_thrown_out_again_and_again():
+    # 8 pages of 4 tokens. The older request grows to 10 + 20 = 30 tokens (8 pages): it needs every page the
+    # younger one holds, one after the other. The younger one is preempted once and comes back when the older has
+    # finished; it is not admitted into the page or two that are free meanwhile, which would cost a recomputation
+    # of its prompt for every page the older one takes.
+    engine = FakeEngine(num_pages=8, page_size=4)
+    s = scheduler(engine, max_batched_tokens=64, prefill_chunk=64)
+    older = s.submit(list(range(10)), SamplingParams(max_new_tokens=20, temperature=0.0))
+    young = SamplingParams(max_new_tokens=16, temperature=0.7, seed=1)
+    younger = s.submit(list(range(20, 26)), young)
+    s.run_until_idle(maximum_steps=200)
+    assert s.request(older).preemptions == 0 and s.request(younger).preemptions == 1
+    assert s.metrics.preemptions == 1
+    assert s.request(younger).generated == alone(range(20, 26), young)
+    assert s.request(older).generated == alone(range(10), SamplingParams(max_new_tokens=20, temperature=0.0))
+    # tokens run through the model: both requests once, and the younger one's prompt and what it had generated again
+    fed_younger = sum(n for batch in engine.batches for r, n in batch if r == younger)
+    assert fed_younger <= 2 * (6 + 16)
+    assert s.metrics.prefill_tokens + s.metrics.decode_tokens == sum(n for batch in engine.batches for _, n in batch)
+    assert engine.cache.free_pages() == [8]
+
+
+class FailingEngine(FakeEngine):
+    """Raises inside the step whose number is given, after the scheduler has reserved its pages."""
+
+    def __init__(self, fail_at, state=False, **options):
+        super().__init__(**options)
+        self.fail_at = fail_at
+        self.calls = 0
+        if state:
+            from microllm_rocm_amd.parts import StateNeed
+            self.cache = CacheManager([PagedKVNeed(1, 8, None), StateNeed((2,))], [None, None], 4, 16, 4, device=None)
+
+    def step(self, entries, reserved=False):
+        self.calls += 1
+        if self.calls == self.fail_at:
+            # what Engine.step does when the model raises: the step's reservations are given back
+            for entry in entries:
+                self.cache.cancel_reservation(self.cache.get(entry.request_id))
+            raise RuntimeError("a kernel refused its arguments")
+        return super().step(entries, reserved)
+
+
+@pytest.mark.parametrize("state", [False, True])
+def test_a_failed_step_counts_for_nothing_and_the_next_one_goes_on(state):
+    engine = FailingEngine(fail_at=3, state=state)
+    s = scheduler(engine, max_batched_tokens=8, prefill_chunk=4)
+    params = SamplingParams(max_new_tokens=4, temperature=0.0)
+    first, second = s.submit(list(range(9)), params), s.submit(list(range(30, 35)), params)
+    s.step()
+    s.step()
+    before = (s.metrics.prefill_tokens, s.metrics.decode_tokens, s.metrics.engine_steps)
+    with pytest.raises(RuntimeError, match="refused"):
+        s.step()
+    assert (s.metrics.prefill_tokens, s.metrics.decode_tokens, s.metrics.engine_steps) == before and s.metrics.failed_steps == 1
+    engine.cache.check()
+    assert all(request.reserved == 0 for request in engine.cache.requests.values())
+    if state:      # per-request state may hold a part of the failed step: every request of it starts again
+        assert not engine.cache.requests and [r.computed for r in s.requests.values()] == [0, 0]
+        assert s.metrics.preemptions == 0
+    else:          # pages hold nothing beyond the positions that count: the requests go on where they were
+        assert sorted(r.computed for r in s.requests.values()) == sorted(
+            engine.cache.get(rid).num_tokens for rid in (first, second))
+    s.run_until_idle(maximum_steps=100)
+    assert s.request(first).generated == alone(range(9), params)
+    assert s.request(second).generated == alone(range(30, 35), params)
+    assert engine.cache.free_pages() == [16] and engine.cache.slots.num_free == 4
+
+
 def test_a_request_alone_always_fits_and_idle_limit_is_an_error():
     engine = FakeEngine(num_pages=4, page_size=4)
     s = scheduler(engine, max_batched_tokens=5, prefill_chunk=5)
