@@ -332,7 +332,7 @@ def run(options: Dict[str, object]) -> int:
                 for sequence, token in zip(sequences, chosen):
                     sequence.append(token)
                 if produced + 1 < new_tokens:
-                    logits = engine.step([StepEntry(request_id, [token], [0]) for request_id, token in zip(ids, chosen)])
+                    logits = engine.step([StepEntry(request_id, [token], [0]) for request_id, token in zip(ids, chosen)], borrow_logits=produced + 2 < new_tokens)
             for request_id in ids:
                 engine.close(request_id)
             return sequences, logits

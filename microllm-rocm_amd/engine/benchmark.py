@@ -40,7 +40,7 @@ def decode_throughput(engine: Engine, batch: int, context: int, steps: int, warm
     tokens = rng.integers(0, engine.spec.vocab_size, size=batch).tolist()
 
     def one_step(current):
-        logits = engine.step([StepEntry(request_id, [token], [0]) for request_id, token in zip(ids, current)])
+        logits = engine.step([StepEntry(request_id, [token], [0]) for request_id, token in zip(ids, current)], borrow_logits=True)
         return sampler.select(logits, params, [0] * batch)
 
     try:

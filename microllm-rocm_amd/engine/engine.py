@@ -10,6 +10,7 @@ with its own batch shape (src/model/model.cpp:1091-1135, 1263-1303, 1316-1354,
 from __future__ import annotations
 
 import os
+from collections import OrderedDict
 from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Union
 
 import torch
@@ -37,6 +38,7 @@ def parse_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
 
 MAX_GRAPH_REQUESTS = 256
 MIN_GRAPH_WIDTH = 16
+MAX_GRAPHS = 48     # captured decode steps kept at a time; the one replayed longest ago goes first
 
 
 class _DecodeGraph:
@@ -115,8 +117,14 @@ class Engine:
         # Steps in which every request brings one token are replayed from HIP graphs, one per (number of
         # requests, block-table width): the launches of a decode step cost more host time than GPU time.
         self.use_graphs = use_graphs and all(part.graph_safe for part in self.model.parts())
-        self._graphs: Dict[tuple, "_DecodeGraph"] = {}
+        # All captures share one memory pool: a graph's activations live only while it runs, so the next graph may
+        # have them; what a graph hands out (its logits) stays its own while the graph is kept. At most
+        # MAX_GRAPHS are kept (continuous batching walks through many numbers of requests): each holds its
+        # logits [requests, vocabulary] in float32 and its metadata buffers.
+        self._graphs: "OrderedDict[tuple, _DecodeGraph]" = OrderedDict()
+        self._graph_pool = None
         self.graph_replays = 0
+        self.graphs_captured = 0
 
     def _two_copies_fit(self, model: Model, decls, num_pages: int, page_size: int) -> bool:
         """Whether the weights as stored, their packed copies and the cache pool fit the GPU with a tenth to spare."""
@@ -176,7 +184,11 @@ class Engine:
         key = (n, width)
         state = self._graphs.get(key)
         if state is None:
+            while len(self._graphs) >= MAX_GRAPHS:
+                self._graphs.popitem(last=False)
             state = self._graphs[key] = _DecodeGraph(self, width)
+        else:
+            self._graphs.move_to_end(key)
         every_row = [[0]] * n   # the graph computes the logits of every row; the wanted ones are picked after
         ahead, self._ahead = self._ahead, None
         if ahead is not None and state.graph is not None and ahead.holds_for(state, requests):
@@ -192,25 +204,33 @@ class Engine:
             self.model.forward(ctx, self._bindings, ctx.want_rows)
             torch.cuda.synchronize(self.device)
             ctx.memo.clear()     # what the parts computed once for the step is computed inside the graph too
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
+            with torch.cuda.graph(graph, pool=self._graph_pool):
                 state.logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
             state.graph = graph
+            self.graphs_captured += 1
         state.graph.replay()
         self.graph_replays += 1
         wanted = [index for index, entry in enumerate(entries) if len(entry.want) > 0]
         if not wanted:
             return None
         if len(wanted) == n:
-            return state.logits
+            return state.logits if self._borrow else state.logits.clone()
         return state.logits[torch.tensor(wanted, device=self.device)]
 
     # ---- the step ------------------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry], reserved: bool = False) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], reserved: bool = False, borrow_logits: bool = False) -> Optional[torch.Tensor]:
         """Run one batch; returns float32 logits ``[wanted, vocab]`` in the order of entries and of ``want``.
 
-        With ``reserved`` the caller (a scheduler) has already taken the pages for every portion.
+        With ``reserved`` the caller (a scheduler) has already taken the pages for every portion. The result is the
+        caller's to keep. With ``borrow_logits`` it may be the buffer that a captured decode step writes, which the
+        next step overwrites in place: for callers that select their tokens before they step again (the scheduler,
+        the generation loop, the benchmark) and save the copy. If the model raises, the step counts for nothing:
+        see ``_roll_back``.
         """
+        self._borrow = borrow_logits
         entries = [entry if isinstance(entry, StepEntry) else StepEntry(*entry) for entry in entries]
         if not entries:
             return None

@@ -74,7 +74,7 @@ def generate_serial(engine: Engine, prompt: Sequence[int], params: Optional[Samp
             tokens.append(token)
             if token in params.stop_tokens or generated + 1 == params.max_new_tokens:
                 break
-            logits = engine.step([StepEntry(request_id, [token], [0])])
+            logits = engine.step([StepEntry(request_id, [token], [0])], borrow_logits=True)
     finally:
         engine.close(request_id)
     return tokens

@@ -262,7 +262,7 @@ class Scheduler:
                 tokens = [request.token_at(index) for index in range(portion.start, portion.start + portion.count)]
                 entries.append(StepEntry(request.id, tokens, [portion.count - 1] if portion.wants_logits else []))
             try:
-                logits = self.engine.step(entries, reserved=True)
+                logits = self.engine.step(entries, reserved=True, borrow_logits=True)
             except Exception:
                 self._step_failed(portions)
                 raise

@@ -8,7 +8,6 @@ from __future__ import annotations
 
 import ctypes
 import os
-import tempfile
 from typing import List, NamedTuple, Optional, Sequence, Tuple
 
 import torch
@@ -439,9 +438,7 @@ def set_library_tuning(on: bool, results_file: Optional[str] = None) -> None:
     import torch.cuda.tunable as tunable
     if on:
         if results_file is None:
-            folder = os.path.join(tempfile.gettempdir(), f"microllm_rocm_amd_{os.getuid()}")
-            os.makedirs(folder, exist_ok=True)
-            results_file = os.path.join(folder, "tunableop_results.csv")
+            results_file = os.path.join(library.private_temporary_folder(), "tunableop_results.csv")
         tunable.set_filename(results_file)
         tunable.set_max_tuning_duration(30)
         tunable.set_max_tuning_iterations(10)

@@ -47,11 +47,39 @@ def _source_hash() -> str:
     return digest.hexdigest()
 
 
+_fallback_dir: Optional[str] = None
+
+
+def private_temporary_folder() -> str:
+    """A folder under the temporary directory that only this user can write: what is loaded from it runs inside
+    this process. The folder with the predictable name is taken only if it is a real folder (no link) that this
+    user owns and no one else may write; anyone could have made it beforehand otherwise. Failing that a fresh
+    folder with a random name is made, which later processes do not find again: they build again."""
+    global _fallback_dir
+    if _fallback_dir is not None:
+        return _fallback_dir
+    named = os.path.join(tempfile.gettempdir(), f"microllm_rocm_amd_{os.getuid()}")
+    try:
+        os.mkdir(named, 0o700)
+    except FileExistsError:
+        pass
+    except OSError:
+        named = None
+    if named is not None:
+        try:
+            status = os.lstat(named)
+            import stat
+            if stat.S_ISDIR(status.st_mode) and status.st_uid == os.getuid() and not status.st_mode & 0o022:
+                _fallback_dir = named
+                return named
+        except OSError:
+            pass
+    _fallback_dir = tempfile.mkdtemp(prefix="microllm_rocm_amd_")
+    return _fallback_dir
+
+
 def _candidate_dirs() -> List[str]:
-    dirs = [CSRC]
-    fallback = os.path.join(tempfile.gettempdir(), f"microllm_rocm_amd_{os.getuid()}")
-    dirs.append(fallback)
-    return dirs
+    return [CSRC, private_temporary_folder()]
 
 
 def _find_built() -> Optional[str]:

@@ -30,7 +30,7 @@ class FakeEngine:
         self.fed = {}
         self.batches = []
 
-    def step(self, entries, reserved=False):
+    def step(self, entries, reserved=False, borrow_logits=False):
         assert reserved
         rows = []
         self.batches.append([(entry.request_id, len(entry.tokens)) for entry in entries])
@@ -189,7 +189,7 @@ def test_a_preempted_request_waits_for_room_instead_of_being_thrown_out_again_an
     # finished; it is not admitted into the page or two that are free meanwhile, which would cost a recomputation
     # of its prompt for every page the older one takes.
     engine = FakeEngine(num_pages=8, page_size=4)
-    s = scheduler(engine, max_batched_tokens=64, prefill_chunk=64)
+    s = scheduler(engine, max_batched_tokens=64, prefill_chunk=4)     # portions of one page: one always "fits"
     older = s.submit(list(range(10)), SamplingParams(max_new_tokens=20, temperature=0.0))
     young = SamplingParams(max_new_tokens=16, temperature=0.7, seed=1)
     younger = s.submit(list(range(20, 26)), young)
@@ -216,7 +216,7 @@ class FailingEngine(FakeEngine):
             from microllm_rocm_amd.parts import StateNeed
             self.cache = CacheManager([PagedKVNeed(1, 8, None), StateNeed((2,))], [None, None], 4, 16, 4, device=None)
 
-    def step(self, entries, reserved=False):
+    def step(self, entries, reserved=False, borrow_logits=False):
         self.calls += 1
         if self.calls == self.fail_at:
             # what Engine.step does when the model raises: the step's reservations are given back
