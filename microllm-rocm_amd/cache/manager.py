@@ -75,10 +75,30 @@ class CacheGroup:
         return max(0, oldest_visible) // self.page_size
 
 
+def window_blocks(window: int, portion: int, page_size: int) -> int:
+    """The most blocks a request holds in a group with this window while steps bring it at most ``portion``
+    tokens: the blocks between the oldest key that the portion's first query sees and its last token."""
+    return -(-(window - 1 + portion) // page_size) + 1
+
+
+def pages_of_group(need: PagedKVNeed, num_pages: int, page_size: int, max_requests: int,
+                   max_portion: Optional[int]) -> int:
+    """How many pages a group's pool gets of the ``num_pages`` asked for: all of them, unless the group has a
+    window and the largest portion of a step is known; then no more than every request slot can hold at once."""
+    if need.window is None or max_portion is None:
+        return num_pages
+    return max(1, min(num_pages, max_requests * window_blocks(need.window, max_portion, page_size)))
+
+
 class CacheManager:
     def __init__(self, needs: Sequence[CacheNeed], reads: Sequence[Optional[int]], page_size: int,
                  num_pages: int, max_requests: int, dtype: torch.dtype = torch.float32,
-                 device: Optional[torch.device] = None, max_blocks: Optional[int] = None):
+                 device: Optional[torch.device] = None, max_blocks: Optional[int] = None,
+                 max_portion: Optional[int] = None):
+        """``num_pages``: the pages of a group that keeps every key. A group with a window gets fewer if
+        ``max_portion`` says how many tokens a step brings a request at most (``pages_of_group``): a model of
+        mostly windowed layers then does not pay for the full pool in every group. ``max_blocks``: the most
+        blocks a request's table has (its positions / page size); by default the pool's size."""
         if page_size <= 0:
             raise ValueError("page_size must be positive")
         if device is not None:
@@ -87,7 +107,8 @@ class CacheManager:
             raise ValueError("one need and one read source per run entry")
         self.page_size = page_size
         self.max_requests = max_requests
-        self.max_blocks = min(num_pages, max_blocks) if max_blocks else num_pages   # most blocks one request can hold
+        self.max_blocks = max_blocks if max_blocks else num_pages   # most blocks a request's table has (a window gives early ones back)
+        self.max_portion = max_portion
         self.dtype = dtype
         self.device = device
         self.groups: List[CacheGroup] = []
@@ -102,15 +123,16 @@ class CacheManager:
             if isinstance(need, PagedKVNeed):
                 group = by_need.get(need)
                 if group is None:
-                    group = CacheGroup(len(self.groups), need, num_pages, page_size, max_requests, self.max_blocks)
+                    group = CacheGroup(len(self.groups), need, pages_of_group(need, num_pages, page_size, max_requests, max_portion),
+                                       page_size, max_requests, self.max_blocks)
                     self.groups.append(group)
                     by_need[need] = group
                 group.entries.append(entry)
                 k = v = None
                 if device is not None:
                     # Zeroed once: a kernel may read a whole tile whose tail was never written.
-                    k = torch.zeros(key_page_shape(num_pages, need.kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
-                    v = torch.zeros(value_page_shape(num_pages, need.kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
+                    k = torch.zeros(key_page_shape(group.pool.num_pages, need.kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
+                    v = torch.zeros(value_page_shape(group.pool.num_pages, need.kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
                 self._bindings[entry] = PagedBinding(group.index, need, k, v, owned=True)
             elif isinstance(need, StateNeed):
                 state = None
@@ -160,6 +182,14 @@ class CacheManager:
 
     def blocks_for(self, tokens: int) -> int:
         return (tokens + self.page_size - 1) // self.page_size
+
+    def most_blocks(self, group: CacheGroup, total: int, portion: int) -> int:
+        """The most pages of ``group`` that a request of ``total`` tokens holds at any time when steps bring it
+        at most ``portion`` tokens."""
+        whole = self.blocks_for(total)
+        if group.need.window is None:
+            return whole
+        return min(whole, window_blocks(group.need.window, max(1, min(portion, total)), self.page_size))
 
     def pages_needed(self, request: RequestCache, count: int) -> List[int]:
         """Pages each group would have to take to hold ``count`` more positions."""

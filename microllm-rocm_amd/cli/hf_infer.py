@@ -19,6 +19,7 @@ whose prompts are cyclic slices of the given token ids (apps/hf_infer.cpp:845-86
 from __future__ import annotations
 
 import json
+import math
 import os
 import sys
 import time
@@ -67,6 +68,17 @@ def parse(argv: List[str]) -> Dict[str, object]:
             raise UsageError(f"option {name} needs a number, got {text!r}") from None
         index += 2
     return options
+
+
+def percentile(values, quantile: float) -> float:
+    """Linear interpolation between the two nearest of the sorted values (apps/hf_infer.cpp:570-580)."""
+    if not values or not 0.0 <= quantile <= 1.0:
+        raise ValueError("percentile input is invalid")
+    ordered = sorted(values)
+    position = quantile * (len(ordered) - 1)
+    lower, upper = int(math.floor(position)), int(math.ceil(position))
+    fraction = position - lower
+    return ordered[lower] * (1.0 - fraction) + ordered[upper] * fraction
 
 
 def integers(text: str, what: str) -> List[int]:
@@ -173,7 +185,8 @@ def run(options: Dict[str, object]) -> int:
                           max_requests=max(int(options["max-requests"]), batch),
                           use_graphs=boolean(str(options["use-graphs"]), "--use-graphs"),
                           weight_copies=str(options["weight-copies"]),
-                          tune_library=boolean(str(options["tune-library"]), "--tune-library"))
+                          tune_library=boolean(str(options["tune-library"]), "--tune-library"),
+                          max_portion=int(options["prefill-chunk"]) if continuous else None)
     if model_dir is not None:
         engine = Engine.from_folder(str(model_dir), **engine_options)
     else:
@@ -241,6 +254,11 @@ def run(options: Dict[str, object]) -> int:
             "peak_active_cache_bytes": metrics.peak_held_pages * (engine.cache.allocated_bytes() // max(1, report["kv_blocks"])),
             "request_ttft_ms": [round((r.first_token_time - r.submit_time) * 1e3, 3) for r in requests],
             "request_completion_ms": [round((r.completion_time - r.submit_time) * 1e3, 3) for r in requests],
+            "request_ttft_p50_ms": round(percentile([(r.first_token_time - r.submit_time) * 1e3 for r in requests], 0.50), 3),
+            "request_ttft_p95_ms": round(percentile([(r.first_token_time - r.submit_time) * 1e3 for r in requests], 0.95), 3),
+            "request_completion_p50_ms": round(percentile([(r.completion_time - r.submit_time) * 1e3 for r in requests], 0.50), 3),
+            "request_completion_p95_ms": round(percentile([(r.completion_time - r.submit_time) * 1e3 for r in requests], 0.95), 3),
+            "kv_cache_byte_utilization": round(metrics.peak_held_pages / max(1, report["kv_blocks"]), 4),
             "generated": generated, "token_checksum": int(sum((i + 1) * t for g in generated for i, t in enumerate(g)) % (1 << 31)),
         })
         print(json.dumps(report), flush=True)

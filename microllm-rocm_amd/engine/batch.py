@@ -8,15 +8,13 @@ packs tokens, positions and rows the same way, src/model/model.cpp:1522-1538).
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Hashable, List, Optional, Sequence
+from types import SimpleNamespace
+from typing import Any, Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, RELEASED, RequestCache
-from ..ops import kernels
-
-QUERY_TILE = kernels.QUERY_TILE   # tokens of one request in one tile of the prefill attention kernel
 
 
 @dataclass
@@ -37,6 +35,37 @@ class PagedView:
 
 
 @dataclass
+class HostStep:
+    """A step as the host sees it: what a part that plans its launches from the batch's shape (tiles of queries,
+    work lists) is given. ``cu[i]`` is where request ``i``'s portion starts in the flat token list, ``starts[i]``
+    the position of its first token, ``totals[i]`` the request's length once the step is done."""
+    n_tokens: int
+    n_seqs: int
+    page_size: int
+    counts: List[int]
+    starts: List[int]
+    totals: List[int]
+    cu: np.ndarray
+
+    @property
+    def single_tokens_only(self) -> bool:
+        return self.n_tokens == self.n_seqs
+
+
+class StepPlanner:
+    """What a part gives the engine if its kernels need metadata of their own for a step.
+
+    ``plan(host)`` returns ``(arrays, values)``: int32 numpy arrays that go to the device with the step's other
+    metadata, in the same single copy, and host values (numbers that choose launches). Parts whose planners have
+    equal ``key`` share one plan a step. For a step in which every request brings one token the arrays' sizes may
+    depend on the number of requests alone (such steps are replayed from graphs at fixed addresses)."""
+    key: Hashable = None
+
+    def plan(self, host: HostStep) -> Tuple[Dict[str, np.ndarray], Dict[str, Any]]:
+        raise NotImplementedError
+
+
+@dataclass
 class StepContext:
     n_tokens: int
     n_seqs: int
@@ -48,12 +77,6 @@ class StepContext:
     seq_total: torch.Tensor     # int32 [requests]: positions in the cache once this step is done
     slots: torch.Tensor         # int32 [requests]: state slot of every request
     want_rows: Optional[torch.Tensor]  # int32 [wanted]: rows of the flat list whose logits are wanted
-    query_tiles: torch.Tensor   # int32 [workgroups, 5]: (request; first token in the flat list and tokens of a tile of
-                                # <= 128 tokens; the same of a second tile, perhaps empty), for the requests that bring
-                                # more than one token (all, if none brings just one); a late tile goes with an early one
-    query_tiles_adjacent: Optional[torch.Tensor]  # the same with neighbouring tiles together, for layers with a window
-                                                  # (None where no layer has one)
-    single_tokens: Optional[torch.Tensor]  # int32: rows of the requests that bring one token, when others bring more
     paged: List[PagedView]
     # the same on the host, for parts written in Python and for choosing kernels
     starts: List[int] = field(default_factory=list)
@@ -62,9 +85,23 @@ class StepContext:
     max_count: int = 0
     max_total: int = 0
     planned_total: int = 0      # the longest request this step's launch shapes are planned for (>= max_total)
-    max_single_total: int = 0   # the longest of the requests listed in single_tokens
+    host: Optional[HostStep] = None
+    # the plans of the parts' planners (key: the planner's): device arrays and host values as attributes
+    planned: Dict[Hashable, SimpleNamespace] = field(default_factory=dict)
     # what a part computes once for the step and its likes in other layers take from here (key: the part's choice)
     memo: dict = field(default_factory=dict)
+
+    def plan_of(self, planner: StepPlanner) -> SimpleNamespace:
+        """The plan of ``planner`` for this step: made with the step if the engine knew the planner (the model's
+        parts name theirs), else made now, with a copy of its own to the device (a part run outside an engine)."""
+        plan = self.planned.get(planner.key)
+        if plan is None:
+            arrays, values = planner.plan(self.host)
+            device = self.tokens.device
+            plan = SimpleNamespace(**values, **{name: torch.from_numpy(np.ascontiguousarray(array, dtype=np.int32)).to(device)
+                                                for name, array in arrays.items()})
+            self.planned[planner.key] = plan
+        return plan
 
 
 class BatchBuilder:
@@ -75,9 +112,13 @@ class BatchBuilder:
     finds every array at the address it had when the graph was captured.
     """
 
-    def __init__(self, cache: CacheManager, device: torch.device):
+    def __init__(self, cache: CacheManager, device: torch.device, planners: Sequence[StepPlanner] = ()):
         self.cache = cache
         self.device = device
+        self.planners: List[StepPlanner] = []
+        for planner in planners:       # one plan a key
+            if all(planner.key != known.key for known in self.planners):
+                self.planners.append(planner)
         self._staging: Optional[torch.Tensor] = None
         self._device_buffer: Optional[torch.Tensor] = None
         self._copied = None
@@ -150,28 +191,20 @@ class BatchBuilder:
             tables.append(table)
             mappings.append(mapping.astype(np.int32, copy=False))
             widths.append(width)
-        windowed = any(getattr(group.need, "window", None) is not None for group in self.cache.groups)
-        if n_tokens == n_seqs:
-            index = np.arange(n_seqs, dtype=np.int32)
-            zero = np.zeros(n_seqs, dtype=np.int32)
-            query_tiles = np.stack([index, index, np.ones(n_seqs, dtype=np.int32), zero, zero], axis=1)
-            adjacent_tiles = query_tiles if windowed else np.zeros((0, 5), dtype=np.int32)
-            single_tokens = np.zeros(0, dtype=np.int32)
-            max_single_total = 0
-        else:
-            mixed = any(count == 1 for count in counts)
-            tile_list = [(index, int(cu[index]) + offset, min(QUERY_TILE, count - offset), starts[index] + offset)
-                         for index, count in enumerate(counts) if not (mixed and count == 1)
-                         for offset in range(0, count, QUERY_TILE)]
-            query_tiles = np.asarray(kernels.pair_query_tiles(tile_list), dtype=np.int32).reshape(-1, 5)
-            adjacent_tiles = np.asarray(kernels.pair_query_tiles(tile_list, adjacent=True) if windowed else [],
-                                        dtype=np.int32).reshape(-1, 5)
-            single_tokens = np.asarray([cu[index] for index, count in enumerate(counts) if mixed and count == 1], dtype=np.int32)
-            max_single_total = max((totals[index] for index, count in enumerate(counts) if mixed and count == 1), default=0)
-        pieces = [tokens, positions, seq_of_token, cu, starts_array, totals_array, slots, want_rows,
-                  query_tiles.reshape(-1), single_tokens, adjacent_tiles.reshape(-1)]
+        host_step = HostStep(n_tokens=n_tokens, n_seqs=n_seqs, page_size=page_size, counts=counts, starts=starts,
+                             totals=totals, cu=cu)
+        pieces = [tokens, positions, seq_of_token, cu, starts_array, totals_array, slots, want_rows]
         for table, mapping in zip(tables, mappings):
             pieces += [table.reshape(-1), mapping]
+        plans = []          # (key, host values, {name: (piece index, shape)})
+        for planner in self.planners:
+            arrays, values = planner.plan(host_step)
+            places = {}
+            for name, array in arrays.items():
+                array = np.ascontiguousarray(array, dtype=np.int32)
+                places[name] = (len(pieces), array.shape)
+                pieces.append(array.reshape(-1))
+            plans.append((planner.key, values, places))
         offsets, cursor = [], 0
         for piece in pieces:
             offsets.append(cursor)
@@ -190,15 +223,15 @@ class BatchBuilder:
 
         paged = []
         for g, group in enumerate(self.cache.groups):
-            paged.append(PagedView(piece_at(11 + 2 * g, (n_seqs, widths[g])), piece_at(12 + 2 * g),
+            paged.append(PagedView(piece_at(8 + 2 * g, (n_seqs, widths[g])), piece_at(9 + 2 * g),
                                    page_size, widths[g]))
+        planned = {key: SimpleNamespace(**values, **{name: piece_at(index, shape) for name, (index, shape) in places.items()})
+                   for key, values, places in plans}
         longest = max(totals) if totals else 0
         return StepContext(
             n_tokens=n_tokens, n_seqs=n_seqs, tokens=piece_at(0), positions=piece_at(1), seq_of_token=piece_at(2),
             cu_tokens=piece_at(3), seq_start=piece_at(4), seq_total=piece_at(5), slots=piece_at(6),
-            want_rows=piece_at(7) if want_rows.size else None, query_tiles=piece_at(8, (-1, 5)),
-            query_tiles_adjacent=piece_at(10, (-1, 5)) if windowed else None,
-            single_tokens=piece_at(9) if single_tokens.size else None, max_single_total=max_single_total, paged=paged,
+            want_rows=piece_at(7) if want_rows.size else None, paged=paged,
             starts=starts, counts=counts, host_slots=slots.tolist(),
             max_count=max(counts) if counts else 0, max_total=longest,
-            planned_total=longest if fixed_width is None else fixed_width * page_size)
+            planned_total=longest if fixed_width is None else fixed_width * page_size, host=host_step, planned=planned)

@@ -15,7 +15,7 @@ from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Union
 
 import torch
 
-from ..cache.manager import CacheManager, RequestCache
+from ..cache.manager import CacheManager, RequestCache, pages_of_group
 from ..cache.pages import OutOfPages
 from ..config.registry import architecture_named, load_config
 from ..ops import kernels, library
@@ -45,7 +45,7 @@ class _DecodeGraph:
     """One captured decode step: its own metadata buffers, the graph and the logits it writes."""
 
     def __init__(self, engine: "Engine", width: int):
-        self.builder = BatchBuilder(engine.cache, engine.device)
+        self.builder = BatchBuilder(engine.cache, engine.device, engine.model.step_planners())
         self.width = width
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
@@ -72,8 +72,10 @@ class Engine:
                  device: Union[str, torch.device] = "cuda:0", page_size: int = 16,
                  max_tokens: Optional[int] = None, num_pages: Optional[int] = None, max_requests: int = 64,
                  tensors_placed: bool = False, use_graphs: bool = True, weight_copies: str = "auto",
-                 consume_tensors: bool = False, tune_library: bool = False):
-        """``weight_copies``: a bfloat16 weight is kept ``"both"`` as stored (for the library's product of steps
+                 consume_tensors: bool = False, tune_library: bool = False, max_portion: Optional[int] = None):
+        """``max_portion``: the most tokens a step brings one request, if the caller keeps to one (a scheduler's
+        prefill chunk): cache groups with a window then get pools no larger than their requests can fill.
+        ``weight_copies``: a bfloat16 weight is kept ``"both"`` as stored (for the library's product of steps
         with many rows) and packed (for the streaming products), or ``"packed"`` only, where memory is short;
         ``"auto"`` keeps both if two copies and the cache fit the GPU's memory. With ``consume_tensors`` the
         entries of ``tensors`` (a dict) are taken out as the parts take them. ``tune_library``: the library times
@@ -99,7 +101,7 @@ class Engine:
         probe = Model(spec, Runtime(dtype=self.dtype, device=self.device))
         decls = probe.tensors()
         if weight_copies == "auto":
-            weight_copies = "both" if self._two_copies_fit(probe, decls, num_pages, page_size) else "packed"
+            weight_copies = "both" if self._two_copies_fit(probe, decls, num_pages, page_size, max_requests, max_portion) else "packed"
         self.weight_copies = weight_copies
         self.runtime = Runtime(dtype=self.dtype, device=self.device, keep_plain_weights=weight_copies == "both")
         self.model = Model(spec, self.runtime)
@@ -108,11 +110,12 @@ class Engine:
         self.model.bind(placed if isinstance(placed, dict) else dict(placed), consume=consume)
         del tensors, placed
         reads = [entry.reads_cache_of for entry in spec.order]
+        self.max_portion = max_portion
         self.cache = CacheManager(self.model.cache_needs(), reads, page_size, num_pages, max_requests,
                                   dtype=self.dtype, device=self.device,
-                                  max_blocks=-(-spec.max_positions // page_size))
+                                  max_blocks=-(-spec.max_positions // page_size), max_portion=max_portion)
         self._bindings = self.cache.bindings()
-        self._builder = BatchBuilder(self.cache, self.device)
+        self._builder = BatchBuilder(self.cache, self.device, self.model.step_planners())
         self.steps_run = 0
         # Steps in which every request brings one token are replayed from HIP graphs, one per (number of
         # requests, block-table width): the launches of a decode step cost more host time than GPU time.
@@ -126,7 +129,8 @@ class Engine:
         self.graph_replays = 0
         self.graphs_captured = 0
 
-    def _two_copies_fit(self, model: Model, decls, num_pages: int, page_size: int) -> bool:
+    def _two_copies_fit(self, model: Model, decls, num_pages: int, page_size: int, max_requests: int,
+                        max_portion: Optional[int]) -> bool:
         """Whether the weights as stored, their packed copies and the cache pool fit the GPU with a tenth to spare."""
         if self.dtype != torch.bfloat16:
             return True     # a float32 engine has no packed copies
@@ -135,7 +139,8 @@ class Engine:
         cache = 0
         for need in model.cache_needs():
             if need is not None and hasattr(need, "kv_heads"):
-                cache += 2 * num_pages * page_size * need.kv_heads * need.head_dim * element
+                pages = pages_of_group(need, num_pages, page_size, max_requests, max_portion)
+                cache += 2 * pages * page_size * need.kv_heads * need.head_dim * element
         total = torch.cuda.get_device_properties(self.device).total_memory
         return 2 * weights + cache <= 0.9 * total
 
@@ -250,6 +255,9 @@ class Engine:
             for token in entry.tokens:
                 if not 0 <= int(token) < self.spec.vocab_size:
                     raise ValueError(f"token {token} of request {entry.request_id!r} is outside the vocabulary")
+            if self.max_portion is not None and count > self.max_portion:
+                raise ValueError(f"request {entry.request_id!r} brings {count} tokens; this engine's cache was sized "
+                                 f"for portions of at most {self.max_portion}")
             if request.num_tokens + count > self.spec.max_positions:
                 raise ValueError(f"request {entry.request_id!r} would pass max positions {self.spec.max_positions}")
             for place in entry.want:

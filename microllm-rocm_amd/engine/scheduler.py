@@ -110,7 +110,8 @@ class Scheduler:
         self.engine = engine
         self.cache = engine.cache
         self.max_batched_tokens = max_batched_tokens
-        self.prefill_chunk = prefill_chunk
+        # a cache whose windowed groups were sized for portions of some length takes no longer ones
+        self.prefill_chunk = min(prefill_chunk, getattr(self.cache, "max_portion", None) or prefill_chunk)
         self.max_requests = min(max_requests or self.cache.max_requests, self.cache.max_requests)
         self.sampler = sampler or Sampler()
         self.requests: Dict[int, Request] = {}
@@ -137,7 +138,7 @@ class Scheduler:
         if total > self.engine.spec.max_positions:
             raise ValueError(f"prompt plus max_new_tokens is {total}, beyond max positions {self.engine.spec.max_positions}")
         for group in self.cache.groups:
-            if self.cache.blocks_for(total) > group.pool.num_pages:
+            if self.cache.most_blocks(group, total, self.prefill_chunk) > group.pool.num_pages:
                 raise ValueError(f"prompt plus max_new_tokens is {total} tokens, more than the cache holds "
                                  f"({group.pool.num_pages * self.cache.page_size})")
         request = Request(self._next_id, prompt, params, arrival_step if arrival_step is not None else self.current_step,
@@ -244,8 +245,8 @@ class Scheduler:
         thrown out again by the next page an older request needs."""
         if not self.running:
             return True      # alone it fits: submit saw to that
-        blocks = self.cache.blocks_for(request.known + 1)
-        return all(blocks <= group.pool.num_free for group in self.cache.groups)
+        return all(self.cache.most_blocks(group, request.known + 1, self.prefill_chunk) <= group.pool.num_free
+                   for group in self.cache.groups)
 
     def step(self) -> List[int]:
         """Run one batch; returns the ids of requests that got a token in this step."""

@@ -649,11 +649,12 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, view, ctx,
-                    scale: float, window: int, heads: int, kv_heads: int, head_dim: int) -> torch.Tensor:
+                    scale: float, window: int, heads: int, kv_heads: int, head_dim: int, planner=None) -> torch.Tensor:
     """Attention of the step's queries over their requests' pages; chooses the kernel for the batch's shape.
 
     bfloat16 with a head size in steps of 16: the MFMA kernels, split over the keys when every request brings
-    one token, tiled over the queries otherwise. Everything else (float32, other head sizes): the plain kernel.
+    one token, tiled over the queries otherwise (``planner``: the attention part's, whose plan for the step
+    holds the tiles). Everything else (float32, other head sizes): the plain kernel.
     """
     mfma_fits = q.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256
     if mfma_fits and ctx.max_count == 1:
@@ -664,16 +665,17 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                       scale, window, heads, kv_heads, head_dim, splits)
     if mfma_fits:
         # Portions go to the tiled kernel; requests that bring one token, if any, to the split kernel.
+        _need(planner is not None, "portions of prompts need the attention part's planner for their tiles")
+        plan = ctx.plan_of(planner)
         out = torch.empty_like(q)
-        if ctx.query_tiles.shape[0] > 0:
-            tiles = ctx.query_tiles_adjacent if window > 0 and ctx.query_tiles_adjacent is not None else ctx.query_tiles
-            paged_attention_prefill(q, k_cache, v_cache, view.block_table, tiles, ctx.positions,
+        if plan.tiles.shape[0] > 0:
+            paged_attention_prefill(q, k_cache, v_cache, view.block_table, plan.tiles, ctx.positions,
                                     scale, window, heads, kv_heads, head_dim, out=out)
-        if ctx.single_tokens is not None:
-            visible = min(ctx.max_single_total, window) if window > 0 else ctx.max_single_total
-            splits = decode_splits(ctx.single_tokens.shape[0], kv_heads, visible)
+        if plan.single_tokens.shape[0] > 0:
+            visible = min(plan.max_single_total, window) if window > 0 else plan.max_single_total
+            splits = decode_splits(plan.single_tokens.shape[0], kv_heads, visible)
             paged_attention_decode(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
-                                   scale, window, heads, kv_heads, head_dim, splits, out=out, token_ids=ctx.single_tokens)
+                                   scale, window, heads, kv_heads, head_dim, splits, out=out, token_ids=plan.single_tokens)
         return out
     return paged_attention_rowwise(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
                                    scale, window, heads, kv_heads, head_dim)

@@ -13,6 +13,7 @@ from __future__ import annotations
 import math
 from typing import Dict, Mapping, Optional
 
+import numpy as np
 import torch
 
 from ..ops import kernels
@@ -20,6 +21,34 @@ from .base import MATRIX, Mixer, PagedKVNeed, Runtime, TensorDecl, VECTOR
 from .linear import SKINNY_ROWS, UnscaledRows, Weight, linear, linear_into_stream, takes_packed, takes_unscaled
 from .registry import build_part, register_part
 from .spec import PartSpec
+
+
+class QueryTilePlanner:
+    """The step metadata of the MFMA attention kernels (an ``engine.batch.StepPlanner``): requests that bring
+    several tokens are cut into tiles of ``kernels.QUERY_TILE`` queries, which go to the prefill kernel's
+    workgroups in twos (``kernels.pair_query_tiles``: a late tile with an early one, or neighbours under a
+    window); requests that bring one token beside them are listed for the decode kernel. In a step of single
+    tokens only there is nothing to plan: the decode kernel takes every row.
+
+    Plan: ``tiles`` int32 [workgroups, 5]; ``single_tokens`` int32 [rows]; ``max_single_total``, the longest of
+    the requests listed there."""
+
+    def __init__(self, adjacent: bool):
+        self.adjacent = adjacent
+        self.key = ("paged_attention_query_tiles", adjacent)
+
+    def plan(self, host):
+        counts, cu = host.counts, host.cu
+        if host.single_tokens_only:
+            return {"tiles": np.zeros((0, 5), np.int32), "single_tokens": np.zeros(0, np.int32)}, {"max_single_total": 0}
+        mixed = any(count == 1 for count in counts)
+        tile_list = [(index, int(cu[index]) + offset, min(kernels.QUERY_TILE, count - offset), host.starts[index] + offset)
+                     for index, count in enumerate(counts) if not (mixed and count == 1)
+                     for offset in range(0, count, kernels.QUERY_TILE)]
+        tiles = np.asarray(kernels.pair_query_tiles(tile_list, adjacent=self.adjacent), dtype=np.int32).reshape(-1, 5)
+        single = np.asarray([cu[index] for index, count in enumerate(counts) if mixed and count == 1], dtype=np.int32)
+        longest = max((host.totals[index] for index, count in enumerate(counts) if mixed and count == 1), default=0)
+        return {"tiles": tiles, "single_tokens": single}, {"max_single_total": longest}
 
 
 class PagedAttention(Mixer):
@@ -40,6 +69,7 @@ class PagedAttention(Mixer):
             raise ValueError("num_heads must divide into num_kv_heads groups")
         position = p.get("position")
         self.position = build_part("position", position, runtime) if position is not None else None
+        self.planner = QueryTilePlanner(adjacent=bool(self.window))
         self.qkv_weight: Optional[torch.Tensor] = None
         self.qkv_bias_vector: Optional[torch.Tensor] = None
         self.o_weight: Optional[torch.Tensor] = None
@@ -77,6 +107,12 @@ class PagedAttention(Mixer):
             biases = [tensors[self.name(f"{role}_proj.bias")] for role, _ in self._projections()]
             self.qkv_bias_vector = torch.cat(biases, dim=0).contiguous() if len(biases) > 1 else biases[0]
         self.o_weight = Weight(tensors[self.name("o_proj.weight")], keep_plain=self.runtime.keep_plain_weights)
+
+    def sub_parts(self):
+        return (self.position,) if self.position is not None else ()
+
+    def step_planner(self):
+        return self.planner
 
     def cache_need(self):
         if not self.owns_kv:
@@ -119,7 +155,7 @@ class PagedAttention(Mixer):
                                        pair_order=pair_order, cos_sin=cos_sin)
         window = int(self.window) if self.window else 0
         o = kernels.paged_attention(q, cache.k, cache.v, view, ctx, self.scale, window,
-                                    self.heads, kv_heads, self.head_dim)
+                                    self.heads, kv_heads, self.head_dim, planner=self.planner)
         if residual is not None:
             begun = linear_into_stream(o, self.o_weight, residual)
             if begun is not None:

@@ -8,7 +8,7 @@ with the spec. Categories are ``norm``, ``position``, ``mixer``, ``ffn``,
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, Mapping, Optional, Tuple, Union
+from typing import Dict, Mapping, Optional, Sequence, Tuple, Union
 
 import torch
 
@@ -70,6 +70,17 @@ class Part:
 
     def bind(self, tensors: Mapping[str, torch.Tensor]) -> None:
         """Take the loaded tensors (by file name); called once, before the first forward."""
+
+    def sub_parts(self) -> Sequence["Part"]:
+        """Parts that this part built for itself (an attention's position encoding): the model asks, so that it
+        knows every part it runs without knowing how any is put together."""
+        return ()
+
+    def step_planner(self):
+        """A ``StepPlanner`` (engine/batch.py) if this part's kernels need metadata of their own for every step
+        (tiles of queries, work lists), made on the host from the batch's shape and copied to the device with
+        the step's other metadata; None otherwise. ``ctx.plan_of(planner)`` gives the plan in ``forward``."""
+        return None
 
     def name(self, role: str) -> str:
         try:

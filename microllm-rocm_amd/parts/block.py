@@ -29,11 +29,17 @@ class Block:
         self.spec = spec
         self.mixer_norm = build_part("norm", spec.mixer_norm, runtime)
         self.mixer = build_part("mixer", spec.mixer, runtime)
-        self.ffn_norm = build_part("norm", spec.ffn_norm, runtime)
-        self.ffn = build_part("ffn", spec.ffn, runtime)
+        if (spec.ffn is None) != (spec.ffn_norm is None):
+            raise ValueError("a layer has a feed-forward and its norm, or neither")
+        self.ffn_norm = build_part("norm", spec.ffn_norm, runtime) if spec.ffn_norm is not None else None
+        self.ffn = build_part("ffn", spec.ffn, runtime) if spec.ffn is not None else None
+        self.extra: Dict[str, Part] = {name: build_part(category, part_spec, runtime)
+                                       for name, (category, part_spec) in spec.extra.items()}
 
     def parts(self):
-        return (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
+        """Every part of the layer (the cache manager asks ``mixer`` alone for a cache)."""
+        own = (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
+        return tuple(part for part in own if part is not None) + tuple(self.extra.values())
 
     def tensors(self) -> Dict[str, TensorDecl]:
         decls: Dict[str, TensorDecl] = {}
@@ -70,6 +76,9 @@ class PreNormBlock(Block):
     def forward(self, h, pending, ctx, cache, next_block=None):
         rows = h.shape[0]
         x = pending if isinstance(pending, UnscaledRows) else self.mixer_norm.forward(h, delta=pending, write_h=True)
+        if self.ffn is None:        # no feed-forward: the mixer's delta goes to whatever norm comes next
+            residual = next_block.first_norm_after(self.mixer, rows, h) if next_block is not None else None
+            return self.mixer.forward(x, ctx, cache, residual=residual) if residual is not None else self.mixer.forward(x, ctx, cache)
         residual = residual_for(self.mixer, self.ffn_norm, self.ffn, rows, h)
         mixed = self.mixer.forward(x, ctx, cache, residual=residual) if residual is not None else self.mixer.forward(x, ctx, cache)
         x = mixed if isinstance(mixed, UnscaledRows) else self.ffn_norm.forward(h, delta=mixed, write_h=True)

@@ -124,13 +124,29 @@ class Model:
         self.head.bind(tensors)
 
     def parts(self) -> List[Part]:
-        found: List[Part] = [self.embedding, self.final_norm, self.head]
+        """Every part the model runs, the parts' own sub-parts included."""
+        found: List[Part] = []
+
+        def add(part: Part) -> None:
+            found.append(part)
+            for inner in part.sub_parts():
+                add(inner)
+
+        for part in (self.embedding, self.final_norm, self.head):
+            add(part)
         for block in self.blocks:
-            found += list(block.parts())
-            position = getattr(block.mixer, "position", None)
-            if position is not None:
-                found.append(position)
+            for part in block.parts():
+                add(part)
         return found
+
+    def step_planners(self) -> list:
+        """The planners of the parts that want step metadata of their own, one per key."""
+        planners = []
+        for part in self.parts():
+            planner = part.step_planner()
+            if planner is not None and all(planner.key != known.key for known in planners):
+                planners.append(planner)
+        return planners
 
     def cache_needs(self) -> List[CacheNeed]:
         """The cache need of every run entry; None for an entry that owns none."""

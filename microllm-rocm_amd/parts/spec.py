@@ -23,12 +23,18 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: a mixer and a feed-forward, each behind its norm, in an arrangement."""
+    """One layer: a mixer and, usually, a feed-forward, each behind its norm, in an arrangement.
+
+    A layer without a feed-forward leaves ``ffn`` and ``ffn_norm`` out. What an arrangement needs beyond these
+    (a norm after the mixer, norms of queries and keys outside the mixer, a second mixer) goes into ``extra``:
+    a name of the arrangement's choice -> (category, spec); the block builds each and finds it in
+    ``Block.extra[name]``."""
     arrangement: str  # e.g. "pre_norm"
     mixer_norm: PartSpec
     mixer: PartSpec
-    ffn_norm: PartSpec
-    ffn: PartSpec
+    ffn_norm: Optional[PartSpec] = None
+    ffn: Optional[PartSpec] = None
+    extra: Mapping[str, Tuple[str, PartSpec]] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)

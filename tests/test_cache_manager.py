@@ -162,3 +162,40 @@ def test_random_orders_never_lose_a_page(seed):
         cache.close(key)
     cache.check()
     assert cache.free_pages() == [12, 12] and cache.slots.num_free == 4
+
+
+def test_a_group_with_a_window_sizes_its_own_pool_and_long_requests_fit_it():
+    from microllm_rocm_amd.cache.manager import pages_of_group, window_blocks
+    # window 24, portions of at most 16, pages of 16: a request never holds more than 4 blocks of the windowed group
+    assert window_blocks(24, 16, 16) == 4
+    assert pages_of_group(WINDOW, 1000, 16, 4, 16) == 16 and pages_of_group(FULL, 1000, 16, 4, 16) == 1000
+    assert pages_of_group(WINDOW, 1000, 16, 4, None) == 1000 and pages_of_group(WINDOW, 10, 16, 4, 16) == 10
+    cache = CacheManager([FULL, WINDOW], [None, None], 16, 128, 2, device=None, max_blocks=64, max_portion=16)
+    assert [group.pool.num_pages for group in cache.groups] == [128, 8]
+    assert cache.allocated_bytes() == (128 + 8) * 2 * 2 * 16 * 16 * 4
+    # two requests of 500 tokens each, in portions of up to 16: the windowed pool of 8 pages is enough, and the
+    # bound on what a request holds is never passed
+    rng = np.random.default_rng(0)
+    requests = [cache.open(name) for name in "ab"]
+    lengths = [0, 0]
+    most = 0
+    while min(lengths) < 500:
+        which = int(rng.integers(0, 2)) if max(lengths) < 900 else int(np.argmin(lengths))
+        count = int(rng.integers(1, 17))
+        cache.reserve(requests[which], count)
+        most = max(most, max(sum(page != RELEASED for page in request.pages[1]) for request in requests))
+        cache.commit(requests[which], count)
+        lengths[which] += count
+        if rng.random() < 0.1:
+            cache.check()
+    assert most <= 4 and cache.most_blocks(cache.groups[1], 500, 16) == 4 and cache.most_blocks(cache.groups[0], 500, 16) == 32
+    assert cache.most_blocks(cache.groups[1], 20, 16) == 2          # a short request never holds more than its length
+    cache.check()
+    # a portion longer than the pool was sized for is refused as a whole, nothing taken
+    held = cache.held_pages()
+    with pytest.raises(OutOfPages):
+        cache.reserve(requests[0], 16 * 9)
+    assert cache.held_pages() == held
+    for name in "ab":
+        cache.close(name)
+    assert cache.free_pages() == [128, 8]

@@ -115,3 +115,11 @@ def test_which_product_a_linear_takes():
     wide = Weight(torch.zeros((16, 8), dtype=torch.bfloat16), pack=False)
     wide.packed, wide.out_features = packed.packed, 2048 * 16
     assert takes_packed(wide, 40) and not takes_packed(wide, 41), "weights with many tiles go to the library from 41 rows on"
+
+
+def test_percentile_interpolates_between_the_two_nearest_sorted_values():
+    from microllm_rocm_amd.cli.hf_infer import percentile
+    assert percentile([4, 1, 3, 2], 0.5) == 2.5 and percentile([7.0], 0.95) == 7.0
+    assert percentile([1, 2, 3, 4, 5], 0.95) == pytest.approx(4.8) and percentile([5, 1], 0.0) == 1 and percentile([5, 1], 1.0) == 5
+    with pytest.raises(ValueError):
+        percentile([], 0.5)

@@ -793,3 +793,63 @@ def test_library_tuning_keeps_the_product_and_is_switched_per_shape(tmp_path):
     finally:
         ka.set_library_tuning(False)
     assert not ka.library_tuning() and not tunable.is_enabled()
+
+
+# ---- the products at the largest sizes the engine runs: a full vocabulary, the widths of the largest model ---------
+def float32_oracle(a, w):
+    """``a @ w.T`` of the widened bfloat16 operands, in true float32 on the GPU with a long double check on a sample:
+    an oracle that does not share a line with the kernels and fits the memory at these sizes."""
+    previous = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        expected = a.float() @ w.float().t()
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = previous
+    rng = np.random.default_rng(0)
+    rows, cols = rng.integers(0, a.shape[0], size=64), rng.integers(0, w.shape[0], size=64)
+    exact = (a[rows].double() * w[cols].double()).sum(dim=1)
+    scale = expected.abs().max().item()
+    assert (expected[rows, cols].double() - exact).abs().max().item() <= 2e-6 * scale
+    return expected
+
+
+@pytest.mark.parametrize("n,k", [(152064, 3584), (152064, 8192), (8192, 29568), (2 * 29568, 8192)])
+def test_products_at_full_vocabulary_and_the_largest_widths(n, k):
+    """The head over 152 064 tokens and the projections of hidden 8192 / intermediate 29 568, through each of the
+    three products, against a float32 product of the same operands: skinny at 1, 8 and 16 rows, medium at 17 and
+    64, tiled at 300 (two tiles of rows, the second ragged)."""
+    ka = kernels()
+    generator = torch.Generator(device=DEVICE).manual_seed(n + k)
+    w = (torch.randn((n, k), generator=generator, device=DEVICE) * 0.05).to(torch.bfloat16)
+    a = torch.randn((300, k), generator=generator, device=DEVICE).to(torch.bfloat16)
+    a[7, 100] = 50.0          # one large entry: a row whose sum a wrong k range or a dropped tail would miss
+    w[n - 1, k - 1] = 1.0     # the last element of the last row counts
+    a[0, k - 1] = 30.0
+    packed = ka.pack_weight(w)
+    expected = float32_oracle(a, w)
+    scale = expected.abs().max().item()
+
+    def check(out, rows, bound):
+        assert out.shape == (rows, n)
+        error = (out.float() - expected[:rows]).abs().max().item()
+        assert error <= bound * scale, f"n {n} k {k} rows {rows}: error {error / scale:.2e} of the scale"
+
+    for rows in (1, 8, 16):
+        check(ka.gemm_skinny(a[:rows].contiguous(), packed, n, "f32"), rows, 2e-5)
+    check(ka.gemm_skinny(a[:16].contiguous(), packed, n, "bf16"), 16, 5e-3)
+    for rows in (17, 64):
+        out = ka.gemm_medium(a[:rows].contiguous(), packed, n, "f32")
+        check(out.sum(dim=0) if out.dim() == 3 else out, rows, 2e-5)
+        check(ka.gemm_medium(a[:rows].contiguous(), packed, n, "bf16"), rows, 5e-3)
+    check(ka.gemm_tiled(a, packed, n, "f32"), 300, 2e-5)
+    check(ka.gemm_tiled(a, packed, n, "bf16"), 300, 5e-3)
+    splits = ka.tiled_splits(300, n, k)
+    if splits > 1:
+        check(ka.gemm_tiled(a, packed, n, "f32", splits=splits).sum(dim=0), 300, 2e-5)
+    if n == 2 * 29568:        # gate and up of the largest feed-forward: the gated epilogues
+        gated = ka.pack_weight(w, interleave_halves=True)
+        want = torch.nn.functional.silu(expected[:, :n // 2]) * expected[:, n // 2:]
+        bound = 1.2e-2 * want.abs().max().item()
+        for rows, product in ((16, ka.gemm_skinny), (40, ka.gemm_medium), (300, ka.gemm_tiled)):
+            got = product(a[:rows].contiguous(), gated, n, "gated")
+            assert got.shape == (rows, n // 2) and (got.float() - want[:rows]).abs().max().item() <= bound

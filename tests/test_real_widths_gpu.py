@@ -22,6 +22,10 @@ WIDE = {
     "0.5b": Qwen2Config(vocab_size=15013, hidden_size=896, num_hidden_layers=2, num_attention_heads=14, num_key_value_heads=2,
                         head_dim=64, intermediate_size=4864, max_position_embeddings=4096, rope_theta=1e6, rms_norm_eps=1e-6,
                         tie_word_embeddings=True),
+    # one layer at the widths of the largest model (kept in the packed order alone on one GPU)
+    "72b": Qwen2Config(vocab_size=10007, hidden_size=8192, num_hidden_layers=1, num_attention_heads=64, num_key_value_heads=8,
+                       head_dim=128, intermediate_size=29568, max_position_embeddings=4096, rope_theta=1e6, rms_norm_eps=1e-6,
+                       tie_word_embeddings=False),
 }
 _models = {}
 
@@ -90,3 +94,86 @@ def test_real_widths_with_the_packed_weights_alone(tmp_path_factory, tmp_path, w
     steps, peak = mixed(requests, seed=9)
     run_trace(folder, "bfloat16", steps, tmp_path / "mixed", max_tokens=peak, weight_copies="packed")
     compare(collect(steps, tmp_path / "mixed", config.vocab_size), requests, plain_model, "bfloat16")
+
+
+def staggered_then_together(requests, tail, wave):
+    """Prompts come in waves of ``wave`` requests a step, each whole but for its last ``tail`` tokens, beside single
+    tokens of up to three requests of earlier waves (which therefore run ahead); then every request decodes, all of
+    them in every step, until each has fed its tokens: steps of as many rows as there are live requests."""
+    ids = list(requests)
+    fed = {rid: 0 for rid in ids}
+    steps = []
+    for first in range(0, len(ids), wave):
+        entries = []
+        for rid in ids[:first][:3]:
+            if len(requests[rid]) - fed[rid] > 2:        # keeps at least two tokens for the steps together
+                entries.append({"id": rid, "tokens": [requests[rid][fed[rid]]], "want": [0]})
+                fed[rid] += 1
+        for rid in ids[first:first + wave]:
+            count = len(requests[rid]) - tail
+            entries.append({"id": rid, "tokens": requests[rid][:count], "want": list(range(count))})
+            fed[rid] = count
+        steps.append({"step": len(steps), "entries": entries, "end": []})
+    while any(fed[rid] < len(requests[rid]) for rid in ids):
+        entries, ended = [], []
+        for rid in ids:
+            if fed[rid] < len(requests[rid]):
+                entries.append({"id": rid, "tokens": [requests[rid][fed[rid]]], "want": [0]})
+                fed[rid] += 1
+                if fed[rid] == len(requests[rid]):
+                    ended.append(rid)
+        steps.append({"step": len(steps), "entries": entries, "end": ended})
+    return steps
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_many_requests_decode_together_at_real_widths(tmp_path_factory, tmp_path, dtype):
+    """Decode steps of 17, 40, 64 and 96 rows at 7B widths: from 17 rows on the products share their activations
+    through LDS and the norms, the rotation and SiLU run as kernels of their own; beyond 64 rows the library's
+    products run inside the captured graph; block tables have dozens of rows of differing lengths."""
+    from microllm_rocm_amd.engine import Engine
+    from microllm_rocm_amd.engine.replay import replay
+    config = WIDE["7b"]
+    folder, plain_model = model_for(tmp_path_factory, "7b")
+    lengths = np.random.default_rng(17).integers(9, 30, size=96)
+    everyone = {f"m{index}": random_tokens(500 + index, int(length), config.vocab_size) for index, length in enumerate(lengths)}
+    engine = Engine.from_folder(folder, dtype=dtype, max_tokens=96 * 64, max_requests=128)
+    alone = {}
+    for count in (17, 40, 64, 96):
+        requests = dict(list(everyone.items())[:count])
+        steps = staggered_then_together(requests, tail=5, wave=11)
+        assert max(len(step["entries"]) for step in steps) == count
+        out = tmp_path / f"together_{count}"
+        replays_before = engine.graph_replays
+        replay(engine, io.StringIO(to_lines(steps)), str(out), io.StringIO())
+        engine.cache.check()
+        assert not engine.cache.requests and engine.graph_replays > replays_before
+        got = collect(steps, out, config.vocab_size)
+        compare(got, requests, plain_model, dtype)
+        if dtype == "float32":
+            if not alone:
+                steps_alone = whole(everyone)
+                replay(engine, io.StringIO(to_lines(steps_alone)), str(tmp_path / "alone"), io.StringIO())
+                alone = collect(steps_alone, tmp_path / "alone", config.vocab_size)
+            for key, row in got.items():
+                assert np.array_equal(row, alone[key]), f"{count} together: {key} differs from the request run alone"
+
+
+def test_one_layer_at_the_largest_widths_with_the_packed_weights_alone(tmp_path_factory, tmp_path):
+    """Hidden 8192, 64 query heads in 8 groups, a feed-forward of 29 568: prompts through the tiled product, decoding
+    and mixed steps through the streaming products, no copy of the weights for the library."""
+    config = WIDE["72b"]
+    folder, plain_model = model_for(tmp_path_factory, "72b")
+    requests = {f"r{index}": random_tokens(90 + index, length, config.vocab_size) for index, length in enumerate([140, 37, 70])}
+    steps = whole(requests)
+    engine = run_trace(folder, "bfloat16", steps, tmp_path / "whole", weight_copies="packed",
+                       max_tokens=round_up(sum(len(t) for t in requests.values()), 64) + 256)
+    assert all(block.ffn.down_weight.tensor is None and block.mixer.qkv_weight.tensor is None for block in engine.model.blocks)
+    compare(collect(steps, tmp_path / "whole", config.vocab_size), requests, plain_model, "bfloat16")
+    del engine
+    steps, peak = mixed(requests, seed=3)
+    run_trace(folder, "bfloat16", steps, tmp_path / "mixed", max_tokens=peak, weight_copies="packed")
+    compare(collect(steps, tmp_path / "mixed", config.vocab_size), requests, plain_model, "bfloat16")
+    steps = prefill_then_decode("r0", requests["r0"], tail=32)
+    run_trace(folder, "bfloat16", steps, tmp_path / "decode", max_tokens=round_up(len(requests["r0"]), 64), weight_copies="packed")
+    compare(collect(steps, tmp_path / "decode", config.vocab_size), {"r0": requests["r0"]}, plain_model, "bfloat16")

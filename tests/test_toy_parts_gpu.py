@@ -291,3 +291,96 @@ def test_toy_arrangement_beside_the_packages_own(dtype):
         rows.append(engine.step([StepEntry("cut", [token], [0])]).double().cpu().numpy())
     assert np.abs(np.concatenate(rows) - expected).max() <= tolerance * np.abs(expected).max()
     engine.cache.check()
+
+
+# ---- a layer with a third norm, and one without a feed-forward -------------------------------------------------------
+def sandwich_block_class():
+    """A toy arrangement with a norm that the layer's spec carries under ``extra``: the mixer's result is normalised
+    by itself before it is added to the stream."""
+    from microllm_rocm_amd.parts import Block
+
+    class Sandwich(Block):
+        def first_norm_after(self, producer, rows, h):
+            return None
+
+        def forward(self, h, pending, ctx, cache, next_block=None):
+            x = self.mixer_norm.forward(h, delta=pending, write_h=True)
+            mixed = self.mixer.forward(x, ctx, cache)
+            mixed = (mixed.sum(dim=0) if mixed.dim() == 3 else mixed).float().contiguous()
+            mixed = self.extra["after_mixer"].forward(mixed, write_h=False)          # a norm of the delta alone
+            x = self.ffn_norm.forward(h, delta=mixed, write_h=True)
+            return self.ffn.forward(x, ctx)
+
+    return Sandwich
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_layer_with_a_third_norm_and_a_layer_without_a_feed_forward(dtype):
+    from microllm_rocm_amd.parts import register_arrangement
+    register_arrangement("toy_sandwich", sandwich_block_class(), replace=True)
+    arrangements = ("toy_sandwich", "pre_norm", "pre_norm", "pre_norm")
+    has_ffn = (True, False, True, False)          # the last layer has none either: its mixer's delta goes to the final norm
+    layers = []
+    for index, arrangement in enumerate(arrangements):
+        prefix = f"layers.{index}"
+        names = {f"{role}_proj.{kind}": f"{prefix}.attn.{role}.{kind}" for role in ("q", "k", "v") for kind in ("weight", "bias")}
+        names["o_proj.weight"] = f"{prefix}.attn.o.weight"
+        position = PartSpec("rope_split_half", {"theta": THETA, "head_dim": HEAD_DIM})
+        mixer = PartSpec("paged_attention", {"hidden_size": HIDDEN, "num_heads": HEADS, "num_kv_heads": KV_HEADS, "head_dim": HEAD_DIM,
+                                             "qkv_bias": True, "window": None, "position": position}, names)
+        norm = lambda name: PartSpec("rms_norm", {"size": HIDDEN, "eps": EPS}, {"weight": f"{prefix}.{name}"})
+        ffn = PartSpec("swiglu", {"hidden_size": HIDDEN, "intermediate_size": INTER},
+                       {f"{r}_proj.weight": f"{prefix}.ffn.{r}" for r in ("gate", "up", "down")})
+        extra = {"after_mixer": ("norm", norm("norm_after_mixer"))} if arrangement == "toy_sandwich" else {}
+        if has_ffn[index]:
+            layers.append(LayerSpec(arrangement, norm("norm1"), mixer, norm("norm2"), ffn, extra=extra))
+        else:
+            layers.append(LayerSpec(arrangement, norm("norm1"), mixer))
+    sizes = {"vocab_size": VOCAB, "hidden_size": HIDDEN}
+    spec = ModelSpec("ToyLayers", VOCAB, HIDDEN, 512, PartSpec("token_embedding", sizes, {"weight": "embed"}), tuple(layers),
+                     tuple(RunEntry(index) for index in range(len(layers))),
+                     PartSpec("rms_norm", {"size": HIDDEN, "eps": EPS}, {"weight": "norm"}), PartSpec("lm_head", sizes, {"weight": "head"}))
+    tensors = toy_tensors(spec)
+    # the third norm brings the mixer's result to unit size whatever it was, its rounding with it: with a weight of
+    # about a quarter the stream keeps the proportions the other toy models have (and the bound that is theirs)
+    tensors["layers.0.norm_after_mixer"] = (tensors["layers.0.norm_after_mixer"].float() * 0.25).to(torch.bfloat16)
+    assert "layers.0.norm_after_mixer" in tensors and "layers.1.norm2" not in tensors and "layers.1.ffn.gate" not in tensors
+    engine = Engine(spec, tensors, dtype=dtype, max_tokens=512)
+    tokens = np.random.default_rng(6).integers(0, VOCAB, size=60).tolist()
+
+    w = {name: value.double().numpy() for name, value in tensors.items()}
+    h = plain.embedding(w["embed"], tokens)
+    count, positions = len(tokens), np.arange(len(tokens))
+    for index, arrangement in enumerate(arrangements):
+        p = f"layers.{index}"
+        x = plain.rms_norm(h, w[f"{p}.norm1"], EPS)
+        q = plain.linear(x, w[f"{p}.attn.q.weight"], w[f"{p}.attn.q.bias"]).reshape(count, HEADS, HEAD_DIM)
+        k = plain.linear(x, w[f"{p}.attn.k.weight"], w[f"{p}.attn.k.bias"]).reshape(count, KV_HEADS, HEAD_DIM)
+        v = plain.linear(x, w[f"{p}.attn.v.weight"], w[f"{p}.attn.v.bias"]).reshape(count, KV_HEADS, HEAD_DIM)
+        q, k = plain.rope_split_half(q, positions, THETA), plain.rope_split_half(k, positions, THETA)
+        o = plain.causal_gqa_attention(q, k, v, 1.0 / math.sqrt(HEAD_DIM), None).reshape(count, HEADS * HEAD_DIM)
+        mixed = plain.linear(o, w[f"{p}.attn.o.weight"])
+        if arrangement == "toy_sandwich":
+            mixed = plain.rms_norm(mixed, w[f"{p}.norm_after_mixer"], EPS)
+        h = h + mixed
+        if has_ffn[index]:
+            h = h + plain.swiglu_ffn(plain.rms_norm(h, w[f"{p}.norm2"], EPS), w[f"{p}.ffn.gate"], w[f"{p}.ffn.up"], w[f"{p}.ffn.down"])
+    expected = plain.rms_norm(h, w["norm"], EPS) @ w["head"].T
+    tolerance = 2e-5 if dtype == "float32" else 4e-2
+
+    engine.open("whole")
+    whole = engine.step([StepEntry("whole", tokens, list(range(count)))]).double().cpu().numpy()
+    engine.close("whole")
+    assert np.abs(whole - expected).max() <= tolerance * np.abs(expected).max()
+    # in portions, then token by token from a graph (every part here says it is graph-safe): with few rows the
+    # layer without a feed-forward hands its mixer's sum and the next layer's norm to the products around them
+    assert engine.use_graphs
+    engine.open("cut")
+    rows, position = [], 0
+    for size in (21, 2, 19):
+        rows.append(engine.step([StepEntry("cut", tokens[position:position + size], list(range(size)))]).double().cpu().numpy())
+        position += size
+    for token in tokens[position:]:
+        rows.append(engine.step([StepEntry("cut", [token], [0])]).double().cpu().numpy())
+    assert np.abs(np.concatenate(rows) - expected).max() <= tolerance * np.abs(expected).max()
+    engine.cache.check()
