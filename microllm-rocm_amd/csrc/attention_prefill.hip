@@ -1,24 +1,27 @@
 // Paged attention for portions of prompts in bfloat16: MFMA for both products, online softmax in float32.
 //
 // A workgroup (8 waves) takes two tiles of up to 128 consecutive tokens each, of one request's portion and one
-// query head. A wave takes two blocks of 16 tokens (16 columns of the MFMA): 16 tokens of the first tile and 16 of
-// the second. The host pairs a tile that sees many keys with one that sees few, so that every workgroup walks
-// about as many keys and the compute units finish together (under a causal mask the last tile of a prompt has
-// as many times the work of the first as there are tiles); both tiles read the same keys from LDS, and every
-// wave has work to the end of the longer walk. The second tile may be empty: then waves 0-3 take 32 consecutive
-// tokens each.
+// query head: waves 0 to 3 a block of 32 tokens each of the first tile, waves 4 to 7 of the second; the 32 tokens
+// are the 32 columns of v_mfma_f32_32x32x16_bf16. Every SIMD thus has a wave of either tile, whose matrix and
+// vector work overlap. The host pairs a tile that sees many keys with one that sees few where a prompt has few
+// tiles, so that every workgroup walks about as many keys and the compute units finish together (under a causal
+// mask the last tile of a prompt has as many times the work of the first as there are tiles), and neighbouring
+// tiles where there are many or under a window: these read nearly the same keys, and the longest workgroups go
+// first. Both tiles read the same keys from LDS. The second tile may be empty.
 // The workgroup walks the keys its tokens can see in blocks of 128 (64 for head sizes above 128): the block's key
 // and value tiles are copied from the pages straight into LDS as they lie there (the pages are in MFMA order,
 // cache_layout.h), the next block's being on its way while this one is used. The two stages are two LDS
-// variables, so that the compiler need not wait for a load into one before it reads the other. As in the decode
-// kernel, scores are computed transposed, S^T = K . Q^T, the 16 columns being query positions, and
-// O^T = V^T . P^T follows from registers; every fragment of K and V read from LDS serves both column blocks.
-// Only pairs of key tiles that touch the causal diagonal or the window's edge pay for the mask (they run a second
-// instance of the inner loop's body), and values that no token of the workgroup can see are cleared in LDS before
-// a block at an end of the walk is used, so that stale memory never meets a zero weight.
-// The vector unit and the reads from LDS, not the MFMA, bound this kernel: the scale is folded into the exponent's
-// multiply-add and the accumulators are rescaled only when some maximum has moved.
-// The list of workgroups (request; first token in the flat list and tokens, for either tile) is built on the host.
+// variables, so that the compiler need not wait for a load into one before it reads the other.
+// Scores are computed transposed, S^T = K . Q^T: a lane then holds 16 keys of one token (its column), and the other
+// half of the wave the other 16, so a token's maximum takes 15 comparisons and one exchange, and its sum is kept in
+// two halves that meet once, at the end. O^T = V^T . P^T follows from registers: the lane's scores of a 16-key tile
+// are the 8 values the second product wants from it, if the values' operand is read in the same order.
+// Only steps that touch the causal diagonal or the window's edge pay for the mask (a second
+// instance of the loop's body), and values that no token of the workgroup can see are cleared in LDS before a
+// block at an end of the walk is used, so that stale memory never meets a zero weight.
+// The scale is folded into the exponent's multiply-add and the accumulators are rescaled only when some maximum
+// has moved. The list of workgroups (request; first token in the flat list and tokens, for either tile) is built on
+// the host.
 #include <type_traits>
 
 #include "cache_layout.h"
@@ -30,16 +33,26 @@ namespace mll {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kPrefillWaves = 8;
 constexpr int kPrefillThreads = kPrefillWaves * kWave;
-constexpr int kPrefillTile = 16 * kPrefillWaves;   // tokens of one tile; a workgroup takes two tiles
+constexpr int kPrefillTile = 128;     // tokens of one tile: four blocks of 32, a wave each
 
 union PFrag8 {
     bf16x8 v;
     bf16x4 h[2];
     uint4 raw;
 };
+
+// op over the two lanes {l, l ^ 32} of a wave, both of which get the result (v_permlane32_swap of gfx950).
+template <typename Op>
+__device__ inline float reduce_lanes_32_apart(float value, Op op) {
+    const unsigned bits = __builtin_bit_cast(unsigned, value);
+    const auto halves = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+    const unsigned low = halves[0], high = halves[1];
+    return op(__builtin_bit_cast(float, low), __builtin_bit_cast(float, high));
+}
 
 template <int HD_TILES>
 __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_kernel(
@@ -48,10 +61,11 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     const int32_t* __restrict__ positions, bf16* __restrict__ out, float scale, int window, int heads,
     int kv_heads, int page_size) {
     constexpr int HD = HD_TILES * 16;
-    constexpr int K_STEPS = (HD + 31) / 32;
-    constexpr int K_CHUNKS = HD / 8;
+    constexpr int K_STEPS = HD_TILES;                            // steps of 16 dims of the first product
+    constexpr int D_BLOCKS = (HD + 31) / 32;                     // blocks of 32 dims of the second product's result
     constexpr int BLOCK_KEYS = HD <= 128 ? 128 : 64;
     constexpr int BLOCK_TILES = BLOCK_KEYS / 16;
+    constexpr int STEPS = BLOCK_KEYS / 32;                       // steps of 32 keys in a block
     constexpr int TILE_ELEMENTS = HD * 16;                       // of keys and of values alike
     constexpr int TILE_CHUNKS = TILE_ELEMENTS / 8;               // pieces of 16 bytes
     constexpr int STAGE_ELEMENTS = 2 * BLOCK_TILES * TILE_ELEMENTS;
@@ -60,12 +74,11 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     __shared__ __align__(16) bf16 stage_even[STAGE_ELEMENTS];
     __shared__ __align__(16) bf16 stage_odd[STAGE_ELEMENTS];
 
+    const int32_t* entry = tiles + 5 * blockIdx.x;
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
-    const int col = lane % 16;
-    const int quad = lane / 16;
-
-    const int32_t* entry = tiles + 5 * blockIdx.x;
+    const int column = lane % 32;     // token of the block (B operands, results) or key / dim row (A operands)
+    const int half = lane / 32;       // which 8 of a step's 16 k-slots this lane supplies
     const int seq = entry[0];
     const int head = blockIdx.y;
     const int kv_head = head / (heads / kv_heads);
@@ -74,13 +87,13 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
 
     // Either tile's tokens and the keys any of them can see (tokens of a portion have consecutive positions);
     // an empty tile sees nothing: no key lies in its range.
-    int range_low[2], range_last[2];
+    int range_low[2], range_last[2], tile_positions[2];
 #pragma unroll
     for (int side = 0; side < 2; ++side) {
         const int count = entry[2 + 2 * side];
-        const int position = count > 0 ? positions[entry[1 + 2 * side]] : 0;
-        range_last[side] = count > 0 ? position + count - 1 : -1;
-        range_low[side] = count > 0 ? (window > 0 ? max(0, position - window + 1) : 0) : (1 << 30);
+        tile_positions[side] = count > 0 ? positions[entry[1 + 2 * side]] : 0;
+        range_last[side] = count > 0 ? tile_positions[side] + count - 1 : -1;
+        range_low[side] = count > 0 ? (window > 0 ? max(0, tile_positions[side] - window + 1) : 0) : (1 << 30);
     }
     const int group_low = min(range_low[0], range_low[1]);
     const int group_last = max(range_last[0], range_last[1]);
@@ -101,51 +114,38 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
         return (last >= range_low[0] && first <= range_last[0]) || (last >= range_low[1] && first <= range_last[1]);
     };
 
-    // This wave's two blocks of 16 columns. With two tiles in the workgroup the first block is 16 tokens of the
-    // first tile and the second 16 tokens of the second: every wave then walks the keys of both, and the waves of
-    // a compute unit stay busy together to the end of the longer walk. With one tile, waves 0 to 3 take 32
-    // consecutive tokens each.
-    const bool two_tiles = entry[2] > 0 && entry[4] > 0;
-    const int only_side = entry[2] > 0 ? 0 : 1;
-    int block_token[2], block_valid[2], block_position[2], block_last[2], block_low[2], block_last_low[2];
+    // This wave's block of 32 tokens: waves 0 to 3 take the first tile, waves 4 to 7 the second.
+    const int side = wave / 4;
+    const int count = entry[2 + 2 * side];
+    const int first_token = entry[1 + 2 * side];
+    const int tile_position = tile_positions[side];
+    const int block_first = 32 * (wave % 4);                              // in the tile
+    const int block_valid = min(32, max(0, count - block_first));
+    const int block_position = tile_position + block_first;
+    const int block_last = block_position + block_valid - 1;
+    const int block_low = window > 0 ? max(0, block_position - window + 1) : 0;        // the lowest key its first token sees
+    const int block_last_low = window > 0 ? max(0, block_last - window + 1) : 0;       // and its last token
+    const int index = min(column, max(block_valid - 1, 0));                // columns past the end repeat the last token
+    const int my_position = block_position + index;
+    const int my_low = window > 0 ? max(0, my_position - window + 1) : 0;
+
+    PFrag8 q_frag[K_STEPS];
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-        const int side = two_tiles ? c : only_side;
-        const int first = 16 * (two_tiles ? wave : 2 * wave + c);          // in the tile
-        const int count = entry[2 + 2 * side];
-        block_token[c] = entry[1 + 2 * side] + first;
-        block_valid[c] = min(16, max(0, count - first));
-        block_position[c] = (block_valid[c] > 0 ? positions[entry[1 + 2 * side]] : 0) + first;
-        block_last[c] = block_position[c] + block_valid[c] - 1;
-        block_low[c] = window > 0 ? max(0, block_position[c] - window + 1) : 0;        // the lowest key its first token sees
-        block_last_low[c] = window > 0 ? max(0, block_last[c] - window + 1) : 0;       // and its last token
+    for (int ks = 0; ks < K_STEPS; ++ks) {
+        q_frag[ks].raw = make_uint4(0, 0, 0, 0);
+        if (block_valid > 0)
+            q_frag[ks].raw = *reinterpret_cast<const uint4*>(
+                q + (static_cast<int64_t>(first_token + block_first + index) * heads + head) * HD + ks * 16 + half * 8);
     }
 
-    PFrag8 q_frag[2][K_STEPS];
-    int my_position[2], my_low[2];
+    floatx16 o_acc[D_BLOCKS];
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-        const int valid = block_valid[c];
-        const int index = min(col, max(valid - 1, 0));      // columns past the end repeat the last token
-        my_position[c] = block_position[c] + index;
-        my_low[c] = window > 0 ? max(0, my_position[c] - window + 1) : 0;
+    for (int d = 0; d < D_BLOCKS; ++d)
 #pragma unroll
-        for (int ks = 0; ks < K_STEPS; ++ks) {
-            const int dim = ks * 32 + quad * 8;
-            q_frag[c][ks].raw = make_uint4(0, 0, 0, 0);
-            if (valid > 0 && dim < HD)
-                q_frag[c][ks].raw = *reinterpret_cast<const uint4*>(
-                    q + (static_cast<int64_t>(block_token[c] + index) * heads + head) * HD + dim);
-        }
-    }
-
-    floatx4 o_acc[2][HD_TILES];
-    float running_max[2] = {-INFINITY, -INFINITY}, running_sum[2] = {0.0f, 0.0f};
-    float running_offset[2] = {0.0f, 0.0f};      // -(running maximum) in units of log 2; 0 while the maximum is -inf
-#pragma unroll
-    for (int c = 0; c < 2; ++c)
-#pragma unroll
-        for (int d = 0; d < HD_TILES; ++d) o_acc[c][d] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int i = 0; i < 16; ++i) o_acc[d][i] = 0.0f;
+    float running_max = -INFINITY;
+    float running_sum = 0.0f;         // over this lane's keys only; the two halves of the wave meet at the end
+    float running_offset = 0.0f;      // -(running maximum) in units of log 2; 0 while the maximum is -inf
 
     // Copy of one block's tiles, from the pages straight into LDS (no registers in between): a wave moves 64
     // consecutive pieces of 16 bytes of the block's key tiles as they lie in LDS, piece pass * threads + thread,
@@ -200,9 +200,9 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
             }
         }
     };
-    // A block at an end of what the workgroup's tokens see, once it lies in LDS: values at positions that no
-    // token sees may be stale memory, and the places of tiles that were not brought in hold what was there
-    // before. Both are cleared (their scores are masked where they are computed).
+    // A block at an end of what the tile's tokens see, once it lies in LDS: values at positions that no token
+    // sees may be stale memory, and the places of tiles that were not brought in hold what was there before.
+    // Both are cleared (their scores are masked where they are computed).
     auto clear_unseen = [&](int block, bf16* stage) {
 #pragma unroll
         for (int pass = 0; pass < PASSES; ++pass) {
@@ -221,121 +221,101 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
             *place = values.raw;
         }
     };
+    const int first_block = group_low / BLOCK_KEYS;
+    const int last_block = group_last / BLOCK_KEYS;
     // The wave's loads into LDS have landed (the compiler does not wait for loads that return nothing), and so
     // have everyone's; everyone is done with the stage that is written next.
     auto landed = [&](int block, bf16* stage) {
         wait_for_loads();
         __syncthreads();
-        if (block <= group_last / BLOCK_KEYS && !inside(block)) {
+        if (block <= last_block && !inside(block)) {
             clear_unseen(block, stage);
             __syncthreads();
         }
     };
+
+    // One step of 32 keys against the wave's 32 tokens. MASKED: some key of the step is hidden from some token
+    // (the causal diagonal, the window's edge, the end of the sequence).
+    // Scores stay in the product's units; p = 2^((s - max) * scale_log2) is one multiply-add and one exponent.
+    auto process_step = [&](auto masked_tag, const bf16* k_lds, const bf16* v_lds, int step, int key0) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        // S^T: row = key `column` of the step (tile column / 16, position column % 16), 8 dims (chunk 2 ks + half) per lane.
+        const bf16* k_rows = k_lds + (2 * step + column / 16) * TILE_ELEMENTS + (half * 16 + column % 16) * 8;
+        floatx16 s;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[i] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < K_STEPS; ++ks) {
+            PFrag8 k_frag;
+            k_frag.raw = *reinterpret_cast<const uint4*>(k_rows + ks * 256);
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag.v, q_frag[ks].v, s, 0, 0, 0);
+        }
+        // s[i]: key key0 + 8 (i / 4) + 4 half + i % 4, token `column`.
+        if (MASKED) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int key = key0 + 8 * (i / 4) + 4 * half + (i % 4);
+                if (key > my_position || key < my_low) s[i] = -INFINITY;
+            }
+        }
+        float tile_max = fmaxf(fmaxf(s[0], s[1]), s[2]);
+#pragma unroll
+        for (int i = 3; i < 15; i += 2) tile_max = fmaxf(fmaxf(tile_max, s[i]), s[i + 1]);
+        tile_max = fmaxf(tile_max, s[15]);
+        // Far into a prompt a step rarely holds a new maximum for any of the wave's tokens: then the two halves
+        // need not compare notes, and nothing is rescaled (the same numbers either way).
+        float rescale = 1.0f;
+        if (__any(tile_max > running_max)) {
+            tile_max = reduce_lanes_32_apart(tile_max, [](float a, float b) { return fmaxf(a, b); });
+            const float new_max = fmaxf(running_max, tile_max);
+            // A token may see nothing of a step that others see (the window's edge): its maximum stays -inf.
+            const float safe_max = (MASKED && new_max == -INFINITY) ? 0.0f : new_max;
+            running_offset = -safe_max * scale_log2;
+            // exactly 1 for a token whose maximum stays (the rounding of maximum * scale would else leave a factor
+            // of 1 +- 1e-7, and every sum would be multiplied by it)
+            rescale = new_max == running_max ? 1.0f : __builtin_amdgcn_exp2f(fmaf(running_max, scale_log2, running_offset));
+            running_max = new_max;
+        }
+        const float offset = running_offset;
+        float step_sum = 0.0f;
+        PFrag8 p_frag[2];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float p = __builtin_amdgcn_exp2f(fmaf(s[i], scale_log2, offset));
+            step_sum += p;
+            p_frag[i / 8].v[i % 8] = static_cast<__bf16>(p);
+        }
+        running_sum = running_sum * rescale + step_sum;
+        // Once the running maxima have settled, no column's sums need rescaling: one branch for the whole wave.
+        if (__any(rescale != 1.0f)) {
+#pragma unroll
+            for (int d = 0; d < D_BLOCKS; ++d) o_acc[d] *= rescale;
+        }
+        // O^T += V^T . P^T, 16 keys (one tile) a product: row = dim `column` of a block of 32 dims; the lane's 8
+        // k-slots are the keys its scores came for: positions 4 half .. + 3 and 8 + 4 half .. + 3 of the tile.
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const bf16* v_tile = v_lds + (2 * step + t) * TILE_ELEMENTS + half * 64;
+#pragma unroll
+            for (int d = 0; d < D_BLOCKS; ++d) {
+                const int dim = d * 32 + column;
+                PFrag8 v_frag;
+                v_frag.raw = make_uint4(0, 0, 0, 0);
+                if (HD % 32 == 0 || dim < HD) {
+                    const bf16* v_row = v_tile + (dim / 16) * 256 + (dim % 16) * 4;
+                    v_frag.h[0] = *reinterpret_cast<const bf16x4*>(v_row);
+                    v_frag.h[1] = *reinterpret_cast<const bf16x4*>(v_row + 128);
+                }
+                o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag.v, p_frag[t].v, o_acc[d], 0, 0, 0);
+            }
+        }
+    };
+
     auto next_seen = [&](int block) {      // the next block after this one of which something is seen
         ++block;
         while (block * BLOCK_KEYS <= group_last && !block_seen(block)) ++block;
         return block;
     };
-
-    // One pair of key tiles (32 keys) against the wave's two blocks of 16 tokens; see0 / see1: whether the block
-    // sees any of the pair. MASKED: some key of the pair is hidden from some token of a block that sees the pair
-    // (the causal diagonal, the window's edge, the end of the sequence).
-    // Scores stay in the product's units; p = 2^((s - max) * scale_log2) is one multiply-add and one exponent.
-    auto process_pair = [&](auto masked_tag, const bf16* k_lds, const bf16* v_lds, int pair, int key0, bool see0, bool see1) {
-        constexpr bool MASKED = decltype(masked_tag)::value;
-        PFrag8 k_frag[2][K_STEPS];
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int ks = 0; ks < K_STEPS; ++ks) {
-                const int piece = ks * 4 + quad;
-                k_frag[t][ks].raw = make_uint4(0, 0, 0, 0);
-                if (piece < K_CHUNKS)
-                    k_frag[t][ks].raw = *reinterpret_cast<const uint4*>(
-                        k_lds + (2 * pair + t) * TILE_ELEMENTS + piece * 128 + col * 8);
-            }
-        PFrag8 p_frag[2];
-        float rescale[2];
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            if (!(c == 0 ? see0 : see1)) {
-                p_frag[c].raw = make_uint4(0, 0, 0, 0);
-                rescale[c] = 1.0f;
-                continue;
-            }
-            float score[8];
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                floatx4 s = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-                for (int ks = 0; ks < K_STEPS; ++ks)
-                    s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_frag[t][ks].v, q_frag[c][ks].v, s, 0, 0, 0);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) score[4 * t + i] = s[i];
-            }
-            if (MASKED) {
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int key = key0 + 16 * (j / 4) + 4 * quad + (j % 4);
-                    if (key > my_position[c] || key < my_low[c]) score[j] = -INFINITY;
-                }
-            }
-            float tile_max = score[0];
-#pragma unroll
-            for (int j = 1; j < 8; ++j) tile_max = fmaxf(tile_max, score[j]);
-            // Far into a prompt a pair rarely holds a new maximum for any of the wave's tokens: then the four
-            // lanes of a token need not compare notes, and nothing is rescaled (the same numbers either way).
-            rescale[c] = 1.0f;
-            if (__any(tile_max > running_max[c])) {
-                tile_max = max_lanes_16_apart(tile_max);
-                const float new_max = fmaxf(running_max[c], tile_max);
-                // A query may see nothing of a pair that others see (the window's edge): its maximum stays -inf.
-                const float safe_max = (MASKED && new_max == -INFINITY) ? 0.0f : new_max;
-                running_offset[c] = -safe_max * scale_log2;
-                // exactly 1 for a token whose maximum stays (the rounding of maximum * scale would else leave a factor
-                // of 1 +- 1e-7, and every sum would be multiplied by it)
-                rescale[c] = new_max == running_max[c] ? 1.0f : __builtin_amdgcn_exp2f(fmaf(running_max[c], scale_log2, running_offset[c]));
-                running_max[c] = new_max;
-            }
-            const float offset = running_offset[c];
-            float tile_sum = 0.0f;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float p = __builtin_amdgcn_exp2f(fmaf(score[j], scale_log2, offset));
-                tile_sum += p;
-                p_frag[c].v[j] = static_cast<__bf16>(p);
-            }
-            tile_sum = sum_lanes_16_apart(tile_sum);
-            running_sum[c] = running_sum[c] * rescale[c] + tile_sum;
-        }
-        // Once the running maxima have settled, no column's sum needs rescaling: one branch for the whole wave.
-        if (__any(rescale[0] != 1.0f || rescale[1] != 1.0f)) {
-#pragma unroll
-            for (int c = 0; c < 2; ++c)
-#pragma unroll
-                for (int d = 0; d < HD_TILES; ++d) o_acc[c][d] *= rescale[c];
-        }
-        auto values_times_weights = [&](auto first_tag, auto second_tag) {
-#pragma unroll
-            for (int d = 0; d < HD_TILES; ++d) {
-                PFrag8 v_frag;
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-                    v_frag.h[t] = *reinterpret_cast<const bf16x4*>(
-                        v_lds + (2 * pair + t) * TILE_ELEMENTS + d * 256 + (quad * 16 + col) * 4);
-                if (decltype(first_tag)::value)
-                    o_acc[0][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_frag.v, p_frag[0].v, o_acc[0][d], 0, 0, 0);
-                if (decltype(second_tag)::value)
-                    o_acc[1][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_frag.v, p_frag[1].v, o_acc[1][d], 0, 0, 0);
-            }
-        };
-        if (see0 && see1) values_times_weights(std::true_type{}, std::true_type{});
-        else if (see0) values_times_weights(std::true_type{}, std::false_type{});
-        else values_times_weights(std::false_type{}, std::true_type{});
-    };
-
-    const int first_block = group_low / BLOCK_KEYS;
-    const int last_block = group_last / BLOCK_KEYS;
     // One block: the next one is sent for, this one is used. Called by turns with the stages exchanged.
     int block = first_block;
     int following = next_seen(first_block);
@@ -347,18 +327,17 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
         }
         const bf16* k_lds = stage;
         const bf16* v_lds = stage + HALF_CHUNKS * 8;
-#pragma unroll 1
-        for (int pair = 0; pair < BLOCK_TILES / 2; ++pair) {
-            const int key0 = block * BLOCK_KEYS + 32 * pair;
-            bool see[2], hidden = false;
+        // Unrolled: every read from LDS then has the stage's own address plus a constant, and the compiler can tell
+        // that the loads on their way into the other stage do not touch it (of an address that a loop carries along
+        // it cannot, and waits for those loads before the first read).
 #pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                see[c] = block_valid[c] > 0 && key0 <= block_last[c] && key0 + 31 >= block_low[c];
-                hidden = hidden || (see[c] && (key0 + 31 > block_position[c] || key0 < block_last_low[c]));
-            }
-            if (!see[0] && !see[1]) continue;      // nothing of this pair is visible to the wave
-            if (hidden) process_pair(std::true_type{}, k_lds, v_lds, pair, key0, see[0], see[1]);
-            else process_pair(std::false_type{}, k_lds, v_lds, pair, key0, see[0], see[1]);
+        for (int step = 0; step < STEPS; ++step) {
+            const int key0 = block * BLOCK_KEYS + 32 * step;
+            const bool see = block_valid > 0 && key0 <= block_last && key0 + 31 >= block_low;
+            if (!see) continue;      // nothing of this step is visible to the wave
+            const bool hidden = key0 + 31 > block_position || key0 < block_last_low;
+            if (hidden) process_step(std::true_type{}, k_lds, v_lds, step, key0);
+            else process_step(std::false_type{}, k_lds, v_lds, step, key0);
         }
         landed(following, next_stage);
         block = following;
@@ -373,20 +352,23 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
         if (block > last_block) break;
         walk(stage_odd, stage_even);
     }
+    running_sum = reduce_lanes_32_apart(running_sum, [](float a, float b) { return a + b; });
 
+    // o_acc[d][i]: dim 32 d + 8 (i / 4) + 4 half + i % 4 of token `column`.
+    if (column < block_valid) {
+        const float inverse = 1.0f / running_sum;
+        bf16* out_row = out + (static_cast<int64_t>(first_token + block_first + column) * heads + head) * HD;
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-        if (col < block_valid[c]) {
-            const float inverse = 1.0f / running_sum[c];
-            bf16* out_row = out + (static_cast<int64_t>(block_token[c] + col) * heads + head) * HD;
+        for (int d = 0; d < D_BLOCKS; ++d)
 #pragma unroll
-            for (int d = 0; d < HD_TILES; ++d) {
+            for (int j = 0; j < 4; ++j) {
+                const int dim = d * 32 + 8 * j + 4 * half;
+                if (HD % 32 != 0 && dim >= HD) continue;
                 bf16x4 four;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) four[i] = static_cast<__bf16>(o_acc[c][d][i] * inverse);
-                *reinterpret_cast<bf16x4*>(out_row + d * 16 + quad * 4) = four;
+                for (int i = 0; i < 4; ++i) four[i] = static_cast<__bf16>(o_acc[d][4 * j + i] * inverse);
+                *reinterpret_cast<bf16x4*>(out_row + dim) = four;
             }
-        }
     }
 }
 
@@ -394,8 +376,6 @@ template <int HD_TILES>
 static int launch_prefill(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
                           int table_width, const int32_t* tiles, int n_tiles, const int32_t* positions, void* out,
                           float scale, int window, int heads, int kv_heads, int page_size, hipStream_t stream) {
-    constexpr int HD = HD_TILES * 16;
-    constexpr int BLOCK_KEYS = HD <= 128 ? 128 : 64;
     const dim3 grid(n_tiles, heads);   // n_tiles: workgroups, of two tiles each
     paged_attention_prefill_kernel<HD_TILES><<<grid, kPrefillThreads, 0, stream>>>(
         static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), block_table,

@@ -26,16 +26,23 @@ from .spec import PartSpec
 class QueryTilePlanner:
     """The step metadata of the MFMA attention kernels (an ``engine.batch.StepPlanner``): requests that bring
     several tokens are cut into tiles of ``kernels.QUERY_TILE`` queries, which go to the prefill kernel's
-    workgroups in twos (``kernels.pair_query_tiles``: a late tile with an early one, or neighbours under a
-    window); requests that bring one token beside them are listed for the decode kernel. In a step of single
-    tokens only there is nothing to plan: the decode kernel takes every row.
+    workgroups in twos (``kernels.pair_query_tiles``); requests that bring one token beside them are listed for the
+    decode kernel. In a step of single tokens only there is nothing to plan: the decode kernel takes every row.
+
+    Which two tiles share a workgroup: a late tile of a prompt with an early one, so that all workgroups walk about
+    as many keys, where there are too few workgroups to even out by themselves; neighbours (which read nearly the
+    same keys: half the traffic) under a window, or when every compute unit gets ``CROWDED`` workgroups or more,
+    the longest first.
 
     Plan: ``tiles`` int32 [workgroups, 5]; ``single_tokens`` int32 [rows]; ``max_single_total``, the longest of
     the requests listed there."""
+    CROWDED = 4
 
-    def __init__(self, adjacent: bool):
-        self.adjacent = adjacent
-        self.key = ("paged_attention_query_tiles", adjacent)
+    def __init__(self, windowed: bool, heads: int, compute_units: int):
+        self.windowed = windowed
+        self.heads = heads
+        self.compute_units = compute_units
+        self.key = ("paged_attention_query_tiles", windowed, heads)
 
     def plan(self, host):
         counts, cu = host.counts, host.cu
@@ -45,7 +52,8 @@ class QueryTilePlanner:
         tile_list = [(index, int(cu[index]) + offset, min(kernels.QUERY_TILE, count - offset), host.starts[index] + offset)
                      for index, count in enumerate(counts) if not (mixed and count == 1)
                      for offset in range(0, count, kernels.QUERY_TILE)]
-        tiles = np.asarray(kernels.pair_query_tiles(tile_list, adjacent=self.adjacent), dtype=np.int32).reshape(-1, 5)
+        adjacent = self.windowed or len(tile_list) * self.heads >= 2 * self.CROWDED * self.compute_units
+        tiles = np.asarray(kernels.pair_query_tiles(tile_list, adjacent=adjacent), dtype=np.int32).reshape(-1, 5)
         single = np.asarray([cu[index] for index, count in enumerate(counts) if mixed and count == 1], dtype=np.int32)
         longest = max((host.totals[index] for index, count in enumerate(counts) if mixed and count == 1), default=0)
         return {"tiles": tiles, "single_tokens": single}, {"max_single_total": longest}
@@ -69,7 +77,8 @@ class PagedAttention(Mixer):
             raise ValueError("num_heads must divide into num_kv_heads groups")
         position = p.get("position")
         self.position = build_part("position", position, runtime) if position is not None else None
-        self.planner = QueryTilePlanner(adjacent=bool(self.window))
+        units = torch.cuda.get_device_properties(runtime.device).multi_processor_count if runtime.device.type == "cuda" else 256
+        self.planner = QueryTilePlanner(bool(self.window), self.heads, units)
         self.qkv_weight: Optional[torch.Tensor] = None
         self.qkv_bias_vector: Optional[torch.Tensor] = None
         self.o_weight: Optional[torch.Tensor] = None
