@@ -54,6 +54,13 @@ __device__ inline float reduce_lanes_32_apart(float value, Op op) {
     return op(__builtin_bit_cast(float, low), __builtin_bit_cast(float, high));
 }
 
+#ifdef MLL_PREFILL_TIMING
+__device__ unsigned long long prefill_cycles[6];
+#define TICK(slot) do { const long long now_ = clock64(); spent[slot] += now_ - last_tick; last_tick = now_; } while (0)
+#else
+#define TICK(slot)
+#endif
+
 template <int HD_TILES>
 __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
@@ -234,34 +241,47 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
         }
     };
 
-    // One step of 32 keys against the wave's 32 tokens. MASKED: some key of the step is hidden from some token
-    // (the causal diagonal, the window's edge, the end of the sequence).
+    // HALVES (1 or 2) runs of 32 keys against the wave's 32 tokens; the runs are numbered within the block. Two
+    // runs at once share one maximum, one exchange between the halves of the wave and one look at whether anything
+    // must be rescaled, and their two chains of products hide each other's latency. MASKED: some key is hidden
+    // from some token (the causal diagonal, the window's edge, the end of the sequence).
     // Scores stay in the product's units; p = 2^((s - max) * scale_log2) is one multiply-add and one exponent.
-    auto process_step = [&](auto masked_tag, const bf16* k_lds, const bf16* v_lds, int step, int key0) {
+    auto process_keys = [&](auto masked_tag, auto halves_tag, const bf16* k_lds, const bf16* v_lds, int first_run, int key0) {
         constexpr bool MASKED = decltype(masked_tag)::value;
-        // S^T: row = key `column` of the step (tile column / 16, position column % 16), 8 dims (chunk 2 ks + half) per lane.
-        const bf16* k_rows = k_lds + (2 * step + column / 16) * TILE_ELEMENTS + (half * 16 + column % 16) * 8;
-        floatx16 s;
+        constexpr int HALVES = decltype(halves_tag)::value;
+        // S^T: row = key `column` of the run (tile column / 16, position column % 16), 8 dims (chunk 2 ks + half) per lane.
+        const bf16* k_rows = k_lds + (2 * first_run + column / 16) * TILE_ELEMENTS + (half * 16 + column % 16) * 8;
+        floatx16 s[HALVES];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[i] = 0.0f;
+        for (int r = 0; r < HALVES; ++r)
 #pragma unroll
-        for (int ks = 0; ks < K_STEPS; ++ks) {
-            PFrag8 k_frag;
-            k_frag.raw = *reinterpret_cast<const uint4*>(k_rows + ks * 256);
-            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag.v, q_frag[ks].v, s, 0, 0, 0);
-        }
-        // s[i]: key key0 + 8 (i / 4) + 4 half + i % 4, token `column`.
+            for (int i = 0; i < 16; ++i) s[r][i] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < K_STEPS; ++ks)
+#pragma unroll
+            for (int r = 0; r < HALVES; ++r) {
+                PFrag8 k_frag;
+                k_frag.raw = *reinterpret_cast<const uint4*>(k_rows + r * 2 * TILE_ELEMENTS + ks * 256);
+                s[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag.v, q_frag[ks].v, s[r], 0, 0, 0);
+            }
+        // s[r][i]: key key0 + 32 r + 8 (i / 4) + 4 half + i % 4, token `column`.
         if (MASKED) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int key = key0 + 8 * (i / 4) + 4 * half + (i % 4);
-                if (key > my_position || key < my_low) s[i] = -INFINITY;
-            }
-        }
-        float tile_max = fmaxf(fmaxf(s[0], s[1]), s[2]);
+            for (int r = 0; r < HALVES; ++r)
 #pragma unroll
-        for (int i = 3; i < 15; i += 2) tile_max = fmaxf(fmaxf(tile_max, s[i]), s[i + 1]);
-        tile_max = fmaxf(tile_max, s[15]);
+                for (int i = 0; i < 16; ++i) {
+                    const int key = key0 + 32 * r + 8 * (i / 4) + 4 * half + (i % 4);
+                    if (key > my_position || key < my_low) s[r][i] = -INFINITY;
+                }
+        }
+        float tile_max = fmaxf(fmaxf(s[0][0], s[0][1]), s[0][2]);
+#pragma unroll
+        for (int i = 3; i < 15; i += 2) tile_max = fmaxf(fmaxf(tile_max, s[0][i]), s[0][i + 1]);
+        tile_max = fmaxf(tile_max, s[0][15]);
+#pragma unroll
+        for (int r = 1; r < HALVES; ++r)
+#pragma unroll
+            for (int i = 0; i < 16; i += 2) tile_max = fmaxf(fmaxf(tile_max, s[r][i]), s[r][i + 1]);
         // Far into a prompt a step rarely holds a new maximum for any of the wave's tokens: then the two halves
         // need not compare notes, and nothing is rescaled (the same numbers either way).
         float rescale = 1.0f;
@@ -278,13 +298,15 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
         }
         const float offset = running_offset;
         float step_sum = 0.0f;
-        PFrag8 p_frag[2];
+        PFrag8 p_frag[2 * HALVES];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const float p = __builtin_amdgcn_exp2f(fmaf(s[i], scale_log2, offset));
-            step_sum += p;
-            p_frag[i / 8].v[i % 8] = static_cast<__bf16>(p);
-        }
+        for (int r = 0; r < HALVES; ++r)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const float p = __builtin_amdgcn_exp2f(fmaf(s[r][i], scale_log2, offset));
+                step_sum += p;
+                p_frag[2 * r + i / 8].v[i % 8] = static_cast<__bf16>(p);
+            }
         running_sum = running_sum * rescale + step_sum;
         // Once the running maxima have settled, no column's sums need rescaling: one branch for the whole wave.
         if (__any(rescale != 1.0f)) {
@@ -293,22 +315,20 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
         }
         // O^T += V^T . P^T, 16 keys (one tile) a product: row = dim `column` of a block of 32 dims; the lane's 8
         // k-slots are the keys its scores came for: positions 4 half .. + 3 and 8 + 4 half .. + 3 of the tile.
+        const bf16* v_rows = v_lds + 2 * first_run * TILE_ELEMENTS + (column / 16) * 256 + (column % 16) * 4 + half * 64;
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const bf16* v_tile = v_lds + (2 * step + t) * TILE_ELEMENTS + half * 64;
+        for (int t = 0; t < 2 * HALVES; ++t)
 #pragma unroll
             for (int d = 0; d < D_BLOCKS; ++d) {
-                const int dim = d * 32 + column;
                 PFrag8 v_frag;
                 v_frag.raw = make_uint4(0, 0, 0, 0);
-                if (HD % 32 == 0 || dim < HD) {
-                    const bf16* v_row = v_tile + (dim / 16) * 256 + (dim % 16) * 4;
+                if (HD % 32 == 0 || d * 32 + column < HD) {
+                    const bf16* v_row = v_rows + t * TILE_ELEMENTS + d * 512;
                     v_frag.h[0] = *reinterpret_cast<const bf16x4*>(v_row);
                     v_frag.h[1] = *reinterpret_cast<const bf16x4*>(v_row + 128);
                 }
                 o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag.v, p_frag[t].v, o_acc[d], 0, 0, 0);
             }
-        }
     };
 
     auto next_seen = [&](int block) {      // the next block after this one of which something is seen
@@ -319,7 +339,12 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     // One block: the next one is sent for, this one is used. Called by turns with the stages exchanged.
     int block = first_block;
     int following = next_seen(first_block);
+#ifdef MLL_PREFILL_TIMING
+    long long spent[6] = {0, 0, 0, 0, 0, 0};
+    long long last_tick = clock64();
+#endif
     auto walk = [&](const bf16* stage, bf16* next_stage) {
+        TICK(4);
         if (following <= last_block) {
             fetch(following, next_stage);
             const int after = next_seen(following);
@@ -327,19 +352,38 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
         }
         const bf16* k_lds = stage;
         const bf16* v_lds = stage + HALF_CHUNKS * 8;
+        TICK(0);
         // Unrolled: every read from LDS then has the stage's own address plus a constant, and the compiler can tell
         // that the loads on their way into the other stage do not touch it (of an address that a loop carries along
         // it cannot, and waits for those loads before the first read).
 #pragma unroll
-        for (int step = 0; step < STEPS; ++step) {
-            const int key0 = block * BLOCK_KEYS + 32 * step;
-            const bool see = block_valid > 0 && key0 <= block_last && key0 + 31 >= block_low;
-            if (!see) continue;      // nothing of this step is visible to the wave
-            const bool hidden = key0 + 31 > block_position || key0 < block_last_low;
-            if (hidden) process_step(std::true_type{}, k_lds, v_lds, step, key0);
-            else process_step(std::false_type{}, k_lds, v_lds, step, key0);
+        for (int pair = 0; pair < STEPS / 2; ++pair) {
+            const int key0 = block * BLOCK_KEYS + 64 * pair;
+            bool see[2], hidden[2];
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                see[r] = block_valid > 0 && key0 + 32 * r <= block_last && key0 + 32 * r + 31 >= block_low;
+                hidden[r] = key0 + 32 * r + 31 > block_position || key0 + 32 * r < block_last_low;
+            }
+            if (see[0] && see[1] && !hidden[0] && !hidden[1]) {
+                process_keys(std::false_type{}, std::integral_constant<int, 2>{}, k_lds, v_lds, 2 * pair, key0);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 2; ++r) {
+                    if (!see[r]) continue;      // nothing of this run is visible to the wave
+                    if (hidden[r]) process_keys(std::true_type{}, std::integral_constant<int, 1>{}, k_lds, v_lds, 2 * pair + r, key0 + 32 * r);
+                    else process_keys(std::false_type{}, std::integral_constant<int, 1>{}, k_lds, v_lds, 2 * pair + r, key0 + 32 * r);
+                }
+            }
         }
+        TICK(1);
+        wait_for_loads();
+        TICK(2);
         landed(following, next_stage);
+        TICK(3);
+#ifdef MLL_PREFILL_TIMING
+        spent[5] += 1;
+#endif
         block = following;
         following = next_seen(block);
     };
@@ -353,6 +397,10 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
         walk(stage_odd, stage_even);
     }
     running_sum = reduce_lanes_32_apart(running_sum, [](float a, float b) { return a + b; });
+#ifdef MLL_PREFILL_TIMING
+    if (lane == 0 && block_valid > 0 && wave < 4)
+        for (int slot = 0; slot < 6; ++slot) atomicAdd(&prefill_cycles[slot], static_cast<unsigned long long>(spent[slot]));
+#endif
 
     // o_acc[d][i]: dim 32 d + 8 (i / 4) + 4 half + i % 4 of token `column`.
     if (column < block_valid) {
@@ -388,6 +436,17 @@ static int launch_prefill(const void* q, const void* k_cache, const void* v_cach
 using namespace mll;
 
 extern "C" int mll_paged_attention_prefill_tile() { return kPrefillTile; }
+
+#ifdef MLL_PREFILL_TIMING
+extern "C" int mll_prefill_timing(long long* out) {
+    unsigned long long host[6];
+    (void)hipMemcpyFromSymbol(host, HIP_SYMBOL(prefill_cycles), sizeof(host));
+    for (int i = 0; i < 6; ++i) out[i] = static_cast<long long>(host[i]);
+    unsigned long long zero[6] = {0, 0, 0, 0, 0, 0};
+    (void)hipMemcpyToSymbol(HIP_SYMBOL(prefill_cycles), zero, sizeof(zero));
+    return 0;
+}
+#endif
 
 
 extern "C" int mll_paged_attention_prefill(const void* q, const void* k_cache, const void* v_cache,
