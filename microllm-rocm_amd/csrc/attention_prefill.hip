@@ -170,9 +170,18 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     const int wave_chunk = __builtin_amdgcn_readfirstlane(wave) * kWave;      // the wave's first piece of pass 0
     auto tile_of = [&](int pass) { return (pass * kPrefillThreads + wave_chunk + (UNIFORM ? 0 : lane)) / TILE_CHUNKS; };   // in the block
     auto piece_of = [&](int pass) { return (pass * kPrefillThreads + wave_chunk + (UNIFORM ? 0 : lane)) % TILE_CHUNKS + (UNIFORM ? lane : 0); };
+    constexpr bool FULL_PASSES = HALF_CHUNKS % kPrefillThreads == 0;      // every pass of every wave lies within the block
     auto wanted = [&](int block, int pass) {      // whether the tile is brought in: some token sees some of it
         const int tile_key = block * BLOCK_KEYS + 16 * tile_of(pass);
-        return tile_of(pass) < BLOCK_TILES && tile_key <= group_last && (inside(block) || tile_seen(tile_key));
+        return (FULL_PASSES || tile_of(pass) < BLOCK_TILES) && tile_key <= group_last && (inside(block) || tile_seen(tile_key));
+    };
+    // Pages mostly hold a power of two of tiles (often one): then the page of a tile is a shift, else a division.
+    // The choice is made once per block, not per tile.
+    auto page_index = [&](auto shift_tag, int tile_index) {
+        return decltype(shift_tag)::value ? tile_index >> page_shift : tile_index / tiles_per_page;
+    };
+    auto tile_in_its_page = [&](auto shift_tag, int tile_index) {
+        return decltype(shift_tag)::value ? tile_index & (tiles_per_page - 1) : tile_index % tiles_per_page;
     };
     // The pages of a block's tiles are looked up one block ahead of the tiles themselves, so that no load waits
     // for another. The look-up is a load of the vector unit also where the whole wave asks for one entry: those
@@ -181,20 +190,24 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     int pages[PASSES];
     int no_lane = 0;
     asm volatile("v_mov_b32 %0, 0" : "=v"(no_lane));      // zero, but the compiler cannot tell: keeps the address per lane
-    auto look_up = [&](int block) {
+    auto look_up_with = [&](auto shift_tag, int block) {
+        const bool whole = FULL_PASSES && inside(block);      // the usual case: every tile of the block, no questions
 #pragma unroll
         for (int pass = 0; pass < PASSES; ++pass) {
             const int tile_index = block * BLOCK_TILES + tile_of(pass);
             pages[pass] = -1;
-            if (wanted(block, pass))
-                pages[pass] = table[(page_shift >= 0 ? tile_index >> page_shift : tile_index / tiles_per_page) + no_lane];
+            if (whole || wanted(block, pass)) pages[pass] = table[page_index(shift_tag, tile_index) + no_lane];
         }
     };
-    auto fetch = [&](int block, bf16* stage) {      // after look_up(block)
+    auto look_up = [&](int block) {
+        if (page_shift >= 0) look_up_with(std::true_type{}, block);
+        else look_up_with(std::false_type{}, block);
+    };
+    auto fetch_with = [&](auto shift_tag, int block, bf16* stage) {      // after look_up(block)
 #pragma unroll
         for (int pass = 0; pass < PASSES; ++pass) {
             const int tile_index = block * BLOCK_TILES + tile_of(pass);
-            const int tile_in_page = page_shift >= 0 ? tile_index & (tiles_per_page - 1) : tile_index % tiles_per_page;
+            const int tile_in_page = tile_in_its_page(shift_tag, tile_index);
             const int page = UNIFORM ? __builtin_amdgcn_readfirstlane(pages[pass]) : pages[pass];
             if (page >= 0) {
                 const int64_t tile_start = page * page_elements + head_elements + tile_in_page * TILE_ELEMENTS;
@@ -206,6 +219,10 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
                 __builtin_amdgcn_global_load_lds(value_piece, value_place, 16, 0, 0);
             }
         }
+    };
+    auto fetch = [&](int block, bf16* stage) {
+        if (page_shift >= 0) fetch_with(std::true_type{}, block, stage);
+        else fetch_with(std::false_type{}, block, stage);
     };
     // A block at an end of what the tile's tokens see, once it lies in LDS: values at positions that no token
     // sees may be stale memory, and the places of tiles that were not brought in hold what was there before.
@@ -256,14 +273,25 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
         for (int r = 0; r < HALVES; ++r)
 #pragma unroll
             for (int i = 0; i < 16; ++i) s[r][i] = 0.0f;
+        // The keys' operands are read kAhead products ahead of their use (the runs by turns, so that two chains of
+        // products are under way), and the compiler is told to keep reads and products in this order: left to
+        // itself it reads each operand right before its product and waits for it.
+        constexpr int PRODUCTS = HALVES * K_STEPS;
+        constexpr int kAhead = PRODUCTS < 4 ? PRODUCTS : 4;
+        PFrag8 k_frag[PRODUCTS];
+        auto read_keys = [&](int j) {
+            k_frag[j].raw = *reinterpret_cast<const uint4*>(k_rows + (j % HALVES) * 2 * TILE_ELEMENTS + (j / HALVES) * 256);
+        };
 #pragma unroll
-        for (int ks = 0; ks < K_STEPS; ++ks)
+        for (int j = 0; j < kAhead; ++j) read_keys(j);
+        __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
 #pragma unroll
-            for (int r = 0; r < HALVES; ++r) {
-                PFrag8 k_frag;
-                k_frag.raw = *reinterpret_cast<const uint4*>(k_rows + r * 2 * TILE_ELEMENTS + ks * 256);
-                s[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag.v, q_frag[ks].v, s[r], 0, 0, 0);
-            }
+        for (int j = 0; j < PRODUCTS; ++j) {
+            if (j + kAhead < PRODUCTS) read_keys(j + kAhead);
+            s[j % HALVES] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag[j].v, q_frag[j / HALVES].v, s[j % HALVES], 0, 0, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (j + kAhead < PRODUCTS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
         // s[r][i]: key key0 + 32 r + 8 (i / 4) + 4 half + i % 4, token `column`.
         if (MASKED) {
 #pragma unroll
