@@ -44,6 +44,7 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
     __shared__ float l_shared[kSlots][16];
 
     const int token = token_ids ? token_ids[blockIdx.x] : blockIdx.x;   // a step may give the kernel some of its tokens only
+    if (token < 0) return;      // an entry that only pads the list to a fixed length
     const int group = heads / kv_heads;
     const int chunks = (group + 15) / 16;
     const int kv_head = blockIdx.y / chunks;
@@ -270,6 +271,7 @@ __global__ void paged_attention_join_kernel(const float* __restrict__ part_o, co
                                             const int32_t* __restrict__ token_ids, bf16* __restrict__ out, int heads,
                                             int head_dim, int n_splits) {
     const int token = token_ids ? token_ids[blockIdx.x / heads] : blockIdx.x / heads;
+    if (token < 0) return;      // an entry that only pads the list to a fixed length
     const int64_t row = static_cast<int64_t>(token) * heads + blockIdx.x % heads;
     const int64_t part_row = blockIdx.x;
     // Eight splits at a time: their loads are asked for together, then used in the order of the splits.

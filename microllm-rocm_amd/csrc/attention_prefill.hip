@@ -82,6 +82,7 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     __shared__ __align__(16) bf16 stage_odd[STAGE_ELEMENTS];
 
     const int32_t* entry = tiles + 5 * blockIdx.x;
+    if (entry[2] <= 0 && entry[4] <= 0) return;      // an entry that only pads the list to a fixed length
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
     const int column = lane % 32;     // token of the block (B operands, results) or key / dim row (A operands)

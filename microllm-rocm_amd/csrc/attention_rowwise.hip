@@ -27,6 +27,7 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_kernel(
     const int lane = threadIdx.x;
     const int kv_head = head / (heads / kv_heads);
     const int seq = seq_of_token[token];
+    if (seq < 0) return;      // a row that only pads the step to a fixed shape: its output stays as it is
     const int position = positions[token];
     const int low = window > 0 ? max(0, position - window + 1) : 0;
     const int32_t* table = block_table + static_cast<int64_t>(seq) * table_width;

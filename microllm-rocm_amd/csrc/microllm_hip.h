@@ -53,6 +53,8 @@ int mll_qkv_rope_store(const void* qkv, int in_dtype, int n_partials, int64_t pa
 // Key j is visible to a query at position p iff j <= p and (window <= 0 or p - j < window).
 // block_table[seq, j / page_size] gives the page of key j. Reduction order depends only on
 // (p, window), so the result does not depend on how tokens were cut into steps.
+// A token whose seq_of_token is negative is skipped and its output row left as it is (a row that pads a step to
+// a fixed shape).
 int mll_paged_attention_rowwise(const void* q, int dtype, const void* k_cache, const void* v_cache,
                                 const int32_t* block_table, int table_width,
                                 const int32_t* seq_of_token, const int32_t* positions, void* out,
@@ -64,6 +66,7 @@ int mll_paged_attention_rowwise(const void* q, int dtype, const void* k_cache, c
 // workgroup, (request index; first token in the flat list and number of tokens of the first tile; the same of the
 // second, whose number may be 0); a tile never spans two requests and its tokens have consecutive positions.
 // Workgroups take as long as the keys of both tiles together: pair a tile late in a prompt with an early one.
+// An entry whose tiles are both empty is skipped (padding of the list to a fixed length).
 int mll_paged_attention_prefill(const void* q, const void* k_cache, const void* v_cache,
                                 const int32_t* block_table, int table_width, const int32_t* tiles,
                                 int n_tiles, const int32_t* positions, void* out, float scale, int window,

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 from types import SimpleNamespace
-from typing import Any, Dict, Hashable, List, Optional, Sequence, Tuple
+from typing import Any, Dict, Hashable, List, Mapping, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -52,6 +52,43 @@ class HostStep:
         return self.n_tokens == self.n_seqs
 
 
+PADDING = -1     # request of a token, or slot of its key and value, where the row only pads a step to a fixed shape
+
+
+@dataclass
+class HostBatch:
+    """A step prepared on the host (``BatchBuilder.prepare``): its arrays and its planners' plans, not yet copied."""
+    step: HostStep
+    tokens: np.ndarray
+    positions: np.ndarray
+    seq_of_token: np.ndarray
+    starts_array: np.ndarray
+    totals_array: np.ndarray
+    slots: np.ndarray
+    want_rows: np.ndarray
+    blocks_needed: int
+    plans: list          # (planner, arrays, values)
+
+    def planned_rows(self) -> Dict[Tuple[Hashable, str], int]:
+        return {(planner.key, name): int(array.shape[0]) for planner, arrays, _ in self.plans for name, array in arrays.items()}
+
+
+@dataclass(frozen=True)
+class FixedShape:
+    """The shape a step is padded to so that it can be replayed from a graph: rows of tokens, of requests and of
+    wanted logits, the block tables' width and the rows of every planner's arrays. Padding rows hold token 0 at
+    position 0 of request ``PADDING`` with slot ``PADDING`` (nothing is stored for them and attention passes them
+    over); padding requests hold no tokens; a planner pads its arrays with the values it names in ``padding``."""
+    tokens: int
+    requests: int
+    wanted: int
+    width: int
+    planned: Mapping[Tuple[Hashable, str], int]
+
+    def key(self) -> tuple:
+        return (self.tokens, self.requests, self.wanted, self.width, tuple(sorted(self.planned.items(), key=repr)))
+
+
 class StepPlanner:
     """What a part gives the engine if its kernels need metadata of their own for a step.
 
@@ -60,6 +97,7 @@ class StepPlanner:
     equal ``key`` share one plan a step. For a step in which every request brings one token the arrays' sizes may
     depend on the number of requests alone (such steps are replayed from graphs at fixed addresses)."""
     key: Hashable = None
+    padding: Dict[str, int] = {}      # array name -> the value of rows that pad it to a fixed number of rows
 
     def plan(self, host: HostStep) -> Tuple[Dict[str, np.ndarray], Dict[str, Any]]:
         raise NotImplementedError
@@ -86,6 +124,7 @@ class StepContext:
     max_total: int = 0
     planned_total: int = 0      # the longest request this step's launch shapes are planned for (>= max_total)
     host: Optional[HostStep] = None
+    fixed: bool = False         # the step was padded to a fixed shape: n_tokens and n_seqs count the padding too
     # the plans of the parts' planners (key: the planner's): device arrays and host values as attributes
     planned: Dict[Hashable, SimpleNamespace] = field(default_factory=dict)
     # what a part computes once for the step and its likes in other layers take from here (key: the part's choice)
@@ -146,6 +185,14 @@ class BatchBuilder:
 
     def build(self, requests: Sequence[RequestCache], token_lists: Sequence[Sequence[int]],
               wants: Sequence[Sequence[int]], fixed_width: Optional[int] = None) -> StepContext:
+        """The step's metadata on the device; with ``fixed_width`` every block table has that many columns."""
+        return self.upload(self.prepare(requests, token_lists, wants), fixed_width=fixed_width)
+
+    def prepare(self, requests: Sequence[RequestCache], token_lists: Sequence[Sequence[int]],
+                wants: Sequence[Sequence[int]]) -> "HostBatch":
+        """Everything about the step that is worked out on the host, the planners' plans included; nothing is
+        copied yet. Whoever wants the step in a fixed shape reads the sizes here, chooses the shape (``FixedShape``)
+        and hands both to ``upload``, of this builder or of another that knows the same planners."""
         page_size = self.cache.page_size
         n_seqs = len(requests)
         counts = [len(tokens) for tokens in token_lists]
@@ -173,35 +220,68 @@ class BatchBuilder:
         else:
             want_rows = np.asarray([cu[index] + place for index, want in enumerate(wants) for place in want],
                                    dtype=np.int32)
-        tables, mappings, widths = [], [], []
         blocks_needed = int((int(totals_array.max()) + page_size - 1) // page_size) if n_seqs else 1
+        host_step = HostStep(n_tokens=n_tokens, n_seqs=n_seqs, page_size=page_size, counts=counts, starts=starts,
+                             totals=totals, cu=cu)
+        plans = [(planner, *planner.plan(host_step)) for planner in self.planners]
+        return HostBatch(host_step, tokens, positions, seq_of_token, starts_array, totals_array, slots, want_rows,
+                         max(1, blocks_needed), plans)
+
+    def upload(self, batch: "HostBatch", fixed_width: Optional[int] = None,
+               fixed: Optional["FixedShape"] = None) -> StepContext:
+        """Pack the prepared step into the staging buffer and copy it to the device. With ``fixed`` every array is
+        padded to that shape (see ``FixedShape``), so that the packed buffer's layout depends on the shape alone."""
+        step = batch.step
+        page_size, n_seqs, n_tokens = step.page_size, step.n_seqs, step.n_tokens
+        if fixed is not None:
+            fixed_width = fixed.width
+            if n_tokens > fixed.tokens or n_seqs > fixed.requests or batch.want_rows.size > fixed.wanted:
+                raise ValueError("the step is larger than the fixed shape")
+        rows_tokens = fixed.tokens if fixed is not None else n_tokens
+        rows_seqs = fixed.requests if fixed is not None else n_seqs
+
+        def padded(array: np.ndarray, rows: int, fill: int) -> np.ndarray:
+            if array.shape[0] == rows:
+                return array
+            out = np.full((rows,) + array.shape[1:], fill, dtype=np.int32)
+            out[:array.shape[0]] = array
+            return out
+
+        tokens = padded(batch.tokens, rows_tokens, 0)
+        positions = padded(batch.positions, rows_tokens, 0)
+        seq_of_token = padded(batch.seq_of_token, rows_tokens, PADDING)
+        cu = padded(step.cu, rows_seqs + 1, n_tokens)
+        starts_array = padded(batch.starts_array, rows_seqs, 0)
+        totals_array = padded(batch.totals_array, rows_seqs, 0)
+        slots = padded(batch.slots, rows_seqs, 0)
+        want_rows = padded(batch.want_rows, fixed.wanted, 0) if fixed is not None else batch.want_rows
+        tables, mappings, widths = [], [], []
         for group in self.cache.groups:
-            width = max(1, blocks_needed)
+            width = batch.blocks_needed
             if fixed_width is not None:
                 if width > fixed_width:
                     raise ValueError("a block table is wider than the fixed width")
                 width = fixed_width
-            rows = group.tables[slots]                      # [requests, most blocks a request can hold]
+            rows = group.tables[batch.slots]                      # [requests, most blocks a request can hold]
             if width <= rows.shape[1]:
                 table = np.ascontiguousarray(rows[:, :width])
             else:
                 table = np.full((n_seqs, width), RELEASED, dtype=np.int32)
                 table[:, :rows.shape[1]] = rows
-            mapping = table[seq_of_token, positions // page_size] * page_size + positions % page_size
-            tables.append(table)
-            mappings.append(mapping.astype(np.int32, copy=False))
+            mapping = table[batch.seq_of_token, batch.positions // page_size] * page_size + batch.positions % page_size
+            tables.append(padded(table, rows_seqs, RELEASED))
+            mappings.append(padded(mapping.astype(np.int32, copy=False), rows_tokens, PADDING))
             widths.append(width)
-        host_step = HostStep(n_tokens=n_tokens, n_seqs=n_seqs, page_size=page_size, counts=counts, starts=starts,
-                             totals=totals, cu=cu)
         pieces = [tokens, positions, seq_of_token, cu, starts_array, totals_array, slots, want_rows]
         for table, mapping in zip(tables, mappings):
             pieces += [table.reshape(-1), mapping]
         plans = []          # (key, host values, {name: (piece index, shape)})
-        for planner in self.planners:
-            arrays, values = planner.plan(host_step)
+        for planner, arrays, values in batch.plans:
             places = {}
             for name, array in arrays.items():
                 array = np.ascontiguousarray(array, dtype=np.int32)
+                if fixed is not None:
+                    array = padded(array, fixed.planned[(planner.key, name)], planner.padding[name])
                 places[name] = (len(pieces), array.shape)
                 pieces.append(array.reshape(-1))
             plans.append((planner.key, values, places))
@@ -223,15 +303,16 @@ class BatchBuilder:
 
         paged = []
         for g, group in enumerate(self.cache.groups):
-            paged.append(PagedView(piece_at(8 + 2 * g, (n_seqs, widths[g])), piece_at(9 + 2 * g),
+            paged.append(PagedView(piece_at(8 + 2 * g, (rows_seqs, widths[g])), piece_at(9 + 2 * g),
                                    page_size, widths[g]))
         planned = {key: SimpleNamespace(**values, **{name: piece_at(index, shape) for name, (index, shape) in places.items()})
                    for key, values, places in plans}
-        longest = max(totals) if totals else 0
+        longest = max(step.totals) if step.totals else 0
         return StepContext(
-            n_tokens=n_tokens, n_seqs=n_seqs, tokens=piece_at(0), positions=piece_at(1), seq_of_token=piece_at(2),
+            n_tokens=rows_tokens, n_seqs=rows_seqs, tokens=piece_at(0), positions=piece_at(1), seq_of_token=piece_at(2),
             cu_tokens=piece_at(3), seq_start=piece_at(4), seq_total=piece_at(5), slots=piece_at(6),
             want_rows=piece_at(7) if want_rows.size else None, paged=paged,
-            starts=starts, counts=counts, host_slots=slots.tolist(),
-            max_count=max(counts) if counts else 0, max_total=longest,
-            planned_total=longest if fixed_width is None else fixed_width * page_size, host=host_step, planned=planned)
+            starts=step.starts, counts=step.counts, host_slots=batch.slots.tolist(),
+            max_count=max(step.counts) if step.counts else 0, max_total=longest,
+            planned_total=longest if fixed_width is None else fixed_width * page_size, host=step, planned=planned,
+            fixed=fixed is not None)

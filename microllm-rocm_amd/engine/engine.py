@@ -21,7 +21,7 @@ from ..config.registry import architecture_named, load_config
 from ..ops import kernels, library
 from ..parts import Model, ModelSpec, Runtime
 from ..weights import load_folder, place_all, random_tensors
-from .batch import BatchBuilder, StepContext, StepEntry
+from .batch import BatchBuilder, FixedShape, HostBatch, StepContext, StepEntry
 
 _DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": torch.bfloat16, "bf16": torch.bfloat16}
 
@@ -38,7 +38,21 @@ def parse_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
 
 MAX_GRAPH_REQUESTS = 256
 MIN_GRAPH_WIDTH = 16
-MAX_GRAPHS = 48     # captured decode steps kept at a time; the one replayed longest ago goes first
+MAX_GRAPHS = 48     # captured steps kept at a time; the one replayed longest ago goes first
+MAX_GRAPH_TOKENS = 4096     # mixed steps of more tokens run eagerly: their launches no longer cost more than their kernels
+MAX_GRAPH_WANTED = 256
+SHAPE_SEEN_TWICE = 2        # a mixed step's shape is captured when it comes for the second time
+
+
+def _power_of_two(value: int, least: int = 1) -> int:
+    return max(least, 1 << (max(value, 1) - 1).bit_length())
+
+
+def _token_rows(tokens: int) -> int:
+    """Rows a mixed step of ``tokens`` tokens is padded to: steps of 16 up to 128, of 64 up to 1024, then of 256
+    (at most an eighth more rows than tokens from 128 on)."""
+    step = 16 if tokens <= 128 else (64 if tokens <= 1024 else 256)
+    return -(-tokens // step) * step
 
 
 class _DecodeGraph:
@@ -72,7 +86,8 @@ class Engine:
                  device: Union[str, torch.device] = "cuda:0", page_size: int = 16,
                  max_tokens: Optional[int] = None, num_pages: Optional[int] = None, max_requests: int = 64,
                  tensors_placed: bool = False, use_graphs: bool = True, weight_copies: str = "auto",
-                 consume_tensors: bool = False, tune_library: bool = False, max_portion: Optional[int] = None):
+                 consume_tensors: bool = False, tune_library: bool = False, max_portion: Optional[int] = None,
+                 graph_mixed_steps: bool = True):
         """``max_portion``: the most tokens a step brings one request, if the caller keeps to one (a scheduler's
         prefill chunk): cache groups with a window then get pools no larger than their requests can fill.
         ``weight_copies``: a bfloat16 weight is kept ``"both"`` as stored (for the library's product of steps
@@ -128,6 +143,12 @@ class Engine:
         self._graph_pool = None
         self.graph_replays = 0
         self.graphs_captured = 0
+        # Steps that mix portions of prompts with single tokens are padded to one of a few shapes and replayed
+        # from graphs too, once a shape has come twice: for small models such a step's launches cost the host
+        # more time than its kernels cost the GPU.
+        self.graph_mixed_steps = graph_mixed_steps
+        self._shape_seen: Dict[tuple, int] = {}
+        self.mixed_graph_replays = 0
 
     def _two_copies_fit(self, model: Model, decls, num_pages: int, page_size: int, max_requests: int,
                         max_portion: Optional[int]) -> bool:
@@ -204,18 +225,7 @@ class Engine:
             ctx = state.builder.build(requests, [entry.tokens for entry in entries], every_row, fixed_width=width)
         self._last_graph = state
         if state.graph is None:
-            # Once eagerly (libraries create their handles and workspaces), then the capture. The step writes
-            # the same keys and values to the same slots each time, so running it twice changes nothing.
-            self.model.forward(ctx, self._bindings, ctx.want_rows)
-            torch.cuda.synchronize(self.device)
-            ctx.memo.clear()     # what the parts computed once for the step is computed inside the graph too
-            if self._graph_pool is None:
-                self._graph_pool = torch.cuda.graph_pool_handle()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
-                state.logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
-            state.graph = graph
-            self.graphs_captured += 1
+            self._capture(state, ctx)
         state.graph.replay()
         self.graph_replays += 1
         wanted = [index for index, entry in enumerate(entries) if len(entry.want) > 0]
@@ -224,6 +234,60 @@ class Engine:
         if len(wanted) == n:
             return state.logits if self._borrow else state.logits.clone()
         return state.logits[torch.tensor(wanted, device=self.device)]
+
+    # ---- mixed steps from graphs -----------------------------------------------------------
+    def _fixed_shape(self, batch: HostBatch) -> Optional[FixedShape]:
+        """The shape this step is padded to for a graph, or None if it runs eagerly: too large, or a shape that
+        has not come before (most shapes of a changing workload come once)."""
+        step = batch.step
+        wanted = int(batch.want_rows.size)
+        if step.n_tokens > MAX_GRAPH_TOKENS or step.n_seqs > MAX_GRAPH_REQUESTS or wanted > MAX_GRAPH_WANTED:
+            return None
+        shape = FixedShape(tokens=_token_rows(step.n_tokens), requests=_power_of_two(step.n_seqs),
+                           wanted=_power_of_two(wanted), width=_power_of_two(batch.blocks_needed, MIN_GRAPH_WIDTH),
+                           planned={name: _power_of_two(rows) for name, rows in batch.planned_rows().items()})
+        key = shape.key()
+        if key in self._graphs:
+            return shape
+        if len(self._shape_seen) > 4096:
+            self._shape_seen.clear()
+        seen = self._shape_seen[key] = self._shape_seen.get(key, 0) + 1
+        return shape if seen >= SHAPE_SEEN_TWICE else None
+
+    def _mixed_graph_step(self, shape: FixedShape, batch: HostBatch) -> Optional[torch.Tensor]:
+        key = shape.key()
+        state = self._graphs.get(key)
+        if state is None:
+            while len(self._graphs) >= MAX_GRAPHS:
+                self._graphs.popitem(last=False)
+            state = self._graphs[key] = _DecodeGraph(self, shape.width)
+        else:
+            self._graphs.move_to_end(key)
+        ctx = state.builder.upload(batch, fixed=shape)
+        if state.graph is None:
+            self._capture(state, ctx)
+        state.graph.replay()
+        self.graph_replays += 1
+        self.mixed_graph_replays += 1
+        wanted = int(batch.want_rows.size)
+        if wanted == 0:
+            return None
+        logits = state.logits[:wanted]
+        return logits if self._borrow else logits.clone()
+
+    def _capture(self, state: "_DecodeGraph", ctx: StepContext) -> None:
+        """Once eagerly (libraries create their handles and workspaces), then the capture. The step writes the same
+        keys and values to the same slots each time, so running it again changes nothing."""
+        self.model.forward(ctx, self._bindings, ctx.want_rows)
+        torch.cuda.synchronize(self.device)
+        ctx.memo.clear()     # what the parts computed once for the step is computed inside the graph too
+        if self._graph_pool is None:
+            self._graph_pool = torch.cuda.graph_pool_handle()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, pool=self._graph_pool):
+            state.logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
+        state.graph = graph
+        self.graphs_captured += 1
 
     # ---- the step ------------------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry], reserved: bool = False, borrow_logits: bool = False) -> Optional[torch.Tensor]:
@@ -283,8 +347,13 @@ class Engine:
                 logits = self._graph_step(requests, entries)
             else:
                 self._last_graph = None
-                ctx = self._builder.build(requests, [entry.tokens for entry in entries], [entry.want for entry in entries])
-                logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
+                batch = self._builder.prepare(requests, [entry.tokens for entry in entries], [entry.want for entry in entries])
+                shape = self._fixed_shape(batch) if self.use_graphs and self.graph_mixed_steps else None
+                if shape is not None:
+                    logits = self._mixed_graph_step(shape, batch)
+                else:
+                    ctx = self._builder.upload(batch)
+                    logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
         except BaseException:
             self._roll_back(requests)
             raise

@@ -672,7 +672,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             paged_attention_prefill(q, k_cache, v_cache, view.block_table, plan.tiles, ctx.positions,
                                     scale, window, heads, kv_heads, head_dim, out=out)
         if plan.single_tokens.shape[0] > 0:
-            visible = min(plan.max_single_total, window) if window > 0 else plan.max_single_total
+            longest = max(plan.max_single_total, ctx.planned_total) if ctx.fixed else plan.max_single_total
+            visible = min(longest, window) if window > 0 else longest
             splits = decode_splits(plan.single_tokens.shape[0], kv_heads, visible)
             paged_attention_decode(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
                                    scale, window, heads, kv_heads, head_dim, splits, out=out, token_ids=plan.single_tokens)

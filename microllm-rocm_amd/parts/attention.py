@@ -37,6 +37,7 @@ class QueryTilePlanner:
     Plan: ``tiles`` int32 [workgroups, 5]; ``single_tokens`` int32 [rows]; ``max_single_total``, the longest of
     the requests listed there."""
     CROWDED = 4
+    padding = {"tiles": 0, "single_tokens": -1}      # an entry of two empty tiles; a row that is none: both passed over
 
     def __init__(self, windowed: bool, heads: int, compute_units: int):
         self.windowed = windowed

@@ -409,3 +409,51 @@ def test_logits_of_a_step_are_the_callers_to_keep(tmp_path):
     before = borrowed.clone()
     engine.step([StepEntry("a", [14], [0])], borrow_logits=True)
     assert not torch.equal(borrowed, before)          # the buffer of the graph: the next step has overwritten it
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_mixed_steps_replayed_from_graphs_equal_eager_steps(tmp_path, dtype, which):
+    """Steps that mix portions of prompts with single tokens are padded to a fixed shape and replayed from a graph once
+    the shape has come twice: every such step gives the bits of the same step run eagerly, whatever the padding
+    (the numbers of tokens, requests, wanted rows and attention tiles change from step to step within a shape), and
+    the keys and values it stores are what later steps read."""
+    from microllm_rocm_amd.engine import StepEntry
+    folder = make_folder(tmp_path, which, SHARP)
+    config = CONFIGS[which]
+    graphs = engine_for(folder, dtype, use_graphs=True, num_pages=24, max_tokens=None, max_requests=8)
+    eager = engine_for(folder, dtype, use_graphs=False, num_pages=24, max_tokens=None, max_requests=8)
+    rng = np.random.default_rng(3)
+
+    def both(entries):
+        out = [engine.step([StepEntry(*entry) for entry in entries]) for engine in (graphs, eager)]
+        torch.cuda.synchronize()
+        assert (out[0] is None) == (out[1] is None)
+        if out[0] is not None:
+            assert out[0].shape == out[1].shape and torch.equal(out[0], out[1]), "a replayed step differs from the eager step"
+
+    def tokens(count):
+        return rng.integers(0, config.vocab_size, size=count).tolist()
+
+    for round_index in range(6):
+        names = [f"r{round_index}_{index}" for index in range(4)]
+        for engine in (graphs, eager):
+            for name in names:
+                engine.open(name)
+        # two requests decode while the other two bring portions of 9 to 16 and 17 to 24 tokens: the same padded
+        # shapes in every round (16, 32 or 48 rows of tokens; 4 requests), other contents
+        both([(names[0], tokens(5), [4]), (names[1], tokens(11), [10])])
+        for step in range(5):
+            first, second = int(rng.integers(9, 17)), int(rng.integers(17, 25))
+            wanted = [[0], [0], [first - 1], []] if step % 2 else [[0], [], [0, first - 1], [second - 1]]
+            both([(names[0], tokens(1), wanted[0]), (names[1], tokens(1), wanted[1]),
+                  (names[2], tokens(first), wanted[2]), (names[3], tokens(second), wanted[3])])
+        both([(name, tokens(1), [0]) for name in names])          # and a decode step over what the mixed steps stored
+        both([(names[2], tokens(2), [1]), (names[0], tokens(1), [0])])
+        for engine in (graphs, eager):
+            for name in names:
+                engine.close(name)
+            engine.cache.check()
+    assert graphs.mixed_graph_replays >= 15 and eager.graph_replays == 0
+    pool = graphs.cache.groups[0].pool
+    assert pool.total_taken > pool.num_pages, "pages were used again"
