@@ -29,6 +29,36 @@ BF16_PEAK_FLOPS = 2.5e15       # MI355X dense bf16 MFMA, published
 FP32_PEAK_FLOPS = 157.3e12
 
 
+def serve(args, config, full_layers: int, page_size: int) -> int:
+    """The reference's continuous-batching workload through the scheduler; prints one JSON line."""
+    from microllm_rocm_amd import Engine
+    from microllm_rocm_amd.engine.benchmark import serving_throughput
+    requests, longest, new_tokens, chunk, budget = args.serve_requests, 2048, 256, 512, 2048
+    max_tokens = requests * (-(-(longest + new_tokens) // page_size) + 1) * page_size
+    engine = Engine.from_random(config, seed=0, dtype=args.dtype, device="cuda:0", on_device=True, page_size=page_size,
+                                max_tokens=max_tokens, max_requests=requests, weight_copies=args.weight_copies,
+                                max_portion=chunk, graph_mixed_steps=not args.no_mixed_graphs)
+    runs = max(1, min(args.steps, 5))
+    warmup = max(1, min(args.warmup, 2))
+    result = serving_throughput(engine, requests=requests, prompt_range=(128, longest), new_tokens=new_tokens,
+                                prefill_chunk=chunk, max_batched_tokens=budget, runs=runs, warmup=warmup)
+    line = {
+        "metric": f"continuous batching, generated tok/s, Qwen2-{args.size.upper()} {'bf16' if args.dtype == 'bfloat16' else 'fp32'}",
+        "value": round(result["tokens_per_second"], 1), "unit": "tok/s", "n_gpus": 1, "steps": runs, "warmup": warmup,
+        "ms_per_step": round(result["ms_per_run"], 2), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: random N(0,0.02) weights, uniform-random token ids and prompt lengths; a step is one whole run of the workload",
+        "config": {"model": f"Qwen2-{args.size.upper()} size", "layers": args.layers, "layers_of_full_model": full_layers,
+                   "requests": requests, "prompt_lengths": "uniform 128..2048", "new_tokens": new_tokens,
+                   "prefill_chunk": chunk, "max_batched_tokens": budget, "kv_block_size": page_size,
+                   "weight_copies": engine.weight_copies, "mixed_step_graphs": not args.no_mixed_graphs,
+                   "parallelism": "single GPU"},
+        "serve": {key: (round(value, 2) if isinstance(value, float) else value) for key, value in result.items()},
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -47,6 +77,11 @@ def main() -> int:
     parser.add_argument("--no-library-tuning", action="store_true",
                         help="leave the choice of the library's algorithm for the prompt's large products to its heuristic")
     parser.add_argument("--no-calibration", action="store_true", help="skip measuring what a read-only and an MFMA-only kernel reach")
+    parser.add_argument("--serve", action="store_true",
+                        help="the continuous-batching workload instead: 64 requests, prompts of 128 to 2048 tokens, 256 new tokens each, "
+                             "portions of 512 (--steps whole runs timed after --warmup untimed ones); meant for --size 0.5b")
+    parser.add_argument("--serve-requests", type=int, default=64)
+    parser.add_argument("--no-mixed-graphs", action="store_true", help="run steps that mix portions and single tokens eagerly")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
@@ -62,6 +97,8 @@ def main() -> int:
         args.layers = full_layers
     config = Qwen2Config(num_hidden_layers=args.layers, max_position_embeddings=32768, rope_theta=1e6, rms_norm_eps=1e-6, **sizes)
     page_size = 16
+    if args.serve:
+        return serve(args, config, full_layers, page_size)
     points = sorted({int(b) for b in args.points.split(",") if b} | {args.batch})
     largest = max(points)
     per_request = args.context + args.steps + args.warmup + 2 * page_size

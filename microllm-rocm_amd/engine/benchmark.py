@@ -137,3 +137,57 @@ def step_flops(engine: Engine, tokens: int) -> float:
             flops += 4.0 * mixer.heads * mixer.head_dim * pairs
     flops += 2.0 * engine.model.head.weight.out_features * engine.model.head.weight.in_features
     return flops
+
+
+def percentile(values, quantile: float) -> float:
+    """Linear interpolation between the two nearest of the sorted values (apps/hf_infer.cpp:570-580)."""
+    ordered = sorted(values)
+    position = quantile * (len(ordered) - 1)
+    lower = int(position)
+    upper = min(lower + 1, len(ordered) - 1)
+    fraction = position - lower
+    return ordered[lower] * (1.0 - fraction) + ordered[upper] * fraction
+
+
+def serving_throughput(engine: Engine, requests: int = 64, prompt_range=(128, 2048), new_tokens: int = 256,
+                       prefill_chunk: int = 512, max_batched_tokens: int = 2048, runs: int = 3, warmup: int = 1,
+                       seed: int = 0) -> Dict[str, float]:
+    """The reference's continuous-batching workload (apps/hf_infer.cpp:862-900): ``requests`` prompts of
+    uniform-random lengths, all there at step 0, ``new_tokens`` greedy tokens each, through the scheduler.
+    The whole workload runs ``warmup`` times untimed and ``runs`` times timed; every run must give the same tokens.
+    Returns generated tokens a second and the latencies of the last run."""
+    from .generate import generate
+    rng = np.random.default_rng(seed)
+    lengths = rng.integers(prompt_range[0], prompt_range[1] + 1, size=requests)
+    prompts = [rng.integers(0, engine.spec.vocab_size, size=int(length)).tolist() for length in lengths]
+    params = SamplingParams(max_new_tokens=new_tokens, temperature=0.0)
+
+    def run_once():
+        return generate(engine, prompts, params, max_batched_tokens=max_batched_tokens, prefill_chunk=prefill_chunk,
+                        return_scheduler=True)
+
+    for _ in range(warmup):
+        run_once()
+    torch.cuda.synchronize()
+    elapsed, outputs, scheduler = 0.0, None, None
+    for _ in range(runs):
+        started = time.perf_counter()
+        current, scheduler = run_once()
+        torch.cuda.synchronize()
+        elapsed += time.perf_counter() - started
+        if outputs is not None and current != outputs:
+            raise RuntimeError("continuous generation changed across measured runs")
+        outputs = current
+    generated = sum(len(output) - len(prompt) for output, prompt in zip(outputs, prompts))
+    served = [scheduler.request(index) for index in range(requests)]
+    ttft = [(r.first_token_time - r.submit_time) * 1e3 for r in served]
+    completion = [(r.completion_time - r.submit_time) * 1e3 for r in served]
+    metrics = scheduler.metrics
+    return {"tokens_per_second": generated * runs / elapsed, "ms_per_run": elapsed / runs * 1e3,
+            "generated_tokens": generated, "prompt_tokens": int(lengths.sum()),
+            "model_tokens_per_second": (generated + int(lengths.sum())) * runs / elapsed,
+            "scheduler_steps": metrics.scheduler_steps, "preemptions": metrics.preemptions,
+            "ttft_p50_ms": percentile(ttft, 0.5), "ttft_p95_ms": percentile(ttft, 0.95),
+            "completion_p50_ms": percentile(completion, 0.5), "completion_p95_ms": percentile(completion, 0.95),
+            "graph_replays": engine.graph_replays, "mixed_graph_replays": engine.mixed_graph_replays,
+            "graphs_captured": engine.graphs_captured}
