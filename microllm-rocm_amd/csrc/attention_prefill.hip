@@ -3,11 +3,10 @@
 // A workgroup (8 waves) takes two tiles of up to 128 consecutive tokens each, of one request's portion and one
 // query head: waves 0 to 3 a block of 32 tokens each of the first tile, waves 4 to 7 of the second; the 32 tokens
 // are the 32 columns of v_mfma_f32_32x32x16_bf16. Every SIMD thus has a wave of either tile, whose matrix and
-// vector work overlap. The host pairs a tile that sees many keys with one that sees few where a prompt has few
-// tiles, so that every workgroup walks about as many keys and the compute units finish together (under a causal
-// mask the last tile of a prompt has as many times the work of the first as there are tiles), and neighbouring
-// tiles where there are many or under a window: these read nearly the same keys, and the longest workgroups go
-// first. Both tiles read the same keys from LDS. The second tile may be empty.
+// vector work overlap. The host pairs a tile that sees many keys with one that sees few, so that every workgroup
+// walks about as many keys and the compute units finish together (under a causal mask the last tile of a prompt
+// has as many times the work of the first as there are tiles), and neighbouring tiles under a window, which read
+// nearly the same keys. Both tiles read the same keys from LDS. The second tile may be empty.
 // The workgroup walks the keys its tokens can see in blocks of 128 (64 for head sizes above 128): the block's key
 // and value tiles are copied from the pages straight into LDS as they lie there (the pages are in MFMA order,
 // cache_layout.h), the next block's being on its way while this one is used. The two stages are two LDS

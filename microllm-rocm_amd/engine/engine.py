@@ -316,9 +316,13 @@ class Engine:
             count = len(entry.tokens)
             if count == 0:
                 raise ValueError(f"request {entry.request_id!r} brings no tokens")
-            for token in entry.tokens:
-                if not 0 <= int(token) < self.spec.vocab_size:
-                    raise ValueError(f"token {token} of request {entry.request_id!r} is outside the vocabulary")
+            if count == 1:
+                lowest = highest = int(entry.tokens[0])
+            else:
+                lowest, highest = int(min(entry.tokens)), int(max(entry.tokens))
+            if lowest < 0 or highest >= self.spec.vocab_size:
+                bad = next(token for token in entry.tokens if not 0 <= int(token) < self.spec.vocab_size)
+                raise ValueError(f"token {bad} of request {entry.request_id!r} is outside the vocabulary")
             if self.max_portion is not None and count > self.max_portion:
                 raise ValueError(f"request {entry.request_id!r} brings {count} tokens; this engine's cache was sized "
                                  f"for portions of at most {self.max_portion}")

@@ -70,6 +70,15 @@ class Request:
     def token_at(self, index: int) -> int:
         return self.prompt[index] if index < len(self.prompt) else self.generated[index - len(self.prompt)]
 
+    def tokens_between(self, start: int, stop: int) -> List[int]:
+        """Tokens ``start`` to ``stop - 1`` of the prompt followed by what was generated."""
+        length = len(self.prompt)
+        if stop <= length:
+            return self.prompt[start:stop]
+        if start >= length:
+            return self.generated[start - length:stop - length]
+        return self.prompt[start:] + self.generated[:stop - length]
+
     @property
     def terminal(self) -> bool:
         return self.state in (RequestState.COMPLETED, RequestState.CANCELLED)
@@ -260,7 +269,7 @@ class Scheduler:
             entries = []
             for portion in portions:
                 request = portion.request
-                tokens = [request.token_at(index) for index in range(portion.start, portion.start + portion.count)]
+                tokens = request.tokens_between(portion.start, portion.start + portion.count)
                 entries.append(StepEntry(request.id, tokens, [portion.count - 1] if portion.wants_logits else []))
             try:
                 logits = self.engine.step(entries, reserved=True, borrow_logits=True)
