@@ -53,12 +53,6 @@ __device__ inline float reduce_lanes_32_apart(float value, Op op) {
     return op(__builtin_bit_cast(float, low), __builtin_bit_cast(float, high));
 }
 
-#ifdef MLL_PREFILL_TIMING
-__device__ unsigned long long prefill_cycles[6];
-#define TICK(slot) do { const long long now_ = clock64(); spent[slot] += now_ - last_tick; last_tick = now_; } while (0)
-#else
-#define TICK(slot)
-#endif
 
 template <int HD_TILES>
 __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_kernel(
@@ -367,12 +361,7 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     // One block: the next one is sent for, this one is used. Called by turns with the stages exchanged.
     int block = first_block;
     int following = next_seen(first_block);
-#ifdef MLL_PREFILL_TIMING
-    long long spent[6] = {0, 0, 0, 0, 0, 0};
-    long long last_tick = clock64();
-#endif
     auto walk = [&](const bf16* stage, bf16* next_stage) {
-        TICK(4);
         if (following <= last_block) {
             fetch(following, next_stage);
             const int after = next_seen(following);
@@ -380,7 +369,6 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
         }
         const bf16* k_lds = stage;
         const bf16* v_lds = stage + HALF_CHUNKS * 8;
-        TICK(0);
         // Unrolled: every read from LDS then has the stage's own address plus a constant, and the compiler can tell
         // that the loads on their way into the other stage do not touch it (of an address that a loop carries along
         // it cannot, and waits for those loads before the first read).
@@ -404,14 +392,8 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
                 }
             }
         }
-        TICK(1);
         wait_for_loads();
-        TICK(2);
         landed(following, next_stage);
-        TICK(3);
-#ifdef MLL_PREFILL_TIMING
-        spent[5] += 1;
-#endif
         block = following;
         following = next_seen(block);
     };
@@ -425,10 +407,6 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
         walk(stage_odd, stage_even);
     }
     running_sum = reduce_lanes_32_apart(running_sum, [](float a, float b) { return a + b; });
-#ifdef MLL_PREFILL_TIMING
-    if (lane == 0 && block_valid > 0 && wave < 4)
-        for (int slot = 0; slot < 6; ++slot) atomicAdd(&prefill_cycles[slot], static_cast<unsigned long long>(spent[slot]));
-#endif
 
     // o_acc[d][i]: dim 32 d + 8 (i / 4) + 4 half + i % 4 of token `column`.
     if (column < block_valid) {
@@ -465,16 +443,6 @@ using namespace mll;
 
 extern "C" int mll_paged_attention_prefill_tile() { return kPrefillTile; }
 
-#ifdef MLL_PREFILL_TIMING
-extern "C" int mll_prefill_timing(long long* out) {
-    unsigned long long host[6];
-    (void)hipMemcpyFromSymbol(host, HIP_SYMBOL(prefill_cycles), sizeof(host));
-    for (int i = 0; i < 6; ++i) out[i] = static_cast<long long>(host[i]);
-    unsigned long long zero[6] = {0, 0, 0, 0, 0, 0};
-    (void)hipMemcpyToSymbol(HIP_SYMBOL(prefill_cycles), zero, sizeof(zero));
-    return 0;
-}
-#endif
 
 
 extern "C" int mll_paged_attention_prefill(const void* q, const void* k_cache, const void* v_cache,

@@ -103,10 +103,8 @@ def weight_bytes(engine: Engine) -> int:
     total += count(model.final_norm.weight) + count(model.head.weight)
     for block in model.blocks:
         for part in block.parts():
-            total += sum(count(value) for value in vars(part).values())
-            position = getattr(part, "position", None)
-            if position is not None:
-                total += sum(count(value) for value in vars(position).values())
+            for piece in (part, *part.sub_parts()):
+                total += sum(count(value) for value in vars(piece).values())
     return total
 
 
