@@ -135,6 +135,7 @@ class Engine:
         # Steps in which every request brings one token are replayed from HIP graphs, one per (number of
         # requests, block-table width): the launches of a decode step cost more host time than GPU time.
         self.use_graphs = use_graphs and all(part.graph_safe for part in self.model.parts())
+        self._graphs_allowed = self.use_graphs
         # All captures share one memory pool: a graph's activations live only while it runs, so the next graph may
         # have them; what a graph hands out (its logits) stays its own while the graph is kept. At most
         # MAX_GRAPHS are kept (continuous batching walks through many numbers of requests): each holds its
@@ -367,6 +368,25 @@ class Engine:
         if self._last_graph is not None:
             self._build_ahead(self._last_graph, requests)
         return logits
+
+    def observe_layers(self, observer) -> None:
+        """Call ``observer(run entry, stream)`` after every run entry of every step from now on, ``stream`` being
+        the float32 residual stream ``[tokens, hidden]`` with that entry's result added (a fresh tensor); None
+        switches it off. Steps run eagerly meanwhile: a graph's replay calls nothing on the host."""
+        if observer is None:
+            self.model.observer = None
+            self.use_graphs = self._graphs_allowed
+            return
+
+        def after_entry(index, h, pending):
+            stream = h.clone()
+            if isinstance(pending, torch.Tensor):   # else the entry's last product added its result itself
+                for part in (pending if pending.dim() == 3 else pending.unsqueeze(0)):
+                    stream += part.to(torch.float32)
+            observer(index, stream)
+
+        self.model.observer = after_entry
+        self.use_graphs = False
 
     def _roll_back(self, requests: List[RequestCache]) -> None:
         """A step failed inside the model (a kernel refused its arguments, a part raised): nothing of it counts.

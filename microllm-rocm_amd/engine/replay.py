@@ -15,16 +15,25 @@ import sys
 from typing import IO, Optional
 
 import numpy as np
+import torch
 
 from .batch import StepEntry
 from .engine import Engine
 
 
-def replay(engine: Engine, lines: IO[str], out_dir: str, report: Optional[IO[str]] = None) -> int:
-    """Run every step read from ``lines``; returns the number of steps run."""
+def replay(engine: Engine, lines: IO[str], out_dir: str, report: Optional[IO[str]] = None,
+           dump_layers: bool = False) -> int:
+    """Run every step read from ``lines``; returns the number of steps run.
+
+    With ``dump_layers`` a step that wants logits also writes ``<step>.layers.f32``: the float32 residual stream
+    at the wanted places after every run entry, ``[entries, wanted, hidden]`` (the reference traces tensors by
+    name instead, include/microllm/profiling/trace.h:63). Steps then run without graphs."""
     os.makedirs(out_dir, exist_ok=True)
     report = report or sys.stdout
     steps = 0
+    streams = []
+    if dump_layers:
+        engine.observe_layers(lambda index, stream: streams.append(stream))
     for line in lines:
         line = line.strip()
         if not line:
@@ -37,10 +46,18 @@ def replay(engine: Engine, lines: IO[str], out_dir: str, report: Optional[IO[str
             if not engine.is_open(request_id):
                 engine.open(request_id)
             entries.append(StepEntry(request_id, list(item["tokens"]), list(item.get("want", []))))
+        streams.clear()
         logits = engine.step(entries) if entries else None
         if logits is not None:
             array = logits.detach().to("cpu").numpy().astype("<f4", copy=False)
             array.tofile(os.path.join(out_dir, f"{step}.f32"))
+            if dump_layers:
+                rows, first = [], 0
+                for entry in entries:
+                    rows += [first + place for place in entry.want]
+                    first += len(entry.tokens)
+                wanted = torch.stack(streams)[:, rows].to("cpu").numpy().astype("<f4", copy=False)
+                wanted.tofile(os.path.join(out_dir, f"{step}.layers.f32"))
         for request_id in record.get("end", []):
             if engine.is_open(request_id):
                 engine.close(request_id)
@@ -60,10 +77,12 @@ def main(argv=None) -> int:
     parser.add_argument("--page-size", type=int, default=16)
     parser.add_argument("--max-requests", type=int, default=16)
     parser.add_argument("--device", default="cuda:0")
+    parser.add_argument("--dump-layers", action="store_true",
+                        help="also write <step>.layers.f32: the residual stream at the wanted places after every layer")
     args = parser.parse_args(argv)
     if args.max_tokens <= 0:
         parser.error("--max-tokens must be positive")
     engine = Engine.from_folder(args.model, dtype=args.dtype, device=args.device, page_size=args.page_size,
                                 max_tokens=args.max_tokens, max_requests=args.max_requests)
-    replay(engine, sys.stdin, args.out)
+    replay(engine, sys.stdin, args.out, dump_layers=args.dump_layers)
     return 0

@@ -93,6 +93,9 @@ class Model:
         self.blocks: List[Block] = [build_block(layer, runtime) for layer in spec.layers]
         self.final_norm = build_part("norm", spec.final_norm, runtime)
         self.head = build_part("head", spec.head, runtime)
+        # Called as observer(run entry, h, pending) after every entry of a step when set (the replay tool's dump of
+        # the stream layer by layer; the reference traces tensors by name, include/microllm/profiling/trace.h:63).
+        self.observer = None
 
     # ---- tensors -------------------------------------------------------------------------
     def tensors(self) -> Dict[str, TensorDecl]:
@@ -169,6 +172,8 @@ class Model:
         for index, entry in enumerate(order):
             next_block = self.blocks[order[index + 1].layer] if index + 1 < len(order) else None
             pending = self.blocks[entry.layer].forward(h, pending, ctx, caches[index], next_block)
+            if self.observer is not None:
+                self.observer(index, h, pending)
         if want_rows is None or want_rows.numel() == 0:
             return None
         x = self.final_norm.forward(h, delta=pending, write_h=False, rows=want_rows)

@@ -183,6 +183,18 @@ def forward(config: dict, weights: Dict[str, np.ndarray], tokens: Sequence[int],
     return linear(x, head)
 
 
+def layer_streams(config: dict, weights: Dict[str, np.ndarray], tokens: Sequence[int]) -> np.ndarray:
+    """The residual stream after every layer, [layers, T, hidden]: what the reference's tensor trace shows layer
+    by layer (include/microllm/profiling/trace.h:63, src/model/model.cpp:851-860)."""
+    windows = layer_windows(config)
+    h = embedding(weights["model.embed_tokens.weight"], tokens)
+    after = []
+    for index in range(config["num_hidden_layers"]):
+        h = block(h, weights, index, config, windows[index])
+        after.append(h)
+    return np.stack(after)
+
+
 # ------------------------------------------------------------------------------------------------
 # token selection
 def greedy(logits: np.ndarray) -> int:

@@ -250,3 +250,15 @@ def test_generate_greedy_extends_by_argmax():
     assert len(out) == 4
     assert out[0] == int(np.argmax(plain.forward(config, w, [1, 2, 3])[-1]))
     assert out[1] == int(np.argmax(plain.forward(config, w, [1, 2, 3, out[0]])[-1]))
+
+
+def test_layer_streams_end_in_the_logits():
+    config, w = _tiny_model(11)
+    tokens = [3, 1, 4, 1, 5, 9]
+    streams = plain.layer_streams(config, w, tokens)
+    assert streams.shape == (config["num_hidden_layers"], len(tokens), config["hidden_size"])
+    h = plain.embedding(w["model.embed_tokens.weight"], tokens)
+    np.testing.assert_array_equal(streams[0], plain.block(h, w, 0, config, plain.layer_windows(config)[0]))
+    head = w["model.embed_tokens.weight"] if config["tie_word_embeddings"] else w["lm_head.weight"]
+    np.testing.assert_allclose(plain.forward(config, w, tokens),
+                               plain.rms_norm(streams[-1], w["model.norm.weight"], config["rms_norm_eps"]) @ head.T, rtol=1e-12)

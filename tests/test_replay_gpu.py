@@ -237,3 +237,32 @@ def test_stale_pages_hold_anything(tmp_path_factory, tmp_path, dtype):
     pool = engine.cache.groups[0].pool
     assert pool.total_taken > pool.num_pages
     compare(collect(steps, tmp_path / "out", config.vocab_size), requests, plain_model, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_stream_layer_by_layer(tmp_path_factory, tmp_path, dtype):
+    """--dump-layers: the residual stream at the wanted places after every layer, against the plain
+    implementation's, in portions of changing size (few rows: the norms are taken by the products; many: not)."""
+    import plain_qwen2 as plain
+    from replay_tools import TOLERANCE
+    config = CONFIGS["B"]
+    folder, plain_model = model_for(tmp_path_factory, "B", SHARP)
+    tokens = random_tokens(77, 90, config.vocab_size)
+    steps = portions("a", tokens, [40, 2, 17, 1, 1, 29])
+    out_dir = tmp_path / "layers"
+    result = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                             "--out", str(out_dir), "--max-tokens", "128", "--dump-layers"],
+                            input=to_lines(steps), capture_output=True, text=True, timeout=300)
+    assert result.returncode == 0, result.stderr
+    compare(collect(steps, out_dir, config.vocab_size), {"a": tokens}, plain_model, dtype)
+    expected = plain.layer_streams(plain_model.config, plain_model.weights, tokens)
+    layers, width = config.num_hidden_layers, config.hidden_size
+    first = 0
+    for step in steps:
+        entry = step["entries"][0]
+        got = np.fromfile(out_dir / f"{step['step']}.layers.f32", dtype="<f4").reshape(layers, len(entry["want"]), width)
+        for layer in range(layers):
+            want = expected[layer][[first + place for place in entry["want"]]]
+            error = np.abs(got[layer] - want).max() / np.abs(expected[layer]).max()
+            assert error <= TOLERANCE[dtype]["max"], f"{dtype}: step {step['step']} layer {layer}: {error:.3e}"
+        first += len(entry["tokens"])
