@@ -4,7 +4,8 @@ Pages hold their positions in tiles of 16, laid out in the order the MFMA kernel
 formulas are in ``csrc/cache_layout.h``):
 
     keys:   [page, kv_head, tile, dim // 8, position % 16, dim % 8]
-    values: [page, kv_head, tile, dim // 16, (position % 16) // 4, dim % 16, position % 4]
+    values: [page, kv_head, tile, dim // 32, (position % 16) // 8, dim % 32, position % 8], the tile flat
+            (a last block of 16 dims, where ``head_dim`` is an odd multiple of 16, is [position // 8, 16, 8])
 
 ``head_dim`` is padded to a multiple of 8 (keys) or 16 (values).
 """
@@ -31,7 +32,7 @@ def key_page_shape(num_pages: int, kv_heads: int, page_size: int, head_dim: int)
 
 def value_page_shape(num_pages: int, kv_heads: int, page_size: int, head_dim: int) -> Tuple[int, ...]:
     check_sizes(page_size, head_dim)
-    return (num_pages, kv_heads, page_size // TILE, -(-head_dim // 16), 4, TILE, 4)
+    return (num_pages, kv_heads, page_size // TILE, -(-head_dim // 16) * 16 * TILE)
 
 
 class _KeyView:
@@ -56,23 +57,31 @@ class _KeyView:
         self._plain().copy_(padded.view(pages, kv_heads, tiles, TILE, chunks, 8))
 
 
+def value_index(dims: int) -> torch.Tensor:
+    """Where (position, dim) of a tile lies in the flat tile, ``[TILE, dims]``; ``dims`` is a multiple of 16."""
+    position = torch.arange(TILE).view(TILE, 1)
+    dim = torch.arange(dims).view(1, dims)
+    block = dim // 32
+    width = torch.clamp(dims - 32 * block, max=32)
+    return block * 512 + ((position // 8) * width + dim % 32) * 8 + position % 8
+
+
 class _ValueView:
     def __init__(self, pages: torch.Tensor, head_dim: int):
         self.pages, self.head_dim = pages, head_dim
-
-    def _plain(self) -> torch.Tensor:
-        # [page, kv_head, tile, dim_tile, quad, dim16, key4] -> [page, kv_head, tile, quad, key4, dim_tile, dim16]
-        return self.pages.permute(0, 1, 2, 4, 6, 3, 5)
+        self.dims = pages.shape[-1] // TILE
+        self.index = value_index(self.dims).to(pages.device)
 
     def read(self) -> torch.Tensor:
-        pages, kv_heads, tiles, dim_tiles, _, _, _ = self.pages.shape
-        return self._plain().reshape(pages, kv_heads, tiles * TILE, dim_tiles * 16)[..., :self.head_dim]
+        pages, kv_heads, tiles, _ = self.pages.shape
+        plain = self.pages[..., self.index]      # [page, kv_head, tile, position16, dim]
+        return plain.reshape(pages, kv_heads, tiles * TILE, self.dims)[..., :self.head_dim]
 
     def write(self, rows: torch.Tensor) -> None:
-        pages, kv_heads, tiles, dim_tiles, _, _, _ = self.pages.shape
-        padded = torch.zeros((pages, kv_heads, tiles * TILE, dim_tiles * 16), dtype=self.pages.dtype, device=self.pages.device)
+        pages, kv_heads, tiles, _ = self.pages.shape
+        padded = torch.zeros((pages, kv_heads, tiles * TILE, self.dims), dtype=self.pages.dtype, device=self.pages.device)
         padded[..., :self.head_dim] = rows
-        self._plain().copy_(padded.view(pages, kv_heads, tiles, 4, 4, dim_tiles, 16))
+        self.pages[..., self.index] = padded.view(pages, kv_heads, tiles, TILE, self.dims)
 
 
 def key_rows(k_pages: torch.Tensor, head_dim: int) -> torch.Tensor:

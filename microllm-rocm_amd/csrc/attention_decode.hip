@@ -87,34 +87,44 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
     for (int d = 0; d < HD_TILES; ++d) o_acc[d] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     float running_max = -INFINITY, running_sum = 0.0f;
 
-    // A pair's keys and values, from the pages into registers. Keys: A operand, row = key `col` of the tile, 8
-    // dims (chunk 4 * ks + quad) per lane. Values: A operand of the second product, row = dim `col` of a dim
-    // tile, k-slots = keys 4*quad..+3 of tile 0, then of tile 1. Every load is issued, none behind a branch (a
-    // tile that no query sees is read from page 0 and masked like a stale one): only of straight-line code does
-    // the compiler know how many loads are still on their way, and waits for one pair alone while the next flies.
+    // A pair's keys and values, from the pages into registers. A lane's 8 k-slots of the second product are the
+    // 8 positions 8 * (quad % 2) .. + 7 of tile quad / 2 of the pair: one load of 16 bytes per 16 dims from the
+    // value pages (which hold blocks of 32 dims as [position / 8][dim][position % 8], cache_layout.h). The first product's rows are taken in the order that makes the scores come out so: of its two
+    // products, product t gives lane (head, quad) the keys 8 * quad + 4 * t .. + 3 of the pair, so its row
+    // 4 * quad' + i (the lane whose `col` that is brings it) is key 8 * quad' + 4 * t + i.
+    // Every load is issued, none behind a branch (a tile that no query sees is read from page 0 and masked like a
+    // stale one): only of straight-line code does the compiler know how many loads are still on their way, and
+    // waits for one pair alone while the next flies.
     auto load_pair = [&](int pair_index, const int (&page)[2], Frag8 (&k_frag)[2][K_STEPS], Frag8 (&v_frag)[HD_TILES]) {
+        const int k_side = col / 8, v_side = quad / 2;      // which tile of the pair the lane's row / its k-slots lie in
+        const int k_offset = (pair_index * 32 + 16 * k_side) % page_size;
+        const int v_offset = (pair_index * 32 + 16 * v_side) % page_size;
+        const bf16* k_tile = k_cache + layout.k_tile(max(k_side ? page[1] : page[0], 0), kv_head, k_offset / 16) +
+                             (8 * ((col / 4) % 2) + col % 4) * 8;
+        const bf16* v_tile = v_cache + layout.v_tile(max(v_side ? page[1] : page[0], 0), kv_head, v_offset / 16);
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const int offset = (pair_index * 32 + 16 * t) % page_size;
-            const bf16* k_tile = k_cache + layout.k_tile(max(page[t], 0), kv_head, offset / 16) + col * 8;
-            const bf16* v_tile = v_cache + layout.v_tile(max(page[t], 0), kv_head, offset / 16) + (quad * 16 + col) * 4;
 #pragma unroll
             for (int ks = 0; ks < K_STEPS; ++ks) {
                 const int piece = ks * 4 + quad;
                 if (HD % 32 == 0) {
-                    k_frag[t][ks].raw = *reinterpret_cast<const uint4*>(k_tile + piece * 128);
+                    k_frag[t][ks].raw = *reinterpret_cast<const uint4*>(k_tile + piece * 128 + t * 32);
                 } else {      // the last 32 dims are not all there: nothing may be read past the tile
                     k_frag[t][ks].raw = make_uint4(0, 0, 0, 0);
-                    if (piece < K_CHUNKS) k_frag[t][ks].raw = *reinterpret_cast<const uint4*>(k_tile + piece * 128);
+                    if (piece < K_CHUNKS) k_frag[t][ks].raw = *reinterpret_cast<const uint4*>(k_tile + piece * 128 + t * 32);
                 }
             }
+        }
 #pragma unroll
-            for (int d = 0; d < HD_TILES; ++d) v_frag[d].h[t] = *reinterpret_cast<const bf16x4*>(v_tile + d * 256);
+        for (int d = 0; d < HD_TILES; ++d) {
+            constexpr int kLast = HD_TILES - 1;
+            const int width = (HD_TILES % 2 == 1 && d == kLast) ? 16 : 32;      // dims of the block of 32 this tile of 16 lies in
+            v_frag[d].raw = *reinterpret_cast<const uint4*>(v_tile + (d / 2) * 512 + ((quad % 2) * width + (d % 2) * 16 + col) * 8);
         }
     };
     auto attend_pair = [&](int pair_index, const Frag8 (&k_frag)[2][K_STEPS], Frag8 (&v_frag)[HD_TILES]) {
         const int key0 = pair_index * 32;
-        // S^T = K . Q^T: lane holds head `col`, keys 4*quad + i of each tile.
+        // S^T = K . Q^T: lane holds head `col`, keys 8 * quad + 4 * t + i of the pair from product t.
         float score[8];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -124,7 +134,7 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
                 s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_frag[t][ks].v, q_frag[ks].v, s, 0, 0, 0);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int key = key0 + 16 * t + 4 * quad + i;
+                const int key = key0 + 8 * quad + 4 * t + i;
                 score[4 * t + i] = (key >= low && key <= position) ? s[i] * scale : -INFINITY;
             }
         }

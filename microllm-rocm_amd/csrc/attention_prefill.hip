@@ -13,8 +13,9 @@
 // variables, so that the compiler need not wait for a load into one before it reads the other.
 // Scores are computed transposed, S^T = K . Q^T: a lane then holds 16 keys of one token (its column), and the other
 // half of the wave the other 16, so a token's maximum takes 15 comparisons and one exchange, and its sum is kept in
-// two halves that meet once, at the end. O^T = V^T . P^T follows from registers: the lane's scores of a 16-key tile
-// are the 8 values the second product wants from it, if the values' operand is read in the same order.
+// two halves that meet once, at the end. O^T = V^T . P^T follows from registers: the rows of the first product are
+// the run's keys in such an order (bits 2 and 3 of the row number exchanged) that the lane's scores of a 16-key
+// tile are for 8 neighbouring positions, the 16 bytes that one read brings from the value tile for its dim.
 // Only steps that touch the causal diagonal or the window's edge pay for the mask (a second
 // instance of the loop's body), and values that no token of the workgroup can see are cleared in LDS before a
 // block at an end of the walk is used, so that stale memory never meets a zero weight.
@@ -184,7 +185,7 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     int pages[PASSES];
     int no_lane = 0;
     asm volatile("v_mov_b32 %0, 0" : "=v"(no_lane));      // zero, but the compiler cannot tell: keeps the address per lane
-    auto look_up_with = [&](auto shift_tag, int block) {
+    auto look_up_with = [&](auto shift_tag, int block) __attribute__((always_inline)) {
         const bool whole = FULL_PASSES && inside(block);      // the usual case: every tile of the block, no questions
 #pragma unroll
         for (int pass = 0; pass < PASSES; ++pass) {
@@ -193,11 +194,11 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
             if (whole || wanted(block, pass)) pages[pass] = table[page_index(shift_tag, tile_index) + no_lane];
         }
     };
-    auto look_up = [&](int block) {
+    auto look_up = [&](int block) __attribute__((always_inline)) {
         if (page_shift >= 0) look_up_with(std::true_type{}, block);
         else look_up_with(std::false_type{}, block);
     };
-    auto fetch_with = [&](auto shift_tag, int block, bf16* stage) {      // after look_up(block)
+    auto fetch_with = [&](auto shift_tag, int block, bf16* stage) __attribute__((always_inline)) {      // after look_up(block)
 #pragma unroll
         for (int pass = 0; pass < PASSES; ++pass) {
             const int tile_index = block * BLOCK_TILES + tile_of(pass);
@@ -214,14 +215,14 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
             }
         }
     };
-    auto fetch = [&](int block, bf16* stage) {
+    auto fetch = [&](int block, bf16* stage) __attribute__((always_inline)) {
         if (page_shift >= 0) fetch_with(std::true_type{}, block, stage);
         else fetch_with(std::false_type{}, block, stage);
     };
     // A block at an end of what the tile's tokens see, once it lies in LDS: values at positions that no token
     // sees may be stale memory, and the places of tiles that were not brought in hold what was there before.
     // Both are cleared (their scores are masked where they are computed).
-    auto clear_unseen = [&](int block, bf16* stage) {
+    auto clear_unseen = [&](int block, bf16* stage) __attribute__((always_inline)) {
 #pragma unroll
         for (int pass = 0; pass < PASSES; ++pass) {
             if (tile_of(pass) >= BLOCK_TILES) continue;
@@ -230,11 +231,14 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
             values.raw = make_uint4(0, 0, 0, 0);
             if (wanted(block, pass)) {
                 values.raw = *place;
-                const int element = piece_of(pass) * 8;      // 2 dims x positions 4 g .. 4 g + 3
-                const int first_key = block * BLOCK_KEYS + 16 * tile_of(pass) + 4 * ((element / 64) % 4);
+                // one dim, positions 0 .. 7 or 8 .. 15 of the tile: a block of 32 dims is [position / 8][32][8], a last
+                // block of 16 dims [position / 8][16][8]
+                const int element = piece_of(pass) * 8;
+                const int width = (HD % 32 != 0 && element / 512 == HD / 32) ? 16 : 32;
+                const int first_key = block * BLOCK_KEYS + 16 * tile_of(pass) + 8 * ((element % 512) / (8 * width));
 #pragma unroll
                 for (int i = 0; i < 8; ++i)
-                    if (!seen(first_key + i % 4)) values.v[i] = static_cast<__bf16>(0.0f);
+                    if (!seen(first_key + i)) values.v[i] = static_cast<__bf16>(0.0f);
             }
             *place = values.raw;
         }
@@ -243,7 +247,7 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     const int last_block = group_last / BLOCK_KEYS;
     // The wave's loads into LDS have landed (the compiler does not wait for loads that return nothing), and so
     // have everyone's; everyone is done with the stage that is written next.
-    auto landed = [&](int block, bf16* stage) {
+    auto landed = [&](int block, bf16* stage) __attribute__((always_inline)) {
         wait_for_loads();
         __syncthreads();
         if (block <= last_block && !inside(block)) {
@@ -257,11 +261,27 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     // must be rescaled, and their two chains of products hide each other's latency. MASKED: some key is hidden
     // from some token (the causal diagonal, the window's edge, the end of the sequence).
     // Scores stay in the product's units; p = 2^((s - max) * scale_log2) is one multiply-add and one exponent.
-    auto process_keys = [&](auto masked_tag, auto halves_tag, const bf16* k_lds, const bf16* v_lds, int first_run, int key0) {
+    // Where a lane reads its operands in a stage, but for the run. The address of every read is the stage's own
+    // variable, plus this, plus a constant: the compiler follows an address back to its LDS variable over a few
+    // additions only, and a read that it cannot place waits for all loads on their way into either stage.
+    // First product: row `column` = the key of the run whose number is `column` with bits 2 and 3 exchanged (tile
+    // column / 16), 8 dims (chunk 2 ks + half) per lane. Second: row = dim `column` of a block of 32 dims; the
+    // lane's 8 k-slots are the keys its scores came for, positions 8 half .. + 7 of the tile, one read of 16 bytes;
+    // the 64 lanes read 1024 consecutive bytes, which LDS gives without bank conflicts.
+    const int key_of_row = (column & ~12) | ((column & 4) << 1) | ((column & 8) >> 1);
+    const int k_lane = (column / 16) * TILE_ELEMENTS + (half * 16 + key_of_row % 16) * 8;
+    const int v_lane = (half * 32 + column) * 8;      // in a block of 32 dims; a last block of 16 has its own
+    auto process_keys = [&](auto masked_tag, auto halves_tag, const bf16* stage, int first_run, int key0) __attribute__((always_inline)) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         constexpr int HALVES = decltype(halves_tag)::value;
-        // S^T: row = key `column` of the run (tile column / 16, position column % 16), 8 dims (chunk 2 ks + half) per lane.
-        const bf16* k_rows = k_lds + (2 * first_run + column / 16) * TILE_ELEMENTS + (half * 16 + column % 16) * 8;
+        // The instances of this body begin with the same reads from LDS. Where two of them are the two sides of a
+        // branch the compiler would lift those reads above the branch, and a read made one from two no longer
+        // says which LDS variable it reads: it then waits for every load that is on its way into the other stage.
+        // Different lines at the top of each instance keep the reads where they are.
+        if (MASKED) asm volatile("; one run of keys, masked");
+        else if (HALVES == 2) asm volatile("; two runs of keys");
+        else asm volatile("; one run of keys");
+        const bf16* k_rows = (stage + k_lane) + 2 * first_run * TILE_ELEMENTS;
         floatx16 s[HALVES];
 #pragma unroll
         for (int r = 0; r < HALVES; ++r)
@@ -286,13 +306,13 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             if (j + kAhead < PRODUCTS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
-        // s[r][i]: key key0 + 32 r + 8 (i / 4) + 4 half + i % 4, token `column`.
+        // s[r][i] is row 8 (i / 4) + 4 half + i % 4: key key0 + 32 r + 16 (i / 8) + 8 half + i % 8, token `column`.
         if (MASKED) {
 #pragma unroll
             for (int r = 0; r < HALVES; ++r)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const int key = key0 + 32 * r + 8 * (i / 4) + 4 * half + (i % 4);
+                    const int key = key0 + 32 * r + 16 * (i / 8) + 8 * half + (i % 8);
                     if (key > my_position || key < my_low) s[r][i] = -INFINITY;
                 }
         }
@@ -335,19 +355,19 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
 #pragma unroll
             for (int d = 0; d < D_BLOCKS; ++d) o_acc[d] *= rescale;
         }
-        // O^T += V^T . P^T, 16 keys (one tile) a product: row = dim `column` of a block of 32 dims; the lane's 8
-        // k-slots are the keys its scores came for: positions 4 half .. + 3 and 8 + 4 half .. + 3 of the tile.
-        const bf16* v_rows = v_lds + 2 * first_run * TILE_ELEMENTS + (column / 16) * 256 + (column % 16) * 4 + half * 64;
+        // O^T += V^T . P^T, 16 keys (one tile) a product.
+        const bf16* v_rows = (stage + v_lane) + (HALF_CHUNKS * 8 + 2 * first_run * TILE_ELEMENTS);
 #pragma unroll
         for (int t = 0; t < 2 * HALVES; ++t)
 #pragma unroll
             for (int d = 0; d < D_BLOCKS; ++d) {
                 PFrag8 v_frag;
                 v_frag.raw = make_uint4(0, 0, 0, 0);
-                if (HD % 32 == 0 || d * 32 + column < HD) {
-                    const bf16* v_row = v_rows + t * TILE_ELEMENTS + d * 512;
-                    v_frag.h[0] = *reinterpret_cast<const bf16x4*>(v_row);
-                    v_frag.h[1] = *reinterpret_cast<const bf16x4*>(v_row + 128);
+                if (HD % 32 == 0 || d < D_BLOCKS - 1) {
+                    v_frag.raw = *reinterpret_cast<const uint4*>(v_rows + t * TILE_ELEMENTS + d * 512);
+                } else if (column < 16) {      // the last block has 16 dims: [position / 8][16][8]
+                    v_frag.raw = *reinterpret_cast<const uint4*>((stage + (half * 16 + column) * 8) +
+                                                                 (HALF_CHUNKS * 8 + (2 * first_run + t) * TILE_ELEMENTS + d * 512));
                 }
                 o_acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v_frag.v, p_frag[t].v, o_acc[d], 0, 0, 0);
             }
@@ -358,17 +378,17 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
         while (block * BLOCK_KEYS <= group_last && !block_seen(block)) ++block;
         return block;
     };
+    // (The lambdas above and below are marked always_inline: left to its own count of instructions the compiler
+    // makes a function of one of them, whose call then costs registers kept in memory.)
     // One block: the next one is sent for, this one is used. Called by turns with the stages exchanged.
     int block = first_block;
     int following = next_seen(first_block);
-    auto walk = [&](const bf16* stage, bf16* next_stage) {
+    auto walk = [&](const bf16* stage, bf16* next_stage) __attribute__((always_inline)) {
         if (following <= last_block) {
             fetch(following, next_stage);
             const int after = next_seen(following);
             if (after <= last_block) look_up(after);
         }
-        const bf16* k_lds = stage;
-        const bf16* v_lds = stage + HALF_CHUNKS * 8;
         // Unrolled: every read from LDS then has the stage's own address plus a constant, and the compiler can tell
         // that the loads on their way into the other stage do not touch it (of an address that a loop carries along
         // it cannot, and waits for those loads before the first read).
@@ -382,13 +402,13 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
                 hidden[r] = key0 + 32 * r + 31 > block_position || key0 + 32 * r < block_last_low;
             }
             if (see[0] && see[1] && !hidden[0] && !hidden[1]) {
-                process_keys(std::false_type{}, std::integral_constant<int, 2>{}, k_lds, v_lds, 2 * pair, key0);
+                process_keys(std::false_type{}, std::integral_constant<int, 2>{}, stage, 2 * pair, key0);
             } else {
 #pragma unroll
                 for (int r = 0; r < 2; ++r) {
                     if (!see[r]) continue;      // nothing of this run is visible to the wave
-                    if (hidden[r]) process_keys(std::true_type{}, std::integral_constant<int, 1>{}, k_lds, v_lds, 2 * pair + r, key0 + 32 * r);
-                    else process_keys(std::false_type{}, std::integral_constant<int, 1>{}, k_lds, v_lds, 2 * pair + r, key0 + 32 * r);
+                    if (hidden[r]) process_keys(std::true_type{}, std::integral_constant<int, 1>{}, stage, 2 * pair + r, key0 + 32 * r);
+                    else process_keys(std::false_type{}, std::integral_constant<int, 1>{}, stage, 2 * pair + r, key0 + 32 * r);
                 }
             }
         }

@@ -51,7 +51,7 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_kernel(
             const int64_t page = table[key / page_size];
             const int offset = key % page_size;
             const T* k_tile = k_cache + layout.k_tile(page, kv_head, offset / 16);
-            v_column = layout.v_tile(page, kv_head, offset / 16) + CacheLayout::v_in_tile(offset % 16, 0);
+            v_column = layout.v_tile(page, kv_head, offset / 16) + offset % 16;      // the tile (a multiple of 16) and the place in it
             float dot = 0.0f;
             for (int d = 0; d < head_dim; ++d) dot += q_shared[d] * to_float(k_tile[CacheLayout::k_in_tile(offset % 16, d)]);
             score = dot * scale;
@@ -73,8 +73,8 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_kernel(
             const int d = lane + i * kWave;
             if (d < head_dim) {
                 float value = acc[i] * rescale;
-                const int v_dim = ((d / 16) * 64 + d % 16) * 4;   // CacheLayout::v_in_tile(0, d)
-                for (int j = first; j <= last; ++j) value += p_shared[j] * to_float(v_cache[v_shared[j] + v_dim]);
+                for (int j = first; j <= last; ++j)
+                    value += p_shared[j] * to_float(v_cache[(v_shared[j] & ~int64_t(15)) + layout.v_in_tile(static_cast<int>(v_shared[j] & 15), d)]);
                 acc[i] = value;
             }
         }

@@ -3,8 +3,11 @@
 // contiguous piece of memory:
 //   keys:   [page][kv_head][tile][dim / 8][position % 16][dim % 8]
 //           (lane (position, quad) of a wave reads 8 dims = 16 bytes of chunk 4 * k_step + quad)
-//   values: [page][kv_head][tile][dim / 16][(position % 16) / 4][dim % 16][position % 4]
-//           (lane (dim, quad) reads the 4 positions 4 * quad .. + 3 = 8 bytes for bfloat16)
+//   values: [page][kv_head][tile][dim / 32][(position % 16) / 8][dim % 32][position % 8]
+//           (lane (dim, half) of a wave reads the 8 positions 8 * half .. + 7 = 16 bytes for bfloat16, the 8
+//           k-slots it supplies to one product, and the 64 lanes of a wave read 1024 consecutive bytes, which
+//           LDS gives without bank conflicts; the keys' rows are taken in the order that makes the scores come
+//           out so. A last block of 16 dims, where head_dim is an odd multiple of 16, is [position / 8][16][8].)
 // head_dim is padded to a multiple of 8 (keys) or 16 (values); the padding is never read as data.
 #pragma once
 
@@ -33,9 +36,12 @@ struct CacheLayout {
     }
     // Element offsets inside a tile.
     __host__ __device__ static int k_in_tile(int position16, int dim) { return ((dim / 8) * 16 + position16) * 8 + dim % 8; }
-    __host__ __device__ static int v_in_tile(int position16, int dim) {
-        return (((dim / 16) * 4 + position16 / 4) * 16 + dim % 16) * 4 + position16 % 4;
+    __host__ __device__ int v_in_tile(int position16, int dim) const {
+        const int block = dim / 32;
+        const int width = min_int(32, v_dim_tiles * 16 - 32 * block);      // dims of this block: 32, or 16 in a last half block
+        return block * 512 + ((position16 / 8) * width + dim % 32) * 8 + position16 % 8;
     }
+    __host__ __device__ static int min_int(int a, int b) { return a < b ? a : b; }
     __host__ __device__ int64_t k_at(int64_t page, int kv_head, int offset, int dim) const {
         return k_tile(page, kv_head, offset / 16) + k_in_tile(offset % 16, dim);
     }

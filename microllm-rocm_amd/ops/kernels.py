@@ -304,7 +304,7 @@ def _check_pages(k_cache, v_cache, dtype, kv_heads, head_dim, page_size=None) ->
     from ..cache.layout import key_page_shape, value_page_shape
     _device_tensor(k_cache, "key pages", dtype)
     _device_tensor(v_cache, "value pages", dtype)
-    _need(k_cache.dim() == 6 and v_cache.dim() == 7, "key pages must have 6 dimensions and value pages 7 (tiled layout)")
+    _need(k_cache.dim() == 6 and v_cache.dim() == 4, "key pages must have 6 dimensions and value pages 4 (tiled layout)")
     found = k_cache.shape[2] * 16
     _need(page_size is None or page_size == found, "the pages do not have the page size given")
     pages = k_cache.shape[0]
