@@ -49,17 +49,24 @@ int mll_qkv_rope_store(const void* qkv, int in_dtype, int n_partials, int64_t pa
                        int n_tokens, int heads, int kv_heads, int head_dim, int page_size, int pair_order,
                        hipStream_t stream);
 
-// Attention of every query token over its request's pages, one wave per (token, head).
+// Attention of every query token over its request's pages, for any dtype and head size.
 // Key j is visible to a query at position p iff j <= p and (window <= 0 or p - j < window).
 // block_table[seq, j / page_size] gives the page of key j. Reduction order depends only on
-// (p, window), so the result does not depend on how tokens were cut into steps.
+// (p, window), so the result does not depend on how tokens were cut into steps, to the last bit.
 // A token whose seq_of_token is negative is skipped and its output row left as it is (a row that pads a step to
 // a fixed shape).
+// max_chunks 0: one wave per (token, head). max_chunks > 0: one wave per (token, head, chunk of
+// mll_paged_attention_rowwise_chunk() keys) and a second kernel that merges the chunks in the same order with
+// the same arithmetic (the same bits), for steps with few rows; no row's visible keys may then span more than
+// max_chunks chunks (chunks lie at absolute positions), and part_o [n_tokens * heads * max_chunks * head_dim]
+// and part_ml [n_tokens * heads * max_chunks * 2] floats are the workspace.
+int mll_paged_attention_rowwise_chunk();
 int mll_paged_attention_rowwise(const void* q, int dtype, const void* k_cache, const void* v_cache,
                                 const int32_t* block_table, int table_width,
                                 const int32_t* seq_of_token, const int32_t* positions, void* out,
-                                float scale, int window, int n_tokens, int heads, int kv_heads,
-                                int head_dim, int page_size, hipStream_t stream);
+                                float* part_o, float* part_ml, int max_chunks, float scale, int window,
+                                int n_tokens, int heads, int kv_heads, int head_dim, int page_size,
+                                hipStream_t stream);
 
 // The same attention for bfloat16 portions of prompts with MFMA: one workgroup per (two tiles of up to
 // mll_paged_attention_prefill_tile() consecutive tokens of one request, query head). `tiles` holds, for each

@@ -322,10 +322,26 @@ def _check_paged(q, k_cache, v_cache, block_table, heads, kv_heads, head_dim) ->
     return page_size
 
 
+ROWWISE_SPLIT_BELOW = 2048      # (token, head) rows: with fewer, a row's chunks of keys get a wave each
+
+
+def rowwise_chunks(longest: int, window: int) -> int:
+    """The most chunks of keys (at absolute positions) that a row's visible keys can span, for rows that see at
+    most ``longest`` keys' positions (position < longest)."""
+    chunk = library.load().mll_paged_attention_rowwise_chunk()
+    if window > 0:
+        return min(-(-longest // chunk), (window + chunk - 2) // chunk + 1)
+    return max(1, -(-longest // chunk))
+
+
 def paged_attention_rowwise(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                             block_table: torch.Tensor, seq_of_token: torch.Tensor, positions: torch.Tensor,
                             scale: float, window: int, heads: int, kv_heads: int, head_dim: int,
-                            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                            out: Optional[torch.Tensor] = None, longest: Optional[int] = None,
+                            split: Optional[bool] = None) -> torch.Tensor:
+    """The plain attention kernel (any dtype, any head size). ``longest``: no position of the step reaches it
+    (default: what the block table can hold). ``split``: a wave per chunk of keys and a merge, or a wave per row;
+    by default by the number of rows. Both give the same bits."""
     lib = library.load()
     page_size = _check_paged(q, k_cache, v_cache, block_table, heads, kv_heads, head_dim)
     n_tokens = q.shape[0]
@@ -337,10 +353,21 @@ def paged_attention_rowwise(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         out = torch.empty_like(q)
     _device_tensor(out, "attention output", q.dtype)
     _need(out.shape == q.shape, "attention output must have the queries' shape")
+    capacity = block_table.shape[1] * page_size
+    longest = capacity if longest is None else min(int(longest), capacity)
+    if split is None:
+        split = n_tokens * heads < ROWWISE_SPLIT_BELOW
+    chunks = rowwise_chunks(max(longest, 1), window) if split else 0
+    part_o = part_ml = None
+    if chunks > 1:
+        part_o = torch.empty((n_tokens, heads, chunks, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((n_tokens, heads, chunks, 2), dtype=torch.float32, device=q.device)
+    else:
+        chunks = 0      # one chunk a row: the wave per row is the wave per chunk
     _check(lib.mll_paged_attention_rowwise(_ptr(q), _code(q.dtype), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
                                            block_table.shape[1], _ptr(seq_of_token), _ptr(positions), _ptr(out),
-                                           ctypes.c_float(scale), int(window), n_tokens, heads, kv_heads, head_dim,
-                                           page_size, _stream()), lib)
+                                           _ptr(part_o), _ptr(part_ml), chunks, ctypes.c_float(scale), int(window),
+                                           n_tokens, heads, kv_heads, head_dim, page_size, _stream()), lib)
     return out
 
 
@@ -679,7 +706,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                    scale, window, heads, kv_heads, head_dim, splits, out=out, token_ids=plan.single_tokens)
         return out
     return paged_attention_rowwise(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
-                                   scale, window, heads, kv_heads, head_dim)
+                                   scale, window, heads, kv_heads, head_dim, longest=max(ctx.planned_total, ctx.max_total))
 
 
 def pack_weight(weight: torch.Tensor, interleave_halves: bool = False,

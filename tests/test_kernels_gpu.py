@@ -266,6 +266,32 @@ def test_rowwise_attention(dtype, heads, kv_heads, hd, page_size, window):
     np.testing.assert_allclose(out.float().cpu().numpy(), reference, **tolerance(dtype))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv_heads,hd,page_size,window", [
+    (4, 2, 16, 16, 0), (3, 1, 40, 16, 130), (6, 3, 128, 32, 0), (2, 1, 72, 16, 257), (5, 5, 48, 48, 1), (2, 2, 24, 16, 128)])
+def test_rowwise_attention_a_wave_per_chunk_gives_the_same_bits(dtype, heads, kv_heads, hd, page_size, window):
+    """The plain kernel walks a row's keys by one wave, or by a wave per chunk of 128 keys with a merge: the same
+    result to the last bit, whatever the row's position (chunk edges, one key beyond, many chunks) and window,
+    and right against the reference. What the block table could hold beyond the longest request is no key."""
+    rng = np.random.default_rng(hd * 3 + window)
+    lengths, counts = [700, 1, 128, 129, 257, 384, 127], [130, 1, 2, 3, 1, 129, 1]
+    t, q_exact, ek, ev, seq, pos = build_paged_case(rng, dtype, lengths, counts, heads, kv_heads, hd, page_size)
+    scale = 0.9 / math.sqrt(hd)
+    k = kernels()
+    chunk = k.library.load().mll_paged_attention_rowwise_chunk()
+    assert chunk == 128
+    args = (t["q"], t["k"], t["v"], t["table"], t["seq"], t["pos"], scale, window, heads, kv_heads, hd)
+    whole = k.paged_attention_rowwise(*args, split=False)
+    by_chunk = k.paged_attention_rowwise(*args, split=True, longest=max(lengths))
+    generous = k.paged_attention_rowwise(*args, split=True)      # as many chunks as the table is wide
+    assert torch.equal(whole, by_chunk) and torch.equal(whole, generous)
+    reference = reference_attention(q_exact, ek, ev, seq, pos, heads, kv_heads, hd, scale, window)
+    np.testing.assert_allclose(whole.float().cpu().numpy(), reference, **tolerance(dtype))
+    assert k.rowwise_chunks(700, 0) == 6 and k.rowwise_chunks(128, 0) == 1 and k.rowwise_chunks(129, 0) == 2
+    assert k.rowwise_chunks(5000, 1) == 1 and k.rowwise_chunks(5000, 2) == 2 and k.rowwise_chunks(5000, 129) == 2
+    assert k.rowwise_chunks(5000, 130) == 3 and k.rowwise_chunks(100, 130) == 1
+
+
 @pytest.mark.parametrize("heads,kv_heads,hd,page_size,window,splits", [
     (4, 2, 16, 16, 0, 1), (3, 1, 32, 16, 24, 2), (5, 5, 48, 16, 100, 3), (28, 4, 128, 16, 0, 8), (14, 2, 64, 32, 0, 5),
     (16, 1, 80, 16, 300, 4), (20, 1, 16, 48, 0, 2), (2, 2, 256, 16, 0, 7), (7, 7, 112, 64, 129, 1), (6, 3, 96, 16, 0, 64)])
