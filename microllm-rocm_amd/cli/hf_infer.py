@@ -9,8 +9,9 @@ standard output. Options the reference has keep their names and meanings; what t
 ``--use-cache false`` generates by running every sequence whole for each new token (the reference's oracle for
 its cached path), ``--cache-prefill-mode token`` feeds the prompt one token a step, ``--prefill-logits full`` computes
 the logits of every prompt position, ``--batch-argmax-mode host`` picks tokens from logits copied to the host,
-``--cache-logits-output`` writes the last decode step's logits, and ``--bf16-ffn`` with ``--bf16-attention``
-choose the precision as ``--dtype`` does (apps/hf_infer.cpp:52-57, 1121-1123, 1238-1305).
+``--cache-logits-output`` writes the last decode step's logits, ``--bf16-ffn`` with ``--bf16-attention``
+choose the precision as ``--dtype`` does (apps/hf_infer.cpp:52-57, 1121-1123, 1238-1305), and ``--trace-output``
+writes a value trace of one prefill, a JSON line per layer and one for the logits (apps/hf_infer.cpp:1132-1160).
 
 Workloads (``--workload``): ``prefill`` times the prompt alone, ``decode`` times steady decoding after it,
 ``both`` (default) generates ``--new-tokens`` tokens after the prompt, ``continuous`` serves several requests
@@ -34,6 +35,7 @@ OPTIONS: Dict[str, object] = {
     "continuous-prompt-offsets": "", "continuous-arrival-steps": "",
     "use-cache": "true", "cache-prefill-mode": "full", "prefill-logits": "last", "batch-argmax-mode": "device",
     "cache-logits-output": None, "bf16-ffn": None, "bf16-attention": None,
+    "trace-output": None, "trace-max-elements": 4096,
     # this engine's own
     "model": None, "dtype": "bfloat16", "temperature": 0.0, "sample-top-k": 0, "seed": 1, "stop-tokens": "",
     "block-size": 16, "num-blocks": 0, "max-batched-tokens": 2048, "prefill-chunk": 512, "max-requests": 64,
@@ -79,6 +81,34 @@ def percentile(values, quantile: float) -> float:
     lower, upper = int(math.floor(position)), int(math.ceil(position))
     fraction = position - lower
     return ordered[lower] * (1.0 - fraction) + ordered[upper] * fraction
+
+
+def trace_record(sequence: int, kind: str, name: str, tensor, max_elements: int) -> dict:
+    """One record of the value trace: what the tensor is, its statistics and its first values, with the reference's
+    field names (src/profiling/trace.cpp:156-196; include/microllm/profiling/trace.h:25-47)."""
+    import torch
+    values = tensor.detach().to(torch.float64).flatten()
+    finite = values[torch.isfinite(values)]
+    some = finite.numel() > 0
+    first = values[:max_elements].cpu().tolist()
+    return {"schema_version": 1, "framework": "microllm_rocm_amd", "run_id": "hf-prefill", "phase": "inference-values",
+            "sequence": sequence, "iteration": 0, "kind": kind, "name": name, "shape": list(tensor.shape),
+            "dtype": str(tensor.dtype).replace("torch.", ""), "device": str(tensor.device), "wall_ms": 0.0,
+            "statistics": {"numel": values.numel(), "finite_count": finite.numel(),
+                           "minimum": float(finite.min()) if some else 0.0, "maximum": float(finite.max()) if some else 0.0,
+                           "mean": float(finite.mean()) if some else 0.0, "l2_norm": float(finite.square().sum().sqrt())},
+            "values_truncated": values.numel() > max_elements,
+            "values": [value if math.isfinite(value) else ("nan" if math.isnan(value) else ("inf" if value > 0 else "-inf"))
+                       for value in first]}
+
+
+def write_trace(path: str, records: List[dict]) -> None:
+    folder = os.path.dirname(path)
+    if folder:
+        os.makedirs(folder, exist_ok=True)
+    with open(path, "w", encoding="utf-8") as handle:
+        for record in records:
+            handle.write(json.dumps(record) + "\n")
 
 
 def integers(text: str, what: str) -> List[int]:
@@ -138,6 +168,11 @@ def run(options: Dict[str, object]) -> int:
                           ("batch-argmax-mode", ("device", "host"))):
         if options[name] not in allowed:
             raise UsageError(f"--{name} must be {' or '.join(allowed)}")      # apps/hf_infer.cpp:194-202
+    if int(options["trace-max-elements"]) <= 0:
+        raise UsageError("--trace-max-elements must be positive")      # apps/hf_infer.cpp:265-266
+    if options["trace-output"] and (options["workload"] != "prefill" or int(options["prefill-warmup"]) != 0
+                                    or int(options["prefill-steps"]) != 1):
+        raise UsageError("--trace-output requires prefill workload, zero prefill warmup, and one prefill step")   # :268-272
     if options["workload"] == "continuous" and not use_cache:
         raise UsageError("the continuous workload needs --use-cache true")      # apps/hf_infer.cpp:241
     if options["cache-logits-output"] and (not use_cache or options["workload"] == "prefill" or int(options["new-tokens"]) < 2):
@@ -277,11 +312,20 @@ def run(options: Dict[str, object]) -> int:
             # --prefill-logits full: the logits of every position are computed, last: of the last alone; the
             # report and --logits-output take the last row either way (apps/hf_infer.cpp:1121-1123, 1166-1181)
             every = options["prefill-logits"] == "full"
+            records = []
+            if options["trace-output"]:
+                engine.observe_layers(lambda index, stream: records.append(trace_record(
+                    len(records), "layer", f"run_entry.{index}", stream.view(batch, len(tokens), -1), int(options["trace-max-elements"]))))
             logits = engine.step([StepEntry(request_id, prompt, list(range(len(prompt))) if every else [len(prompt) - 1])
                                   for request_id, prompt in zip(ids, prompts)])
             if every:
                 logits = logits.view(batch, len(tokens), -1)[:, -1]
             torch.cuda.synchronize()
+            if options["trace-output"]:
+                engine.observe_layers(None)
+                records.append(trace_record(len(records), "model", "logits", logits, int(options["trace-max-elements"])))
+                write_trace(str(options["trace-output"]), records)
+                report["trace_records"] = len(records)
             if iteration >= int(options["prefill-warmup"]):
                 timings.append(time.perf_counter() - begun)
             for request_id in ids:

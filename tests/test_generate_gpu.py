@@ -227,6 +227,42 @@ def test_command_line_ways_of_generating(tmp_path, capsys):
         assert "microllm_hf_infer:" in capsys.readouterr().err
 
 
+def test_command_line_value_trace(tmp_path, capsys):
+    """--trace-output: one JSON line per layer with the residual stream after it and one for the logits, with the
+    reference's field names; values and statistics against the plain implementation."""
+    from microllm_rocm_amd.cli import hf_infer
+    folder = make_folder(tmp_path, "B", SHARP)
+    model = PlainModel(folder)
+    config = CONFIGS["B"]
+    prompt = random_tokens(8, 21, config.vocab_size)
+    trace = tmp_path / "deep" / "trace.jsonl"
+    base = ["--model", folder, "--tokens", ",".join(map(str, prompt)), "--dtype", "float32", "--workload", "prefill",
+            "--trace-output", str(trace)]
+    capsys.readouterr()
+    assert hf_infer.main(base + ["--trace-max-elements", "50"]) == 0
+    report = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    records = [json.loads(line) for line in trace.read_text().splitlines()]
+    assert report["trace_records"] == len(records) == config.num_hidden_layers + 1
+    streams = plain.layer_streams(model.config, model.weights, prompt)
+    for layer, record in enumerate(records[:-1]):
+        assert (record["sequence"], record["kind"], record["shape"]) == (layer, "layer", [1, len(prompt), config.hidden_size])
+        assert record["values_truncated"] and len(record["values"]) == 50
+        expected = streams[layer].reshape(-1)
+        scale = np.abs(expected).max()
+        assert np.abs(np.array(record["values"]) - expected[:50]).max() <= 2e-5 * scale
+        statistics = record["statistics"]
+        assert statistics["numel"] == statistics["finite_count"] == expected.size
+        assert abs(statistics["l2_norm"] - np.sqrt((expected ** 2).sum())) <= 2e-5 * np.sqrt((expected ** 2).sum())
+        assert abs(statistics["minimum"] - expected.min()) <= 2e-5 * scale and abs(statistics["maximum"] - expected.max()) <= 2e-5 * scale
+    last = records[-1]
+    reference = model.logits(prompt)[-1]
+    assert last["kind"] == "model" and last["shape"] == [1, config.vocab_size]
+    assert np.abs(np.array(last["values"]) - reference[:50]).max() <= 2e-5 * np.abs(reference).max()
+    for bad in (["--trace-max-elements", "0"], ["--prefill-steps", "2"], ["--workload", "both"]):
+        assert hf_infer.main(base + bad) == 2, bad
+        assert "microllm_hf_infer:" in capsys.readouterr().err
+
+
 def test_step_refuses_bad_batches_and_leaves_the_cache_as_it_was(tmp_path):
     from microllm_rocm_amd import StepEntry
     from microllm_rocm_amd.cache import OutOfPages
