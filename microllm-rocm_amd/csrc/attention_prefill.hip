@@ -261,27 +261,22 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     // must be rescaled, and their two chains of products hide each other's latency. MASKED: some key is hidden
     // from some token (the causal diagonal, the window's edge, the end of the sequence).
     // Scores stay in the product's units; p = 2^((s - max) * scale_log2) is one multiply-add and one exponent.
-    // Where a lane reads its operands in a stage, but for the run. The address of every read is the stage's own
-    // variable, plus this, plus a constant: the compiler follows an address back to its LDS variable over a few
-    // additions only, and a read that it cannot place waits for all loads on their way into either stage.
     // First product: row `column` = the key of the run whose number is `column` with bits 2 and 3 exchanged (tile
     // column / 16), 8 dims (chunk 2 ks + half) per lane. Second: row = dim `column` of a block of 32 dims; the
     // lane's 8 k-slots are the keys its scores came for, positions 8 half .. + 7 of the tile, one read of 16 bytes;
     // the 64 lanes read 1024 consecutive bytes, which LDS gives without bank conflicts.
+    // The addresses are formed step by step (stage, then tile, then lane). The compiler follows an address back
+    // to its LDS variable over a few additions only, and of a read that it cannot place it assumes that the loads
+    // on their way into the other stage may write it: the first reads of every run of keys therefore wait for
+    // those loads. Formed as one sum (stage plus a per-lane term plus a constant) the reads do not wait, and the
+    // kernel is 5 % slower (836 against 791 us for 8192 tokens, 2680 against 2545 for 16384; waiting for the
+    // loads in other places does not give the same). Measured, not understood: the waits seem to shift the two
+    // waves of a SIMD against each other, so that one's matrix work meets the other's vector work.
     const int key_of_row = (column & ~12) | ((column & 4) << 1) | ((column & 8) >> 1);
-    const int k_lane = (column / 16) * TILE_ELEMENTS + (half * 16 + key_of_row % 16) * 8;
-    const int v_lane = (half * 32 + column) * 8;      // in a block of 32 dims; a last block of 16 has its own
     auto process_keys = [&](auto masked_tag, auto halves_tag, const bf16* stage, int first_run, int key0) __attribute__((always_inline)) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         constexpr int HALVES = decltype(halves_tag)::value;
-        // The instances of this body begin with the same reads from LDS. Where two of them are the two sides of a
-        // branch the compiler would lift those reads above the branch, and a read made one from two no longer
-        // says which LDS variable it reads: it then waits for every load that is on its way into the other stage.
-        // Different lines at the top of each instance keep the reads where they are.
-        if (MASKED) asm volatile("; one run of keys, masked");
-        else if (HALVES == 2) asm volatile("; two runs of keys");
-        else asm volatile("; one run of keys");
-        const bf16* k_rows = (stage + k_lane) + 2 * first_run * TILE_ELEMENTS;
+        const bf16* k_rows = stage + (2 * first_run + column / 16) * TILE_ELEMENTS + (half * 16 + key_of_row % 16) * 8;
         floatx16 s[HALVES];
 #pragma unroll
         for (int r = 0; r < HALVES; ++r)
@@ -356,7 +351,7 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
             for (int d = 0; d < D_BLOCKS; ++d) o_acc[d] *= rescale;
         }
         // O^T += V^T . P^T, 16 keys (one tile) a product.
-        const bf16* v_rows = (stage + v_lane) + (HALF_CHUNKS * 8 + 2 * first_run * TILE_ELEMENTS);
+        const bf16* v_rows = stage + HALF_CHUNKS * 8 + 2 * first_run * TILE_ELEMENTS + column * 8 + half * 256;
 #pragma unroll
         for (int t = 0; t < 2 * HALVES; ++t)
 #pragma unroll
@@ -389,9 +384,8 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
             const int after = next_seen(following);
             if (after <= last_block) look_up(after);
         }
-        // Unrolled: every read from LDS then has the stage's own address plus a constant, and the compiler can tell
-        // that the loads on their way into the other stage do not touch it (of an address that a loop carries along
-        // it cannot, and waits for those loads before the first read).
+        // Unrolled: every read from LDS then has an address of the stage plus a constant (an address that a loop
+        // carries along would make every read wait for the loads on their way into the other stage).
 #pragma unroll
         for (int pair = 0; pair < STEPS / 2; ++pair) {
             const int key0 = block * BLOCK_KEYS + 64 * pair;
