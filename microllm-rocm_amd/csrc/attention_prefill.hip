@@ -270,8 +270,8 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     // on their way into the other stage may write it: the first reads of every run of keys therefore wait for
     // those loads. Formed as one sum (stage plus a per-lane term plus a constant) the reads do not wait, and the
     // kernel is 5 % slower (836 against 791 us for 8192 tokens, 2680 against 2545 for 16384; waiting for the
-    // loads in other places does not give the same). Measured, not understood: the waits seem to shift the two
-    // waves of a SIMD against each other, so that one's matrix work meets the other's vector work.
+    // loads in other places does not give the same, nor does holding one tile's waves back for a while at the
+    // start of a block). Measured, not understood.
     const int key_of_row = (column & ~12) | ((column & 4) << 1) | ((column & 8) >> 1);
     auto process_keys = [&](auto masked_tag, auto halves_tag, const bf16* stage, int first_run, int key0) __attribute__((always_inline)) {
         constexpr bool MASKED = decltype(masked_tag)::value;
