@@ -75,14 +75,32 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     __shared__ __align__(16) bf16 stage_even[STAGE_ELEMENTS];
     __shared__ __align__(16) bf16 stage_odd[STAGE_ELEMENTS];
 
-    const int32_t* entry = tiles + 5 * blockIdx.x;
+    // Which entry and head this workgroup takes. Workgroups go to the GPU's 8 dies (each with a second-level cache
+    // of its own) by turns, in the order of their number; numbered entry-first, every die would read every kv
+    // head's keys and values. Instead a die takes the query heads of one kv head (of 8 / kv_heads dies each), the
+    // entries still in the list's order (longest first): a long prompt's keys then mostly come from the die's own
+    // cache (8192 tokens at 7B sizes: 800 -> 680 us; 16384: 2650 -> 2340). Where the numbers do not divide, the
+    // workgroups keep their plain numbering.
+    int entry_index = blockIdx.x, head = blockIdx.y;
+    {
+        constexpr int kDies = 8;
+        const int group = heads / kv_heads;
+        const int dies_per_kv_head = kv_heads <= kDies && kDies % kv_heads == 0 ? kDies / kv_heads : 0;
+        if (dies_per_kv_head > 0 && (gridDim.x * group) % dies_per_kv_head == 0) {
+            const int number = blockIdx.x + gridDim.x * blockIdx.y;
+            const int die = number % kDies, turn = number / kDies;
+            const int item = turn * dies_per_kv_head + die % dies_per_kv_head;      // among the kv head's entries x heads
+            entry_index = item / group;
+            head = (die / dies_per_kv_head) * group + item % group;
+        }
+    }
+    const int32_t* entry = tiles + 5 * entry_index;
     if (entry[2] <= 0 && entry[4] <= 0) return;      // an entry that only pads the list to a fixed length
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
     const int column = lane % 32;     // token of the block (B operands, results) or key / dim row (A operands)
     const int half = lane / 32;       // which 8 of a step's 16 k-slots this lane supplies
     const int seq = entry[0];
-    const int head = blockIdx.y;
     const int kv_head = head / (heads / kv_heads);
     const int32_t* table = block_table + static_cast<int64_t>(seq) * table_width;
     const float scale_log2 = scale * 1.4426950408889634f;      // scores are kept in units of log 2: p = 2^(s - max)
