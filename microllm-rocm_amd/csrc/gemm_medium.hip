@@ -31,7 +31,7 @@ union Piece {
 
 __device__ inline float silu_f(float value) { return value / (1.0f + __expf(-value)); }
 
-template <int NT, bool TEMPORAL>
+template <int NT>
 __device__ inline void load_batch(Piece (&pieces)[kBatch][NT], const bf16* const (&w_ptr)[NT], const bool (&w_live)[NT],
                                   int first_step, int end_step) {
 #pragma unroll
@@ -42,7 +42,7 @@ __device__ inline void load_batch(Piece (&pieces)[kBatch][NT], const bf16* const
             pieces[u][nt].raw = uintx4{0u, 0u, 0u, 0u};
             if (ks < end_step && w_live[nt]) {
                 const uintx4* source = reinterpret_cast<const uintx4*>(w_ptr[nt] + static_cast<int64_t>(ks) * 512);
-                pieces[u][nt].raw = TEMPORAL ? *source : __builtin_nontemporal_load(source);
+                pieces[u][nt].raw = __builtin_nontemporal_load(source);      // W is read once a step: past the caches
             }
         }
     }
@@ -50,7 +50,7 @@ __device__ inline void load_batch(Piece (&pieces)[kBatch][NT], const bf16* const
 
 // EPILOGUE: 0 = float32 [splits][M, N]; 1 = bfloat16 [M, N]; 2 = bfloat16 [M, N / 2] = silu(even rows of W) * (odd
 // rows). 1 and 2 need splits == 1.
-template <int MT, int NT, int kWaves, int EPILOGUE, bool TEMPORAL>
+template <int MT, int NT, int kWaves, int EPILOGUE>
 __global__ __launch_bounds__(kWaves * kWave) void gemm_medium_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w_packed, void* __restrict__ out,
     int m, int n, int k, int n_tiles, int k_steps, int steps_per_split) {
@@ -118,16 +118,16 @@ __global__ __launch_bounds__(kWaves * kWave) void gemm_medium_kernel(
     uintx4 share[kPiecesPerWave];
     Piece w_even[kBatch][NT], w_odd[kBatch][NT];
     load_share(share, first_step);
-    load_batch<NT, TEMPORAL>(w_even, w_ptr, w_live, first_step, end_step);
+    load_batch<NT>(w_even, w_ptr, w_live, first_step, end_step);
     store_share(share, 0);
     __syncthreads();
     for (int s = 0; s < n_stages; ++s) {
         const int stage_step = first_step + s * kStepsPerStage;
         const int buffer = s % 2;
         if (s + 1 < n_stages) load_share(share, stage_step + kStepsPerStage);
-        load_batch<NT, TEMPORAL>(w_odd, w_ptr, w_live, stage_step + kBatch, end_step);
+        load_batch<NT>(w_odd, w_ptr, w_live, stage_step + kBatch, end_step);
         multiply(w_even, buffer, 0);
-        load_batch<NT, TEMPORAL>(w_even, w_ptr, w_live, stage_step + kStepsPerStage, end_step);
+        load_batch<NT>(w_even, w_ptr, w_live, stage_step + kStepsPerStage, end_step);
         multiply(w_odd, buffer, kBatch);
         // The other buffer was last read in the stage before this one, and every wave has passed that stage's barrier.
         if (s + 1 < n_stages) store_share(share, 1 - buffer);
@@ -180,11 +180,7 @@ static void launch_one(const bf16* a, const bf16* w, void* out, int m, int n, in
     const int stages = (k_steps + kStepsPerStage - 1) / kStepsPerStage;
     const int steps_per_split = ((stages + splits - 1) / splits) * kStepsPerStage;
     const size_t lds = 2 * MT * kStepsPerStage * kWave * sizeof(uintx4);
-    const bool temporal = static_cast<int64_t>(n_tiles) * k_steps * 1024 < (64ll << 20);   // bytes of the packed weight
-    if (temporal)
-        gemm_medium_kernel<MT, NT, kWaves, EPILOGUE, true><<<grid, kWaves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps, steps_per_split);
-    else
-        gemm_medium_kernel<MT, NT, kWaves, EPILOGUE, false><<<grid, kWaves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps, steps_per_split);
+    gemm_medium_kernel<MT, NT, kWaves, EPILOGUE><<<grid, kWaves * kWave, lds, stream>>>(a, w, out, m, n, k, n_tiles, k_steps, steps_per_split);
 }
 
 template <int EPILOGUE>

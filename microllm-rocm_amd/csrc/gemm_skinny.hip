@@ -37,9 +37,10 @@ __device__ inline float silu_f(float value) {
 // with each workgroup's share of the rows' sums of squares (at most 16 rows; see MllResidualNorm).
 // Whatever the epilogue, a row of the product is first multiplied by the factor that MllRowScale describes,
 // if one is given (at most 16 rows).
-// TEMPORAL: W is read with ordinary loads instead of non-temporal ones (measured on MI355X: better for weights
-// of a few tens of MB, worse for the large ones).
-template <int MT, int NT, int EPILOGUE, bool TEMPORAL, bool SCALED, bool PAIRED>
+// W is read past the caches (non-temporal loads): a step reads every weight once, and all of them together are far
+// more than the caches hold. Measured on MI355X inside the decode step, against ordinary loads for weights under 64 MB:
+// 7B sizes +1 % at batch 8, +1.6 % at batch 1, +0.7 % at batch 64; 0.5B sizes +4 % at batch 1, the same otherwise.
+template <int MT, int NT, int EPILOGUE, bool SCALED, bool PAIRED>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w_packed, void* __restrict__ out,
     int m, int n, int k, int n_tiles, int k_steps, MllSkinnyExtras extras) {
@@ -148,10 +149,8 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(
                 for (int nt = 0; nt < NT; ++nt) {
                     w_piece[u][nt].raw = uintx4{0u, 0u, 0u, 0u};
                     if (live && w_live[nt])
-                        w_piece[u][nt].raw =
-                            TEMPORAL ? *reinterpret_cast<const uintx4*>(w_ptr[nt] + static_cast<int64_t>(ks) * 512)
-                                     : __builtin_nontemporal_load(
-                                           reinterpret_cast<const uintx4*>(w_ptr[nt] + static_cast<int64_t>(ks) * 512));
+                        w_piece[u][nt].raw = __builtin_nontemporal_load(
+                            reinterpret_cast<const uintx4*>(w_ptr[nt] + static_cast<int64_t>(ks) * 512));
                 }
                 if constexpr (PAIRED) {
                     // a_piece[u] of an even u: rows 0..7 (both steps of the pair); of the odd u after it: rows 8..15
@@ -344,29 +343,22 @@ static void launch_one(const bf16* a, const bf16* w, void* out, int m, int n, in
     int waves = 1;
     while (waves < 16 && n_tiles * waves * 2 <= 16384 && waves * 2 * kChunk <= k_steps) waves *= 2;
     size_t lds = waves > 1 ? static_cast<size_t>(waves - 1) * NT * MT * kWave * sizeof(floatx4) : 0;
-    const bool temporal = static_cast<int64_t>(n_tiles) * k_steps * 1024 < (64ll << 20);   // bytes of the packed weight
     const bool scaled = extras.scale.sumsq != nullptr;
     // PAIRED pays from three rows on (measured on MI355X: 18944 x 3584 at 8 rows 27 -> 25.6 us, at 16 rows 34 -> 30.7;
     // at one row 22.8 -> 24.4).
-#define MLL_SKINNY_LAUNCH(TEMPORAL_, SCALED_, PAIRED_)                                                                 \
-    gemm_skinny_kernel<MT, NT, EPILOGUE, TEMPORAL_, SCALED_, PAIRED_><<<groups, waves * kWave, lds, stream>>>(         \
+#define MLL_SKINNY_LAUNCH(SCALED_, PAIRED_)                                                                            \
+    gemm_skinny_kernel<MT, NT, EPILOGUE, SCALED_, PAIRED_><<<groups, waves * kWave, lds, stream>>>(                    \
         a, w, out, m, n, k, n_tiles, k_steps, extras)
     if constexpr (MT == 1) {
         const bool paired = m > 2;
         if (scaled) {
             lds += (static_cast<size_t>(m) * extras.scale.stride * sizeof(float) + 1023) / 1024 * 1024;
-            if (temporal) {
-                if (paired) MLL_SKINNY_LAUNCH(true, true, true); else MLL_SKINNY_LAUNCH(true, true, false);
-            } else {
-                if (paired) MLL_SKINNY_LAUNCH(false, true, true); else MLL_SKINNY_LAUNCH(false, true, false);
-            }
-        } else if (temporal) {
-            if (paired) MLL_SKINNY_LAUNCH(true, false, true); else MLL_SKINNY_LAUNCH(true, false, false);
+            if (paired) MLL_SKINNY_LAUNCH(true, true); else MLL_SKINNY_LAUNCH(true, false);
         } else {
-            if (paired) MLL_SKINNY_LAUNCH(false, false, true); else MLL_SKINNY_LAUNCH(false, false, false);
+            if (paired) MLL_SKINNY_LAUNCH(false, true); else MLL_SKINNY_LAUNCH(false, false);
         }
     } else {
-        if (temporal) MLL_SKINNY_LAUNCH(true, false, false); else MLL_SKINNY_LAUNCH(false, false, false);
+        MLL_SKINNY_LAUNCH(false, false);
     }
 #undef MLL_SKINNY_LAUNCH
 }
