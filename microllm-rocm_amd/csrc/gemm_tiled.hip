@@ -1,16 +1,25 @@
 // Matrix products with many rows (prompts): C = A . W^T for bfloat16 A [M, K] (row-major) and the same packed
 // weight the streaming kernel reads ([N/16][K/32][4][16][8]), on v_mfma_f32_16x16x32_bf16.
 //
-// A workgroup of 8 waves (two on every SIMD, so that one wave's reads from LDS run beside the other's products)
-// owns a 256 x 256 tile of C, a wave 128 x 64 of it (8 x 4 MFMA tiles, 128 accumulator registers). Per stage of
-// 64 of k the workgroup's 2 x (16 + 16) pieces of A and W (1 KB each: 16 rows x 32 k in MFMA operand order) are
-// brought into LDS by direct global-to-LDS loads, one piece per wave-wide instruction, two stages deep (128 KB):
-// the next stage's pieces arrive while this stage's 64 products per wave run. The stages are separate LDS
-// variables: of one array the compiler cannot tell that a load into one half does not write what is read from
-// the other, and waits for the load before every read. A piece of W is contiguous in memory as it is; a piece of
-// A is gathered from 16 rows, 64 bytes of each. Addresses are a base the scalar unit steps along k and one
-// offset per lane and piece.
-// Workgroups that share a tile of W are numbered so that they run on the same XCD and share its L2.
+// A workgroup of 8 waves (two on every SIMD) owns a 256 x 256 tile of C, a wave 128 x 64 of it (8 x 4 MFMA tiles,
+// 128 accumulator registers). k is walked in stages of 64. A stage's 256 rows of A and of W (64 KB) are brought
+// into one of two LDS slots by direct global-to-LDS loads, 1 KB a wave-wide instruction: of A 8 rows of 128 bytes
+// (whole cache lines: with half lines, 64 bytes of 16 rows, the loads alone take a quarter longer), of W a piece as
+// it lies in memory. A row's eight 16-byte chunks are stored at places exchanged by (row / 2), so that the 64 lanes
+// of an operand read (row = lane % 16, chunk = 4 step + lane / 16) fall on all banks.
+// A wave holds the operands of two k steps of 32 in registers: while it multiplies one step's (32 products), the
+// next step's 12 reads from LDS are issued between the products, one after every second, and have arrived when the
+// products are done. The workgroup meets once a stage, when the next stage has landed and the slot of the stage
+// before is free for the stage after next. The reads and the products are volatile asm, which pins their order;
+// the compiler neither sees the reads (and so orders nothing against the loads in flight) nor moves the products.
+// Timed on MI355X against reads and a barrier before each stage's products, with half lines of A:
+// 8192 x 37888 x 3584 2200 -> 1800 us (1.24 PFLOP/s), 2048 x 37888 x 3584 580 -> 480 us.
+// Taken apart at 8192 x 37888 x 3584: products and barriers alone 1230 us, the loads alone (one stage in flight)
+// 1550, everything 1790.
+// Workgroups are numbered so that the 32 that run together on one of the 8 XCDs (each with a second-level cache of
+// its own) own 4 x 8 neighbouring tiles of C, and so share their rows of A and of W there.
+#include <utility>
+
 #include "common.h"
 #include "microllm_hip.h"
 
@@ -20,22 +29,72 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) bf16 lds_bf16;
 
 constexpr int kTileM = 256, kTileN = 256;
 constexpr int kTiledWaves = 8;
 constexpr int kTiledThreads = kTiledWaves * kWave;
-constexpr int kPieceElements = 512;                       // 16 rows x 32 k
-constexpr int kPiecesPerSide = kTileM / 16;               // 16 pieces of A and 16 of W per k step
-constexpr int kStageSteps = 2;                            // k steps of 32 in a stage
-constexpr int kSideElements = kStageSteps * kPiecesPerSide * kPieceElements;   // 32 KB of A or of W in a stage
+constexpr int kPieceElements = 512;                       // of W: 16 rows x 32 k in MFMA operand order, 1 KB
 constexpr int kWaveTilesM = 8, kWaveTilesN = 4;           // a wave's 128 x 64 of C
+constexpr int kSlotBytes = 65536;                         // a stage of 64 of k: 32 KB of A, then 32 KB of W
+constexpr int kSlotElements = kSlotBytes / 2;
+constexpr int kWBytes = 32768;                            // where W begins in a slot
+constexpr int kSuperM = 4, kSuperN = 8;                   // tiles of C that run together on an XCD
 
-union TFrag {
-    bf16x8 v;
-    uint4 raw;
-};
+__device__ __align__(16) const unsigned zero_piece[256] = {};      // a piece of W past the end of k
 
 __device__ inline float silu_fast(float value) { return value / (1.0f + __expf(-value)); }
+
+__device__ inline unsigned lds_address(bf16* place) { return static_cast<unsigned>(reinterpret_cast<uintptr_t>((lds_bf16*)place)); }
+
+struct TiledOperands {       // of one k step: the wave's 8 pieces of A and 4 of W, 16 bytes a lane each
+    uintx4 a[kWaveTilesM];
+    uintx4 w[kWaveTilesN];
+};
+
+#define MLL_DS_READ(TARGET, ADDRESS, BYTES) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(TARGET) : "v"(ADDRESS), "n"(BYTES))
+#define MLL_MFMA(ACC, W, A) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(ACC) : "v"(W), "v"(A))
+
+// The INDEX-th of the 12 reads of k step STEP (0, 1) of a stage: pieces of A are 2 KB apart in a slot, tiles of W
+// too, with the tile's second step 1 KB after its first.
+template <int INDEX, int STEP>
+__device__ __attribute__((always_inline)) inline void read_operand(TiledOperands& f, unsigned a_address, unsigned w_address) {
+    constexpr int W = kWBytes + STEP * 1024;
+    if constexpr (INDEX == 0) MLL_DS_READ(f.w[0], w_address, W);
+    if constexpr (INDEX == 1) MLL_DS_READ(f.w[1], w_address, W + 2048);
+    if constexpr (INDEX == 2) MLL_DS_READ(f.a[0], a_address, 0);
+    if constexpr (INDEX == 3) MLL_DS_READ(f.a[1], a_address, 2048);
+    if constexpr (INDEX == 4) MLL_DS_READ(f.w[2], w_address, W + 4096);
+    if constexpr (INDEX == 5) MLL_DS_READ(f.w[3], w_address, W + 6144);
+    if constexpr (INDEX == 6) MLL_DS_READ(f.a[2], a_address, 4096);
+    if constexpr (INDEX == 7) MLL_DS_READ(f.a[3], a_address, 6144);
+    if constexpr (INDEX == 8) MLL_DS_READ(f.a[4], a_address, 8192);
+    if constexpr (INDEX == 9) MLL_DS_READ(f.a[5], a_address, 10240);
+    if constexpr (INDEX == 10) MLL_DS_READ(f.a[6], a_address, 12288);
+    if constexpr (INDEX == 11) MLL_DS_READ(f.a[7], a_address, 14336);
+}
+template <int STEP, int... INDEX>
+__device__ __attribute__((always_inline)) inline void read_operands(TiledOperands& f, unsigned a_address, unsigned w_address,
+                                                                    std::integer_sequence<int, INDEX...>) {
+    (read_operand<INDEX, STEP>(f, a_address, w_address), ...);
+}
+
+// The reads into `f` have arrived (and, LOADS, the wave's loads into LDS have landed). `f` passes through the
+// statement, so that nothing that uses it is placed before.
+template <bool LOADS>
+__device__ __attribute__((always_inline)) inline void operands_arrived(TiledOperands& f) {
+    if constexpr (LOADS)
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)"
+                     : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.a[4]), "+v"(f.a[5]), "+v"(f.a[6]),
+                       "+v"(f.a[7]), "+v"(f.w[0]), "+v"(f.w[1]), "+v"(f.w[2]), "+v"(f.w[3])
+                     :: "memory");
+    else
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.a[4]), "+v"(f.a[5]), "+v"(f.a[6]),
+                       "+v"(f.a[7]), "+v"(f.w[0]), "+v"(f.w[1]), "+v"(f.w[2]), "+v"(f.w[3])
+                     :: "memory");
+}
 
 // EPILOGUE: 0 = float32 [M, N]; 1 = bfloat16 [M, N]; 2 = bfloat16 [M, N / 2] = silu(even rows of W) * (odd rows).
 // With epilogue 0 the stages of k may be dealt to gridDim.y workgroups, each writing its own [M, N] of partial sums.
@@ -43,17 +102,20 @@ template <int EPILOGUE>
 __global__ __launch_bounds__(kTiledThreads, 1) void gemm_tiled_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w_packed,
                                                                       void* __restrict__ out, int m, int n, int k, int n_tiles,
                                                                       int k_steps, int m_blocks, int n_blocks) {
-    __shared__ __align__(16) bf16 a_even[kSideElements];      // [k step in the stage][piece][512]
-    __shared__ __align__(16) bf16 w_even[kSideElements];
-    __shared__ __align__(16) bf16 a_odd[kSideElements];
-    __shared__ __align__(16) bf16 w_odd[kSideElements];
+    // Two slots. In a slot: A as [16 pieces of 16 rows][row][8 places of 16 bytes], the row's chunk c of 8 elements at
+    // place c ^ (row / 2); then W as [16 tiles][2 k steps][1 KB in MFMA operand order]. Only the direct loads write
+    // this memory and only the asm reads read it.
+    __shared__ __align__(16) bf16 slots[2 * kSlotElements];
 
-    // Workgroups 8 apart in number run on one XCD: give them the tiles of C that share a tile of W.
+    // Workgroups 8 apart in number run on one XCD, 32 of them at a time: they take 4 x 8 tiles of C together.
     const int xcd = blockIdx.x % 8;
     const int local = blockIdx.x / 8;
-    const int n_block = (local / m_blocks) * 8 + xcd;
-    const int m_block = local % m_blocks;
-    if (n_block >= n_blocks) return;
+    constexpr int kSuper = kSuperM * kSuperN;
+    const int super_rows = (m_blocks + kSuperM - 1) / kSuperM;
+    const int super = (local / kSuper) * 8 + xcd, within = local % kSuper;
+    const int m_block = (super % super_rows) * kSuperM + within % kSuperM;
+    const int n_block = (super / super_rows) * kSuperN + within / kSuperM;
+    if (n_block >= n_blocks || m_block >= m_blocks) return;
 
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -61,35 +123,57 @@ __global__ __launch_bounds__(kTiledThreads, 1) void gemm_tiled_kernel(const bf16
     const int wave_m = wave / 4, wave_n = wave % 4;        // which 128 x 64 of the tile
     const int m0 = m_block * kTileM, n_tile0 = n_block * (kTileN / 16);
 
-    // What this wave copies per k step: pieces 2 * wave and 2 * wave + 1 of A and of W.
+    // What this wave copies per stage: pieces 2 * wave and 2 * wave + 1 of A, each as two instructions of 8 rows
+    // (lane L: row L / 8 of the 8, place L % 8 of the row), and tiles 2 * wave and 2 * wave + 1 of W, a k step an
+    // instruction.
     const bf16* a_block = a + static_cast<int64_t>(m0) * k;
-    int a_offset[2];          // of the lane's 16 bytes in the piece's rows, from a_block, at k = 0
-    const bf16* w_piece[2];   // the piece at k step 0 (the same for all lanes)
+    int a_offset[2][2];       // of the lane's 16 bytes from a_block, at stage 0
+    const bf16* w_tile[2];    // the lane's 16 bytes of the tile's piece at k step 0
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
         const int piece = wave * 2 + p;
-        const int row = min(piece * 16 + col, m - 1 - m0);            // rows past the end repeat the last one
-        a_offset[p] = row * k + quad * 8;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int row_in_piece = 8 * h + lane / 8;
+            const int row = min(piece * 16 + row_in_piece, m - 1 - m0);            // rows past the end repeat the last one
+            a_offset[p][h] = row * k + (((lane % 8) ^ (row_in_piece / 2)) * 8);
+        }
         const int tile = min(n_tile0 + piece, n_tiles - 1);
-        w_piece[p] = w_packed + static_cast<int64_t>(tile) * k_steps * kPieceElements;
+        w_tile[p] = w_packed + static_cast<int64_t>(tile) * k_steps * kPieceElements + lane * 8;
     }
-    auto copy_stage = [&](int stage, bf16* a_stage, bf16* w_stage) {
+    const int all_stages = (k_steps + 1) / 2;
+    const int stages_per_split = (all_stages + gridDim.y - 1) / gridDim.y;
+    const int first_stage = blockIdx.y * stages_per_split;
+    const int stages = min(all_stages, first_stage + stages_per_split);
+    const int last = stages - 1;
+    // A k step past the end (k an odd multiple of 32; the stage after the last, which the loop's second half may
+    // take) gets zeros for W and, for A, values that lie in the row: the chunks of the stage's second half step
+    // back by 64 bytes there, the stage after the last is the last again.
+    auto copy_stage = [&](int stage, int slot) __attribute__((always_inline)) {
+        bf16* a_place = slots + slot * kSlotElements;
+        bf16* w_place = a_place + kWBytes / 2;
+        const int a_stage = min(stage, last);
+        const bool half_stage = 2 * a_stage + 1 >= k_steps;
 #pragma unroll
-        for (int step = 0; step < kStageSteps; ++step) {
-            const int ks = stage * kStageSteps + step;
-            if (ks >= k_steps) break;
+        for (int p = 0; p < 2; ++p) {
+            const int piece = wave * 2 + p;
 #pragma unroll
-            for (int p = 0; p < 2; ++p) {
-                const int piece = wave * 2 + p;
-                const bf16* a_source = a_block + ks * 32 + a_offset[p];
-                const bf16* w_source = w_piece[p] + static_cast<int64_t>(ks) * kPieceElements + lane * 8;
-                bf16* a_place = a_stage + (step * kPiecesPerSide + piece) * kPieceElements;
-                bf16* w_place = w_stage + (step * kPiecesPerSide + piece) * kPieceElements;
-                __builtin_amdgcn_global_load_lds(a_source, a_place, 16, 0, 0);
-                __builtin_amdgcn_global_load_lds(w_source, w_place, 16, 0, 0);
+            for (int h = 0; h < 2; ++h) {
+                const bool upper = (((lane >> 2) & 1) ^ h) != 0;      // the lane's chunk is one of the row's second four
+                const bf16* a_source = a_block + a_stage * 64 + a_offset[p][h] - ((half_stage && upper) ? 32 : 0);
+                __builtin_amdgcn_global_load_lds(a_source, a_place + piece * 1024 + h * 512, 16, 0, 0);
+                const bool real = stage <= last && 2 * stage + h < k_steps;
+                const bf16* w_source = real ? w_tile[p] + static_cast<int64_t>(2 * stage + h) * kPieceElements
+                                            : reinterpret_cast<const bf16*>(zero_piece) + lane * 8;
+                __builtin_amdgcn_global_load_lds(w_source, w_place + piece * 1024 + h * 512, 16, 0, 0);
             }
         }
     };
+    // Where the lane reads its operands: row `col` of a piece, chunk 4 step + quad at its place.
+    const unsigned base = lds_address(slots);
+    const unsigned a_row = base + wave_m * kWaveTilesM * 2048 + col * 128;
+    const unsigned a_step0 = a_row + ((quad ^ (col / 2)) * 16), a_step1 = a_row + (((4 + quad) ^ (col / 2)) * 16);
+    const unsigned w_lane = base + wave_n * kWaveTilesN * 2048 + lane * 16;
 
     floatx4 acc[kWaveTilesN][kWaveTilesM];     // acc[nt][mt][i] = C[m = mt*16 + col][n = nt*16 + quad*4 + i] of the wave's part
 #pragma unroll
@@ -97,45 +181,58 @@ __global__ __launch_bounds__(kTiledThreads, 1) void gemm_tiled_kernel(const bf16
 #pragma unroll
         for (int mt = 0; mt < kWaveTilesM; ++mt) acc[nt][mt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    auto multiply_stage = [&](int stage, const bf16* a_stage, const bf16* w_stage) {
-#pragma unroll
-        for (int step = 0; step < kStageSteps; ++step) {
-            if (stage * kStageSteps + step >= k_steps) break;
-            TFrag a_frag[kWaveTilesM], w_frag[kWaveTilesN];
-#pragma unroll
-            for (int t = 0; t < kWaveTilesM; ++t)
-                a_frag[t].raw = *reinterpret_cast<const uint4*>(
-                    a_stage + (step * kPiecesPerSide + wave_m * kWaveTilesM + t) * kPieceElements + lane * 8);
-#pragma unroll
-            for (int t = 0; t < kWaveTilesN; ++t)
-                w_frag[t].raw = *reinterpret_cast<const uint4*>(
-                    w_stage + (step * kPiecesPerSide + wave_n * kWaveTilesN + t) * kPieceElements + lane * 8);
-#pragma unroll
-            for (int nt = 0; nt < kWaveTilesN; ++nt)
-#pragma unroll
-                for (int mt = 0; mt < kWaveTilesM; ++mt)
-                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_frag[nt].v, a_frag[mt].v, acc[nt][mt], 0, 0, 0);
+    if (first_stage < stages) {
+        int stage = first_stage;
+        copy_stage(stage, 0);
+        copy_stage(stage + 1, 1);
+        TiledOperands even, odd;      // of a stage's first and second k step
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");      // the first stage's 8 loads of this wave
+        __builtin_amdgcn_s_barrier();
+        read_operands<0>(even, a_step0, w_lane, std::make_integer_sequence<int, 12>{});
+        // The 32 products of a k step, and after every second of the first 24 a read of the next step's operands.
+#define MLL_TILED_PRODUCTS(NOW, NEXT, NEXT_STEP, A_ADDRESS, W_ADDRESS)                                     \
+    {                                                                                                      \
+        const unsigned a_address = A_ADDRESS, w_address = W_ADDRESS;                                       \
+        MLL_MFMA(acc[0][0], NOW.w[0], NOW.a[0]); MLL_MFMA(acc[1][0], NOW.w[1], NOW.a[0]); read_operand<0, NEXT_STEP>(NEXT, a_address, w_address);   \
+        MLL_MFMA(acc[2][0], NOW.w[2], NOW.a[0]); MLL_MFMA(acc[3][0], NOW.w[3], NOW.a[0]); read_operand<1, NEXT_STEP>(NEXT, a_address, w_address);   \
+        MLL_MFMA(acc[0][1], NOW.w[0], NOW.a[1]); MLL_MFMA(acc[1][1], NOW.w[1], NOW.a[1]); read_operand<2, NEXT_STEP>(NEXT, a_address, w_address);   \
+        MLL_MFMA(acc[2][1], NOW.w[2], NOW.a[1]); MLL_MFMA(acc[3][1], NOW.w[3], NOW.a[1]); read_operand<3, NEXT_STEP>(NEXT, a_address, w_address);   \
+        MLL_MFMA(acc[0][2], NOW.w[0], NOW.a[2]); MLL_MFMA(acc[1][2], NOW.w[1], NOW.a[2]); read_operand<4, NEXT_STEP>(NEXT, a_address, w_address);   \
+        MLL_MFMA(acc[2][2], NOW.w[2], NOW.a[2]); MLL_MFMA(acc[3][2], NOW.w[3], NOW.a[2]); read_operand<5, NEXT_STEP>(NEXT, a_address, w_address);   \
+        MLL_MFMA(acc[0][3], NOW.w[0], NOW.a[3]); MLL_MFMA(acc[1][3], NOW.w[1], NOW.a[3]); read_operand<6, NEXT_STEP>(NEXT, a_address, w_address);   \
+        MLL_MFMA(acc[2][3], NOW.w[2], NOW.a[3]); MLL_MFMA(acc[3][3], NOW.w[3], NOW.a[3]); read_operand<7, NEXT_STEP>(NEXT, a_address, w_address);   \
+        MLL_MFMA(acc[0][4], NOW.w[0], NOW.a[4]); MLL_MFMA(acc[1][4], NOW.w[1], NOW.a[4]); read_operand<8, NEXT_STEP>(NEXT, a_address, w_address);   \
+        MLL_MFMA(acc[2][4], NOW.w[2], NOW.a[4]); MLL_MFMA(acc[3][4], NOW.w[3], NOW.a[4]); read_operand<9, NEXT_STEP>(NEXT, a_address, w_address);   \
+        MLL_MFMA(acc[0][5], NOW.w[0], NOW.a[5]); MLL_MFMA(acc[1][5], NOW.w[1], NOW.a[5]); read_operand<10, NEXT_STEP>(NEXT, a_address, w_address);  \
+        MLL_MFMA(acc[2][5], NOW.w[2], NOW.a[5]); MLL_MFMA(acc[3][5], NOW.w[3], NOW.a[5]); read_operand<11, NEXT_STEP>(NEXT, a_address, w_address);  \
+        MLL_MFMA(acc[0][6], NOW.w[0], NOW.a[6]); MLL_MFMA(acc[1][6], NOW.w[1], NOW.a[6]);                  \
+        MLL_MFMA(acc[2][6], NOW.w[2], NOW.a[6]); MLL_MFMA(acc[3][6], NOW.w[3], NOW.a[6]);                  \
+        MLL_MFMA(acc[0][7], NOW.w[0], NOW.a[7]); MLL_MFMA(acc[1][7], NOW.w[1], NOW.a[7]);                  \
+        MLL_MFMA(acc[2][7], NOW.w[2], NOW.a[7]); MLL_MFMA(acc[3][7], NOW.w[3], NOW.a[7]);                  \
+    }
+        // A stage that lies in slot SLOT. Its first step is multiplied while its second is read. Then the wave's
+        // loads of the next stage have landed; after the barrier everyone's have, and everyone has read this stage,
+        // whose slot the stage after next may take. The second step is multiplied while the next stage's first is read.
+#define MLL_TILED_STAGE(SLOT)                                                                              \
+    {                                                                                                      \
+        operands_arrived<false>(even);                                                                     \
+        MLL_TILED_PRODUCTS(even, odd, 1, a_step1 + SLOT * kSlotBytes, w_lane + SLOT * kSlotBytes)          \
+        operands_arrived<true>(odd);                                                                       \
+        __builtin_amdgcn_s_barrier();                                                                      \
+        copy_stage(stage + 2, SLOT);                                                                       \
+        MLL_TILED_PRODUCTS(odd, even, 0, a_step0 + (1 - SLOT) * kSlotBytes, w_lane + (1 - SLOT) * kSlotBytes) \
+        ++stage;                                                                                           \
+    }
+        // Two stages a round; a stage past the end multiplies by zeros.
+        while (stage < stages) {
+            MLL_TILED_STAGE(0)
+            MLL_TILED_STAGE(1)
         }
-    };
-    auto landed = [&]() {
-        wait_for_loads();    // this wave's pieces of the stage are in LDS
-        __syncthreads();     // everyone's are, and everyone is done with the stage before
-    };
-
-    const int all_stages = (k_steps + kStageSteps - 1) / kStageSteps;
-    const int stages_per_split = (all_stages + gridDim.y - 1) / gridDim.y;
-    const int first_stage = blockIdx.y * stages_per_split;
-    const int stages = min(all_stages, first_stage + stages_per_split);
-    if (first_stage < stages) copy_stage(first_stage, a_even, w_even);
-    for (int stage = first_stage; stage < stages; stage += 2) {
-        landed();
-        if (stage + 1 < stages) copy_stage(stage + 1, a_odd, w_odd);
-        multiply_stage(stage, a_even, w_even);
-        if (stage + 1 < stages) {
-            landed();
-            if (stage + 2 < stages) copy_stage(stage + 2, a_even, w_even);
-            multiply_stage(stage + 1, a_odd, w_odd);
-        }
+#undef MLL_TILED_STAGE
+#undef MLL_TILED_PRODUCTS
+        // No load may be on its way into LDS when the workgroup ends, and the last products must have written
+        // their results before these are read (the compiler does not know that the asm statements are products).
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
     }
 
 #pragma unroll
@@ -187,7 +284,8 @@ template <int EPILOGUE>
 static int launch_tiled(const void* a, const void* w_packed, void* out, int m, int n, int k, int splits, hipStream_t stream) {
     const int n_tiles = (n + 15) / 16, k_steps = k / 32;
     const int m_blocks = (m + kTileM - 1) / kTileM, n_blocks = (n + kTileN - 1) / kTileN;
-    const dim3 grid(8 * ((n_blocks + 7) / 8) * m_blocks, splits);
+    const int supers = ((m_blocks + kSuperM - 1) / kSuperM) * ((n_blocks + kSuperN - 1) / kSuperN);
+    const dim3 grid(((supers + 7) / 8) * 8 * kSuperM * kSuperN, splits);      // workgroups outside C leave at once
     gemm_tiled_kernel<EPILOGUE><<<grid, kTiledThreads, 0, stream>>>(static_cast<const bf16*>(a), static_cast<const bf16*>(w_packed),
                                                             out, m, n, k, n_tiles, k_steps, m_blocks, n_blocks);
     return check_launch("gemm_tiled");
