@@ -17,7 +17,8 @@
 // Taken apart at 8192 x 37888 x 3584: products and barriers alone 1230 us, the loads alone (one stage in flight)
 // 1550, everything 1790.
 // Workgroups are numbered so that the 32 that run together on one of the 8 XCDs (each with a second-level cache of
-// its own) own 4 x 8 neighbouring tiles of C, and so share their rows of A and of W there.
+// its own) own about 4 x 8 neighbouring tiles of C, and so share their rows of A and of W there, and so that every
+// XCD gets the same number of tiles.
 #include <utility>
 
 #include "common.h"
@@ -107,15 +108,22 @@ __global__ __launch_bounds__(kTiledThreads, 1) void gemm_tiled_kernel(const bf16
     // this memory and only the asm reads read it.
     __shared__ __align__(16) bf16 slots[2 * kSlotElements];
 
-    // Workgroups 8 apart in number run on one XCD, 32 of them at a time: they take 4 x 8 tiles of C together.
-    const int xcd = blockIdx.x % 8;
-    const int local = blockIdx.x / 8;
-    constexpr int kSuper = kSuperM * kSuperN;
-    const int super_rows = (m_blocks + kSuperM - 1) / kSuperM;
-    const int super = (local / kSuper) * 8 + xcd, within = local % kSuper;
-    const int m_block = (super % super_rows) * kSuperM + within % kSuperM;
-    const int n_block = (super / super_rows) * kSuperN + within / kSuperM;
-    if (n_block >= n_blocks || m_block >= m_blocks) return;
+    // Workgroups 8 apart in number run on one XCD, 32 of them at a time. The tiles of C are put in a row, blocks of
+    // 4 x 8 neighbouring tiles after one another (down the rows of C first, narrower at the edges), and every XCD
+    // takes an equal stretch of that row: the workgroups that run together there own neighbouring tiles, and no XCD
+    // has more than one tile more than another.
+    const int tiles = m_blocks * n_blocks;
+    const int per_xcd = (tiles + 7) / 8;
+    const int place = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (blockIdx.x / 8 >= per_xcd || place >= tiles) return;
+    const int column = place / (m_blocks * kSuperN);                       // of blocks, kSuperN tiles wide
+    const int width = min(kSuperN, n_blocks - column * kSuperN);
+    const int in_column = place - column * m_blocks * kSuperN;
+    const int block = in_column / (kSuperM * width);                       // in the column, kSuperM tiles high
+    const int height = min(kSuperM, m_blocks - block * kSuperM);
+    const int in_block = in_column - block * kSuperM * width;
+    const int m_block = block * kSuperM + in_block % height;
+    const int n_block = column * kSuperN + in_block / height;
 
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -284,8 +292,7 @@ template <int EPILOGUE>
 static int launch_tiled(const void* a, const void* w_packed, void* out, int m, int n, int k, int splits, hipStream_t stream) {
     const int n_tiles = (n + 15) / 16, k_steps = k / 32;
     const int m_blocks = (m + kTileM - 1) / kTileM, n_blocks = (n + kTileN - 1) / kTileN;
-    const int supers = ((m_blocks + kSuperM - 1) / kSuperM) * ((n_blocks + kSuperN - 1) / kSuperN);
-    const dim3 grid(((supers + 7) / 8) * 8 * kSuperM * kSuperN, splits);      // workgroups outside C leave at once
+    const dim3 grid(8 * ((m_blocks * n_blocks + 7) / 8), splits);
     gemm_tiled_kernel<EPILOGUE><<<grid, kTiledThreads, 0, stream>>>(static_cast<const bf16*>(a), static_cast<const bf16*>(w_packed),
                                                             out, m, n, k, n_tiles, k_steps, m_blocks, n_blocks);
     return check_launch("gemm_tiled");
