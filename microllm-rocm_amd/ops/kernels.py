@@ -838,8 +838,9 @@ def tiled_splits(m: int, n: int, k: int) -> int:
 
 
 def gemm_tiled(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f32", splits: int = 1) -> torch.Tensor:
-    """``x @ W.T`` for many bfloat16 rows and a packed weight, on this package's tiled MFMA kernel (0.85 to 0.95 of
-    the library's rate at 2048 rows and more: for weights that are kept in the packed order alone). ``k`` must be
+    """``x @ W.T`` for many bfloat16 rows and a packed weight, on this package's tiled MFMA kernel (0.9 to 1.1 of
+    the library's untuned rate at 2048 rows and more, 1.1 to 1.4 PFLOP/s: for weights that are kept in the packed
+    order alone). ``k`` must be
     a multiple of 32. With ``splits`` > 1 (float32 only) the result is ``[splits, m, n]`` sums over parts of the
     reduction for the caller to add in order."""
     lib = library.load()
