@@ -767,6 +767,7 @@ def gemm_skinny(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "
 
 
 MEDIUM_WORKGROUPS = 224     # workgroups of 8 waves that gemm_medium wants at least (MI355X has 256 compute units)
+MEDIUM_WHOLE_WORKGROUPS = 128     # where the reduction cannot be split, two tiles a wave from this many workgroups on
 
 
 def medium_plan(n: int, k: int, may_split: bool = True) -> Tuple[int, int, int]:
@@ -781,7 +782,7 @@ def medium_plan(n: int, k: int, may_split: bool = True) -> Tuple[int, int, int]:
     most = 1
     while may_split and most * 2 <= min(16, stages):
         most *= 2
-    tiles_per_wave = 2 if -(-n_tiles // 16) * most >= MEDIUM_WORKGROUPS else 1
+    tiles_per_wave = 2 if -(-n_tiles // 16) * most >= (MEDIUM_WORKGROUPS if may_split else MEDIUM_WHOLE_WORKGROUPS) else 1
     groups = -(-n_tiles // (8 * tiles_per_wave))
     splits = 1
     while splits < most and groups * splits < MEDIUM_WORKGROUPS:

@@ -7,7 +7,7 @@ import torch
 from microllm_rocm_amd.architectures.qwen2 import build_spec, init_rules
 from microllm_rocm_amd.ops import kernels
 from microllm_rocm_amd.parts import Model, Runtime
-from microllm_rocm_amd.parts.linear import MEDIUM_ROWS, SKINNY_ROWS, Weight, takes_packed, takes_unscaled
+from microllm_rocm_amd.parts.linear import MEDIUM_GATED_ROWS, MEDIUM_ROWS, SKINNY_ROWS, Weight, takes_packed, takes_unscaled
 from microllm_rocm_amd.weights.random_init import random_tensors
 from tiny import TINY_A, TINY_B
 
@@ -108,7 +108,8 @@ def test_which_product_a_linear_takes():
     packed = Weight(torch.zeros((64, 32), dtype=torch.bfloat16), pack=False)
     packed.packed = torch.zeros((4, 1, 4, 16, 8), dtype=torch.bfloat16)   # as on the GPU
     assert takes_packed(packed, SKINNY_ROWS) and takes_packed(packed, MEDIUM_ROWS) and not takes_packed(packed, MEDIUM_ROWS + 1)
-    assert not takes_packed(packed, SKINNY_ROWS + 1, gated=True), "the gated product of 17 to 64 rows is the library's"
+    assert takes_packed(packed, MEDIUM_GATED_ROWS, gated=True) and not takes_packed(packed, MEDIUM_GATED_ROWS + 1, gated=True), \
+        "the gated product goes to the library (and the SiLU kernel) beyond this many rows"
     assert takes_unscaled(packed, SKINNY_ROWS) and not takes_unscaled(packed, SKINNY_ROWS + 1)
     packed.tensor = None                                                   # one copy: the packed one serves every step
     assert takes_packed(packed, 5000) and takes_packed(packed, 40, gated=True)
