@@ -76,8 +76,10 @@ template <bool VECTOR>
 __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float* __restrict__ a, const float* __restrict__ w,
                                                              const float* __restrict__ bias, float* __restrict__ c,
                                                              int m, int n, int k) {
-    __shared__ float a_tile[16][kSmallDepth + 1];
-    __shared__ float w_tile[kSmallColumns][kSmallDepth + 1];
+    // Rows of kSmallDepth + 4 floats: 16-byte aligned, so that four consecutive k are one read, and four banks on
+    // from row to row, so that the 16 rows (or columns) that a wave reads at one k fall on different banks.
+    __shared__ __align__(16) float a_tile[16][kSmallDepth + 4];
+    __shared__ __align__(16) float w_tile[kSmallColumns][kSmallDepth + 4];
     const int col0 = blockIdx.x * kSmallColumns;
     const int column = threadIdx.x % kSmallColumns;     // this thread's output: row `row`, column col0 + `column`
     const int row = threadIdx.x / kSmallColumns;
@@ -114,15 +116,21 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float* __rest
 #pragma unroll
         for (int part = 0; part < 2; ++part) {
             const int at = 64 * part + load_k;
-            a_tile[load_row][at] = a_next[part].x, a_tile[load_row][at + 1] = a_next[part].y;
-            a_tile[load_row][at + 2] = a_next[part].z, a_tile[load_row][at + 3] = a_next[part].w;
-            w_tile[load_row][at] = w_next[part].x, w_tile[load_row][at + 1] = w_next[part].y;
-            w_tile[load_row][at + 2] = w_next[part].z, w_tile[load_row][at + 3] = w_next[part].w;
+            *reinterpret_cast<float4*>(&a_tile[load_row][at]) = a_next[part];
+            *reinterpret_cast<float4*>(&w_tile[load_row][at]) = w_next[part];
         }
         __syncthreads();
         if (k0 + kSmallDepth < k) fetch(k0 + kSmallDepth);      // the next chunk is on its way while this one is summed
+        // Four k a read, summed one after the other in ascending k as before: the same bits.
 #pragma unroll
-        for (int kk = 0; kk < kSmallDepth; ++kk) acc = fmaf(a_tile[row][kk], w_tile[column][kk], acc);
+        for (int kk = 0; kk < kSmallDepth; kk += 4) {
+            const float4 av = *reinterpret_cast<const float4*>(&a_tile[row][kk]);
+            const float4 wv = *reinterpret_cast<const float4*>(&w_tile[column][kk]);
+            acc = fmaf(av.x, wv.x, acc);
+            acc = fmaf(av.y, wv.y, acc);
+            acc = fmaf(av.z, wv.z, acc);
+            acc = fmaf(av.w, wv.w, acc);
+        }
         __syncthreads();
     }
     const int col = col0 + column;
