@@ -68,7 +68,8 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
 // Each thread sums in ascending k with the same fused multiply-adds as the tiled kernel: the two give the same
 // bits, so a token's result does not depend on how many rows the step had.
 constexpr int kSmallColumns = 16;
-constexpr int kSmallDepth = 128;
+constexpr int kSmallDepth = 256;      // of k in a chunk (128: 3 to 7 % slower)
+constexpr int kSmallParts = kSmallDepth / 64;
 
 // VECTOR: k is a multiple of 4 and both matrices are 16-byte aligned, so a thread's four consecutive elements are
 // one load.
@@ -84,16 +85,16 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float* __rest
     const int column = threadIdx.x % kSmallColumns;     // this thread's output: row `row`, column col0 + `column`
     const int row = threadIdx.x / kSmallColumns;
     // What a thread brings in of a chunk of kSmallDepth of k: of row load_row of A and of W, elements
-    // load_k .. load_k + 3 and 64 + load_k .. 64 + load_k + 3.
+    // load_k .. load_k + 3 of every 64.
     const int load_row = threadIdx.x / 16;
     const int load_k = (threadIdx.x % 16) * 4;
     const bool a_live = load_row < m, w_live = col0 + load_row < n;
     const float* a_row = a + static_cast<int64_t>(a_live ? load_row : 0) * k;
     const float* w_row = w + static_cast<int64_t>(w_live ? col0 + load_row : 0) * k;
-    float4 a_next[2], w_next[2];
+    float4 a_next[kSmallParts], w_next[kSmallParts];
     auto fetch = [&](int k0) {
 #pragma unroll
-        for (int part = 0; part < 2; ++part) {
+        for (int part = 0; part < kSmallParts; ++part) {
             const int kk = k0 + 64 * part + load_k;
             if (VECTOR) {
                 a_next[part] = (a_live && kk < k) ? *reinterpret_cast<const float4*>(a_row + kk) : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -114,7 +115,7 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float* __rest
     fetch(0);
     for (int k0 = 0; k0 < k; k0 += kSmallDepth) {
 #pragma unroll
-        for (int part = 0; part < 2; ++part) {
+        for (int part = 0; part < kSmallParts; ++part) {
             const int at = 64 * part + load_k;
             *reinterpret_cast<float4*>(&a_tile[load_row][at]) = a_next[part];
             *reinterpret_cast<float4*>(&w_tile[load_row][at]) = w_next[part];
@@ -137,6 +138,92 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float* __rest
     if (row < m && col < n) c[static_cast<int64_t>(row) * n + col] = acc + (bias ? bias[col] : 0.0f);
 }
 
+// The same for weights with many rows (gate/up, the head), where the kernel above is bound by its reads from LDS (two a
+// multiply-add): a workgroup of 128 threads takes 32 columns of C and a thread 2 rows x 2 columns (rows r and r + 8,
+// columns c and c + 16): half the reads a multiply-add, and four chains of additions a thread. Every element is still
+// summed by one thread in ascending k: the same bits. Measured on MI355X at 7B sizes, 8 rows: gate/up 179 -> 140 us
+// (3.9 TB/s), the head 602 -> 450 (4.8 TB/s); with few columns it has too few waves (q/k/v 37 -> 65 us, down 136 -> 330).
+// Where W has few rows the kernel above stays at 1.8 to 2.0 TB/s: a wave an element's worth of lanes is all the
+// parallelism there is, and its reads from LDS (512 KB for 16 KB of W) are what a compute unit can give; neither four
+// sums an element instead of one, nor two chunks in flight instead of one, nor reading LDS a batch ahead changes that.
+constexpr int kWideColumns = 32;
+constexpr int kWideThreads = 128;
+constexpr int kWideDepth = 128;                      // of k in a chunk
+constexpr int kWideQuads = kWideDepth / 4;           // float4 in a row of a chunk
+constexpr int kWideLoadsA = 16 * kWideQuads / kWideThreads;
+constexpr int kWideLoadsW = kWideColumns * kWideQuads / kWideThreads;
+constexpr int kWideFrom = 16384;                     // columns of C from which this kernel is taken: 512 workgroups
+
+template <bool VECTOR>
+__global__ __launch_bounds__(kWideThreads) void gemm_f32_small_wide_kernel(const float* __restrict__ a, const float* __restrict__ w,
+                                                                           const float* __restrict__ bias, float* __restrict__ c,
+                                                                           int m, int n, int k) {
+    __shared__ __align__(16) float a_tile[16][kWideDepth + 4];
+    __shared__ __align__(16) float w_tile[kWideColumns][kWideDepth + 4];
+    const int col0 = blockIdx.x * kWideColumns;
+    const int column = threadIdx.x % 16;      // this thread's outputs: rows `row`, row + 8; columns col0 + `column`, + 16
+    const int row = threadIdx.x / 16;
+    // What a thread brings in of a chunk: float4 number threadIdx.x + j * 128 of the chunk's rows of A (16 rows of
+    // kWideQuads) and of W (32 rows).
+    auto load4 = [&](const float* matrix, int rows, int first_row, int index, int k0) {
+        const int r = index / kWideQuads, kk = k0 + (index % kWideQuads) * 4;
+        const bool live = first_row + r < rows;
+        const float* source = matrix + static_cast<int64_t>(live ? first_row + r : 0) * k + kk;
+        if (VECTOR) return (live && kk < k) ? *reinterpret_cast<const float4*>(source) : make_float4(0.f, 0.f, 0.f, 0.f);
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (live && kk + e < k) ? source[e] : 0.0f;
+        return make_float4(v[0], v[1], v[2], v[3]);
+    };
+    float4 a_next[kWideLoadsA], w_next[kWideLoadsW];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int j = 0; j < kWideLoadsA; ++j) a_next[j] = load4(a, m, 0, threadIdx.x + j * kWideThreads, k0);
+#pragma unroll
+        for (int j = 0; j < kWideLoadsW; ++j) w_next[j] = load4(w, n, col0, threadIdx.x + j * kWideThreads, k0);
+    };
+    float acc[2][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}};
+    fetch(0);
+    for (int k0 = 0; k0 < k; k0 += kWideDepth) {
+#pragma unroll
+        for (int j = 0; j < kWideLoadsA; ++j) {
+            const int index = threadIdx.x + j * kWideThreads;
+            *reinterpret_cast<float4*>(&a_tile[index / kWideQuads][(index % kWideQuads) * 4]) = a_next[j];
+        }
+#pragma unroll
+        for (int j = 0; j < kWideLoadsW; ++j) {
+            const int index = threadIdx.x + j * kWideThreads;
+            *reinterpret_cast<float4*>(&w_tile[index / kWideQuads][(index % kWideQuads) * 4]) = w_next[j];
+        }
+        __syncthreads();
+        if (k0 + kWideDepth < k) fetch(k0 + kWideDepth);      // the next chunk is on its way while this one is summed
+        // Four k a read, added one after the other in ascending k.
+#pragma unroll
+        for (int kk = 0; kk < kWideDepth; kk += 4) {
+            const float4 a0 = *reinterpret_cast<const float4*>(&a_tile[row][kk]);
+            const float4 a1 = *reinterpret_cast<const float4*>(&a_tile[row + 8][kk]);
+            const float4 w0 = *reinterpret_cast<const float4*>(&w_tile[column][kk]);
+            const float4 w1 = *reinterpret_cast<const float4*>(&w_tile[column + 16][kk]);
+            acc[0][0] = fmaf(a0.x, w0.x, acc[0][0]); acc[0][1] = fmaf(a0.x, w1.x, acc[0][1]);
+            acc[1][0] = fmaf(a1.x, w0.x, acc[1][0]); acc[1][1] = fmaf(a1.x, w1.x, acc[1][1]);
+            acc[0][0] = fmaf(a0.y, w0.y, acc[0][0]); acc[0][1] = fmaf(a0.y, w1.y, acc[0][1]);
+            acc[1][0] = fmaf(a1.y, w0.y, acc[1][0]); acc[1][1] = fmaf(a1.y, w1.y, acc[1][1]);
+            acc[0][0] = fmaf(a0.z, w0.z, acc[0][0]); acc[0][1] = fmaf(a0.z, w1.z, acc[0][1]);
+            acc[1][0] = fmaf(a1.z, w0.z, acc[1][0]); acc[1][1] = fmaf(a1.z, w1.z, acc[1][1]);
+            acc[0][0] = fmaf(a0.w, w0.w, acc[0][0]); acc[0][1] = fmaf(a0.w, w1.w, acc[0][1]);
+            acc[1][0] = fmaf(a1.w, w0.w, acc[1][0]); acc[1][1] = fmaf(a1.w, w1.w, acc[1][1]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int r = row + 8 * i, col = col0 + column + 16 * j;
+            if (r < m && col < n) c[static_cast<int64_t>(r) * n + col] = acc[i][j] + (bias ? bias[col] : 0.0f);
+        }
+}
+
 }  // namespace mll
 
 using namespace mll;
@@ -147,6 +234,12 @@ extern "C" int mll_gemm_f32(const float* a, const float* w, const float* bias, f
     if (m == 0) return 0;
     if (m <= 16) {
         const bool vector = k % 4 == 0 && reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
+        if (n >= kWideFrom) {
+            const int groups = (n + kWideColumns - 1) / kWideColumns;
+            if (vector) gemm_f32_small_wide_kernel<true><<<groups, kWideThreads, 0, stream>>>(a, w, bias, c, m, n, k);
+            else gemm_f32_small_wide_kernel<false><<<groups, kWideThreads, 0, stream>>>(a, w, bias, c, m, n, k);
+            return check_launch("gemm_f32");
+        }
         const int groups = (n + kSmallColumns - 1) / kSmallColumns;
         if (vector) gemm_f32_small_kernel<true><<<groups, 256, 0, stream>>>(a, w, bias, c, m, n, k);
         else gemm_f32_small_kernel<false><<<groups, 256, 0, stream>>>(a, w, bias, c, m, n, k);
