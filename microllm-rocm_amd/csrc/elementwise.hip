@@ -96,14 +96,24 @@ __global__ void rms_norm_vec4_kernel(float* __restrict__ h, const D* __restrict_
         if (q < quads) {
             value[c] = reinterpret_cast<const float4*>(h_row)[q];
             if (delta_row) {
-                // The parts of the delta are added first, in order, and their sum to the stream.
+                // The parts of the delta are added first, in order, and their sum to the stream. Up to sixteen parts
+                // are asked for at a time and then added: a part an iteration waits for memory once a part (64 rows
+                // of 3584 in 16 parts: 11.4 us that way, 8.5 with eight at a time).
+                constexpr int kAtATime = CHUNKS == 1 ? 16 : 8;
                 float4 sum = load_four(delta_row + 4 * q);
-                for (int part = 1; part < n_partials; ++part) {
-                    const float4 more = load_four(delta_row + part * partial_stride + 4 * q);
-                    sum.x += more.x;
-                    sum.y += more.y;
-                    sum.z += more.z;
-                    sum.w += more.w;
+                for (int base = 1; base < n_partials; base += kAtATime) {
+                    float4 more[kAtATime];
+#pragma unroll
+                    for (int j = 0; j < kAtATime; ++j)
+                        if (base + j < n_partials) more[j] = load_four(delta_row + (base + j) * partial_stride + 4 * q);
+#pragma unroll
+                    for (int j = 0; j < kAtATime; ++j)
+                        if (base + j < n_partials) {
+                            sum.x += more[j].x;
+                            sum.y += more[j].y;
+                            sum.z += more[j].z;
+                            sum.w += more[j].w;
+                        }
                 }
                 value[c].x += sum.x;
                 value[c].y += sum.y;
@@ -228,9 +238,20 @@ __global__ void qkv_rope_store_kernel(const In* __restrict__ qkv, int n_partials
         const int in_first = paired ? 2 * pair : first, in_second = paired ? 2 * pair + 1 : second;
         float x1 = to_float(qkv[in_row + column + in_first]);
         float x2 = to_float(qkv[in_row + column + in_second]);
-        for (int part = 1; part < n_partials; ++part) {
-            x1 += to_float(qkv[part * partial_stride + in_row + column + in_first]);
-            x2 += to_float(qkv[part * partial_stride + in_row + column + in_second]);
+        for (int base = 1; base < n_partials; base += 8) {      // eight parts asked for at a time, then added in order
+            float more1[8], more2[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (base + j < n_partials) {
+                    more1[j] = to_float(qkv[(base + j) * partial_stride + in_row + column + in_first]);
+                    more2[j] = to_float(qkv[(base + j) * partial_stride + in_row + column + in_second]);
+                }
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (base + j < n_partials) {
+                    x1 += more1[j];
+                    x2 += more2[j];
+                }
         }
         if (bias) {
             x1 += bias[column + first];
