@@ -141,6 +141,24 @@ def test_window_rules():
     assert np.abs(windowed[9, 0] - full[9, 0]).max() > 1e-3
 
 
+def test_attention_in_blocks_is_the_row_by_row_formula():
+    """Long sequences take ``causal_gqa_attention_in_blocks``; it must be the row-by-row function, also where a
+    block's first query and the window's edge fall inside a block of keys, and with sharp scores."""
+    rng = np.random.default_rng(4)
+    tokens, heads, kv_heads, hd = 150, 6, 2, 8
+    q, k, v = rng.normal(size=(tokens, heads, hd)) * 3, rng.normal(size=(tokens, kv_heads, hd)), rng.normal(size=(tokens, kv_heads, hd))
+    assert tokens <= plain.ROW_BY_ROW_LIMIT
+    for window in (None, 1, 7, 64, 149, 150, 1000):
+        for block in (1, 32, 37, 256):
+            rows = plain.causal_gqa_attention(q, k, v, 0.4, window)
+            blocks = plain.causal_gqa_attention_in_blocks(q, k, v, 0.4, window, block=block)
+            np.testing.assert_allclose(blocks, rows, rtol=1e-11, atol=1e-13)
+    long = plain.ROW_BY_ROW_LIMIT + 5       # beyond the limit the public function is the blocked one
+    q, k, v = rng.normal(size=(long, 2, 4)), rng.normal(size=(long, 1, 4)), rng.normal(size=(long, 1, 4))
+    np.testing.assert_array_equal(plain.causal_gqa_attention(q, k, v, 0.5, 100),
+                                  plain.causal_gqa_attention_in_blocks(q, k, v, 0.5, 100))
+
+
 def test_rope_reduces_to_a_plane_rotation_for_head_dim_two():
     x = np.array([[[1.0, 0.0]], [[0.0, 2.0]]])
     out = plain.rope_split_half(x, np.array([3, 3]), 77.0)   # hd = 2: one pair, frequency 1
