@@ -9,6 +9,7 @@ from typing import Dict, List, Sequence, Tuple
 import numpy as np
 
 import plain_qwen2 as plain
+import plain_rounded
 
 
 def round_up(value: int, multiple: int) -> int:
@@ -116,6 +117,7 @@ class PlainModel:
         self.config = plain.read_config(folder)
         self.weights = plain.read_safetensors(os.path.join(folder, "model.safetensors"))
         self._cache: Dict[tuple, np.ndarray] = {}
+        self._rounded: Dict[tuple, np.ndarray] = {}
 
     def logits(self, tokens: Sequence[int]) -> np.ndarray:
         key = tuple(tokens)
@@ -125,6 +127,37 @@ class PlainModel:
                     return rows[:len(key)]
             self._cache[key] = plain.forward(self.config, self.weights, list(tokens))
         return self._cache[key]
+
+
+    def rounded_logits(self, tokens: Sequence[int], rows: "plain_rounded.Rows", twin: bool = False) -> np.ndarray:
+        """The plain run with a bfloat16 engine's roundings (``plain_rounded``), every position flagged by ``rows``;
+        with ``twin`` the same made in another, equally valid way."""
+        key = (tuple(tokens), rows.split_norm.tobytes(), rows.round_gate_up.tobytes(), twin)
+        if key not in self._rounded:
+            self._rounded[key] = plain_rounded.forward(self.config, self.weights, list(tokens), rows,
+                                                       plain_rounded.Twin(seed=1) if twin else None)
+        return self._rounded[key]
+
+
+def rows_of_positions(steps: List[dict]) -> Dict[str, List[int]]:
+    """For every request of a trace, the number of rows (tokens of all its requests) of the step that ran each of
+    its positions."""
+    out: Dict[str, List[int]] = {}
+    for step in steps:
+        rows = sum(len(entry["tokens"]) for entry in step["entries"])
+        for entry in step["entries"]:
+            out.setdefault(entry["id"], []).extend([rows] * len(entry["tokens"]))
+    return out
+
+
+def roundings(step_rows: Sequence[int], one_weight_copy: bool = False) -> "plain_rounded.Rows":
+    """How the engine rounds a position that ran in a step of so many rows: up to ``SKINNY_ROWS`` rows its
+    products take the norms between them apart; gate and up are rounded before SiLU where the library multiplies
+    (more than ``MEDIUM_GATED_ROWS`` rows, and a copy of the weights as stored to multiply with)."""
+    from microllm_rocm_amd.parts.linear import MEDIUM_GATED_ROWS, SKINNY_ROWS
+    rows = np.asarray(step_rows)
+    return plain_rounded.Rows(split_norm=rows <= SKINNY_ROWS,
+                              round_gate_up=(rows > MEDIUM_GATED_ROWS) & (not one_weight_copy))
 
 
 # Tolerances, relative to the scale of a request's logits (largest magnitude for "max", root mean square for
@@ -161,3 +194,52 @@ def compare(got: Dict[Tuple[str, int], np.ndarray], requests: Dict[str, List[int
                 f"max error {error_max:.3e} (bound {bound['max']:.1e}), rms error {error_rms:.3e} (bound {bound['rms']:.1e})")
             worst_max, worst_rms = max(worst_max, error_max), max(worst_rms, error_rms)
     return worst_max, worst_rms
+
+
+# Against the plain run that rounds where a bfloat16 engine must (``plain_rounded``) an engine's error is no longer
+# the format's but its own arithmetic's. How small that can be is a property of the model, not of the engine: the
+# attention's probabilities are rounded against whatever maximum a kernel has seen so far, which no whole-sequence
+# run can follow, and after the first layer any difference of that size moves most later roundings to other
+# steps of the grid. ``plain_rounded.Twin`` makes the same roundings in another, equally valid way; how far its
+# logits lie from the rounded run's is how far two faithful bfloat16 implementations of this model lie apart
+# (weights N(0, 0.02): 2e-3 to 5e-3 of the logits' scale; the sharp models: 1e-2 to 1.5e-2, which is the distance to
+# the exact run too). An engine is held to that: no row further than ``ROW_FACTOR`` times the twin's worst row, and
+# the error over all rows of a request no more than ``ALL_ROWS_FACTOR`` times the twin's.
+ROW_FACTOR = 1.5
+ALL_ROWS_FACTOR = 1.0
+
+
+def compare_rounded(got: Dict[Tuple[str, int], np.ndarray], requests: Dict[str, List[int]], steps: List[dict],
+                    model: PlainModel, one_weight_copy: bool = False) -> Tuple[float, float]:
+    """Every row of a bfloat16 engine against the plain run with the same roundings, in units of the distance
+    between that run and its twin; returns (worst row's max error, worst request's error over all rows) in those
+    units."""
+    step_rows = rows_of_positions(steps)
+    worst_row = worst_request = 0.0
+    for rid, tokens in requests.items():
+        if rid not in step_rows:
+            continue
+        assert len(step_rows[rid]) == len(tokens)
+        flags = roundings(step_rows[rid], one_weight_copy)
+        reference = model.rounded_logits(tokens, flags)
+        twin = model.rounded_logits(tokens, flags, twin=True) - reference
+        places = [position for position in range(len(tokens)) if (rid, position) in got]
+        if not places:
+            continue
+        difference = np.stack([got[(rid, position)] for position in places]).astype(np.float64) - reference[places]
+        twin_max = np.abs(twin).max()                              # worst element of the twin's worst row
+        twin_rms = np.sqrt(np.mean(twin ** 2, axis=1)).max()       # worst row of the twin
+        twin_all = np.sqrt(np.mean(twin[places] ** 2))
+        row_max = np.abs(difference).max(axis=1)
+        row_rms = np.sqrt(np.mean(difference ** 2, axis=1))
+        for index, position in enumerate(places):
+            assert row_max[index] <= ROW_FACTOR * twin_max and row_rms[index] <= ROW_FACTOR * twin_rms, (
+                f"bfloat16 against the rounded plain run: first wrong row is request {rid} position {position} of "
+                f"{len(tokens)}: max error {row_max[index] / twin_max:.2f}, rms error {row_rms[index] / twin_rms:.2f} "
+                f"times the twin's worst (bound {ROW_FACTOR})")
+        overall = np.sqrt(np.mean(difference ** 2)) / twin_all
+        assert overall <= ALL_ROWS_FACTOR, (f"bfloat16 against the rounded plain run: request {rid}: the error over all "
+                                            f"rows is {overall:.2f} times the twin's (bound {ALL_ROWS_FACTOR})")
+        worst_row = max(worst_row, float((row_max / twin_max).max()), float((row_rms / twin_rms).max()))
+        worst_request = max(worst_request, float(overall))
+    return worst_row, worst_request

@@ -14,7 +14,7 @@ import torch
 
 from microllm_rocm_amd.config import Qwen2Config
 from microllm_rocm_amd.weights import write_model_folder
-from replay_tools import PlainModel, collect, compare, mixed, portions, round_up, to_lines, whole
+from replay_tools import PlainModel, collect, compare, compare_rounded, mixed, portions, round_up, to_lines, whole
 from tiny import random_tokens
 
 pytestmark = pytest.mark.gpu
@@ -76,6 +76,8 @@ def test_thousands_of_positions_under_every_cut(tmp_path_factory, tmp_path, whic
     run_trace(folder, dtype, steps, tmp_path / "prompt", max_tokens=PROMPT)
     prompt_rows = collect(steps, tmp_path / "prompt", vocab)
     compare(prompt_rows, prompt, plain_model, dtype)
+    if dtype == "bfloat16":
+        compare_rounded(prompt_rows, prompt, steps, plain_model)
 
     # (b) 4500 positions in portions of 512, then 64 single tokens
     steps = portions_then_single_tokens("long", long, 512, TAIL)
@@ -85,6 +87,8 @@ def test_thousands_of_positions_under_every_cut(tmp_path_factory, tmp_path, whic
     in_portions = collect(steps, tmp_path / "portions", vocab)
     assert max(position for _, position in in_portions) == LENGTH - 1
     compare(in_portions, {"long": long}, plain_model, dtype)
+    if dtype == "bfloat16":
+        compare_rounded(in_portions, {"long": long}, steps, plain_model)
 
     # (c) the same request, portions of up to 512 and its last 64 tokens one by one, beside shorter requests that come
     # and go, on a pool so small that their pages are used again
@@ -103,6 +107,8 @@ def test_thousands_of_positions_under_every_cut(tmp_path_factory, tmp_path, whic
     assert pool.total_taken > pool.num_pages, "the pool is small enough for pages to be used again"
     together = collect(steps, tmp_path / "mixed", vocab)
     compare(together, requests, plain_model, dtype)
+    if dtype == "bfloat16":
+        compare_rounded(together, requests, steps, plain_model)
 
     if dtype == "float32":
         steps = whole({"long": long})

@@ -10,7 +10,7 @@ import torch
 
 from microllm_rocm_amd.config import Qwen2Config
 from microllm_rocm_amd.weights import write_model_folder
-from replay_tools import PlainModel, collect, compare, mixed, prefill_then_decode, round_up, to_lines, whole
+from replay_tools import PlainModel, collect, compare, compare_rounded, mixed, prefill_then_decode, round_up, to_lines, whole
 from tiny import random_tokens
 
 pytestmark = pytest.mark.gpu
@@ -65,11 +65,15 @@ def test_real_widths_match_the_plain_implementation(tmp_path_factory, tmp_path, 
     run_trace(folder, dtype, steps, tmp_path / "whole", max_tokens=round_up(sum(len(t) for t in requests.values()), 64) + 256)
     together = collect(steps, tmp_path / "whole", config.vocab_size)
     compare(together, requests, plain_model, dtype)
+    if dtype == "bfloat16":
+        compare_rounded(together, requests, steps, plain_model)
     # most of a request in one step, the last 32 tokens one by one (few rows: the streaming products and their epilogues)
     steps = prefill_then_decode("r0", requests["r0"], tail=32)
     run_trace(folder, dtype, steps, tmp_path / "decode", max_tokens=round_up(len(requests["r0"]), 64))
     decoded = collect(steps, tmp_path / "decode", config.vocab_size)
     compare(decoded, {"r0": requests["r0"]}, plain_model, dtype)
+    if dtype == "bfloat16":
+        compare_rounded(decoded, {"r0": requests["r0"]}, steps, plain_model)
     # portions of some beside decoded tokens of others, on a pool so small that pages are used again
     steps, peak = mixed(requests, seed=5)
     engine = run_trace(folder, dtype, steps, tmp_path / "mixed", max_tokens=peak)
@@ -77,6 +81,8 @@ def test_real_widths_match_the_plain_implementation(tmp_path_factory, tmp_path, 
     assert pool.total_taken > pool.num_pages
     got = collect(steps, tmp_path / "mixed", config.vocab_size)
     compare(got, requests, plain_model, dtype)
+    if dtype == "bfloat16":
+        compare_rounded(got, requests, steps, plain_model)
     if dtype == "float32":
         for key, row in got.items():
             assert np.array_equal(row, together[key]), f"mixed: {key} differs from the request run whole"

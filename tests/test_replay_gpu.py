@@ -9,7 +9,7 @@ import sys
 import numpy as np
 import pytest
 
-from replay_tools import (PlainModel, collect, compare, mixed, portions, prefill_then_decode, round_up, to_lines,
+from replay_tools import (PlainModel, collect, compare, compare_rounded, mixed, portions, prefill_then_decode, round_up, to_lines,
                           whole)
 from tiny import CONFIGS, make_folder, random_tokens
 
@@ -62,17 +62,23 @@ def test_every_cut_matches_the_plain_implementation(tmp_path_factory, tmp_path, 
     run_trace(folder, dtype, steps, tmp_path / "whole", max_tokens=round_up(max(lengths), 64))
     results["whole"] = collect(steps, tmp_path / "whole", vocab)
     compare(results["whole"], requests, plain_model, dtype)
+    if dtype == "bfloat16":
+        compare_rounded(results["whole"], requests, steps, plain_model)
 
     for rid, tokens in requests.items():
         steps = prefill_then_decode(rid, tokens, tail=32)
         run_trace(folder, dtype, steps, tmp_path / f"decode_{rid}", max_tokens=round_up(len(tokens), 64))
         results[f"decode_{rid}"] = collect(steps, tmp_path / f"decode_{rid}", vocab)
         compare(results[f"decode_{rid}"], {rid: tokens}, plain_model, dtype)
+        if dtype == "bfloat16":
+            compare_rounded(results[f"decode_{rid}"], {rid: tokens}, steps, plain_model)
 
         steps = portions(rid, tokens, sizes=[7, 2, 5, 16, 3, 2, 33, 2, 17])
         run_trace(folder, dtype, steps, tmp_path / f"portions_{rid}", max_tokens=round_up(len(tokens), 64))
         results[f"portions_{rid}"] = collect(steps, tmp_path / f"portions_{rid}", vocab)
         compare(results[f"portions_{rid}"], {rid: tokens}, plain_model, dtype)
+        if dtype == "bfloat16":
+            compare_rounded(results[f"portions_{rid}"], {rid: tokens}, steps, plain_model)
 
     if dtype == "float32":
         # In 32-bit every kernel sums in an order that depends on the row alone: the cuts agree bit for bit.
@@ -98,6 +104,8 @@ def test_mixed_batches_with_reused_pages(tmp_path_factory, tmp_path, which, stds
     assert pool.total_taken > pool.num_pages, "the pool is small enough for pages to be used again"
     got = collect(steps, tmp_path / "mixed", config.vocab_size)
     compare(got, requests, plain_model, dtype)
+    if dtype == "bfloat16":
+        compare_rounded(got, requests, steps, plain_model)
     if dtype == "float32":
         alone = whole(requests)
         run_trace(folder, dtype, alone, tmp_path / "alone", max_tokens=round_up(max(lengths), 64))
@@ -116,6 +124,8 @@ def test_the_first_tokens_and_long_decoding(tmp_path_factory, tmp_path, dtype):
     run_trace(folder, dtype, steps, tmp_path / "long", max_tokens=round_up(len(tokens), 64))
     got = collect(steps, tmp_path / "long", config.vocab_size)
     compare(got, {"long": tokens}, plain_model, dtype)
+    if dtype == "bfloat16":
+        compare_rounded(got, {"long": tokens}, steps, plain_model)
     for count in (1, 2, 3):
         steps = whole({"first": tokens[:count]})
         run_trace(folder, dtype, steps, tmp_path / f"first{count}", max_tokens=64)
@@ -135,9 +145,11 @@ def test_one_copy_of_the_weights(tmp_path_factory, tmp_path, which):
     assert block.ffn.down_weight.tensor is None and block.ffn.down_weight.packed is not None
     assert block.mixer.qkv_weight.tensor is None and engine.model.head.weight.packed is not None
     compare(collect(steps, tmp_path / "whole", config.vocab_size), requests, plain_model, "bfloat16")
+    compare_rounded(collect(steps, tmp_path / "whole", config.vocab_size), requests, steps, plain_model, one_weight_copy=True)
     steps, peak = mixed(requests, seed=9)
     run_trace(folder, "bfloat16", steps, tmp_path / "mixed", max_tokens=peak, weight_copies="packed")
     compare(collect(steps, tmp_path / "mixed", config.vocab_size), requests, plain_model, "bfloat16")
+    compare_rounded(collect(steps, tmp_path / "mixed", config.vocab_size), requests, steps, plain_model, one_weight_copy=True)
     both = run_trace(folder, "bfloat16", whole({"r0": requests["r0"]}), tmp_path / "both", max_tokens=256)
     assert both.weight_copies == "both" and both.model.blocks[0].ffn.down_weight.tensor is not None
 
