@@ -1,10 +1,10 @@
-"""The cache manager: pages of keys and values with a block table per request, and state slots.
+"""The cache manager: pages with a block table per request, and state slots.
 
-Run entries of the model declare what they need: keys and values in pages
-(``PagedKVNeed``, perhaps with a window) or per-request state of fixed size
-(``StateNeed``). Entries with equal paged needs form a group; a group has a pool
-and page arrays of its own, keys and values per entry (laid out in tiles of 16 positions, see
-``cache.layout``), and every request has one block table per group. Pages are taken when
+Run entries of the model declare what they need (``cache.needs``): something in pages
+(keys and values, ``PagedKVNeed``, perhaps with a window; or whatever payload a need's class
+allocates) or per-request state of fixed size (``StateNeed``). Entries with equal paged needs form a
+group; a group has a pool of its own, every entry its own page arrays (keys and values lie in tiles of
+16 positions, see ``cache.layout``), and every request has one block table per group. Pages are taken when
 a request's tokens cross a page's edge, given back when the request is closed,
 and, in a group with a window, as soon as every position on them is older than
 any later query can see. Nothing is cleared on reuse: lengths, not contents,
@@ -19,29 +19,10 @@ from typing import Dict, Hashable, List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..parts.base import CacheNeed, PagedKVNeed, StateNeed
-from .layout import check_sizes, key_page_shape, value_page_shape
+from .needs import Binding, CacheNeed, PagedBinding, PagedKVNeed, StateBinding, StateNeed
 from .pages import OutOfPages, PagePool, SlotPool
 
 RELEASED = -1  # block-table entry of a page that a window has passed
-
-
-@dataclass
-class PagedBinding:
-    """What a mixer gets for paged keys and values: its entry's page arrays and its group."""
-    group: int
-    need: PagedKVNeed
-    k: Optional[torch.Tensor]
-    v: Optional[torch.Tensor]
-    owned: bool = True
-
-
-@dataclass
-class StateBinding:
-    """What a mixer gets for per-request state: ``state[slot]`` is the request's, zero when it opens."""
-    need: StateNeed
-    state: Optional[torch.Tensor]
-    owned: bool = True
 
 
 @dataclass
@@ -56,7 +37,7 @@ class RequestCache:
 
 
 class CacheGroup:
-    def __init__(self, index: int, need: PagedKVNeed, num_pages: int, page_size: int, max_requests: int,
+    def __init__(self, index: int, need: CacheNeed, num_pages: int, page_size: int, max_requests: int,
                  max_blocks: int):
         self.index = index
         self.need = need
@@ -81,7 +62,7 @@ def window_blocks(window: int, portion: int, page_size: int) -> int:
     return -(-(window - 1 + portion) // page_size) + 1
 
 
-def pages_of_group(need: PagedKVNeed, num_pages: int, page_size: int, max_requests: int,
+def pages_of_group(need: CacheNeed, num_pages: int, page_size: int, max_requests: int,
                    max_portion: Optional[int]) -> int:
     """How many pages a group's pool gets of the ``num_pages`` asked for: all of them, unless the group has a
     window and the largest portion of a step is known; then no more than every request slot can hold at once."""
@@ -101,8 +82,6 @@ class CacheManager:
         blocks a request's table has (its positions / page size); by default the pool's size."""
         if page_size <= 0:
             raise ValueError("page_size must be positive")
-        if device is not None:
-            check_sizes(page_size, 1)   # device pages are tiled by 16 positions; the bookkeeping alone is not
         if len(needs) != len(reads):
             raise ValueError("one need and one read source per run entry")
         self.page_size = page_size
@@ -114,13 +93,17 @@ class CacheManager:
         self.groups: List[CacheGroup] = []
         self.slots = SlotPool(max_requests)
         self.requests: Dict[Hashable, RequestCache] = {}
-        self._bindings: List[object] = [None] * len(needs)
-        self._state_tensors: List[torch.Tensor] = []
-        by_need: Dict[PagedKVNeed, CacheGroup] = {}
+        self._bindings: List[Optional[Binding]] = [None] * len(needs)
+        self._slot_storage: List[tuple] = []        # (need, storage) of every run entry that keeps state in slots
+        by_need: Dict[CacheNeed, CacheGroup] = {}
         for entry, need in enumerate(needs):
-            if reads[entry] is not None:
+            if reads[entry] is not None or need is None:
                 continue
-            if isinstance(need, PagedKVNeed):
+            if not isinstance(need, CacheNeed):
+                raise TypeError(f"run entry {entry} declares an unknown cache need {need!r}")
+            if need.paged:
+                if device is not None:
+                    need.check_page_size(page_size)   # the layout on the device may ask more of a page than the books do
                 group = by_need.get(need)
                 if group is None:
                     group = CacheGroup(len(self.groups), need, pages_of_group(need, num_pages, page_size, max_requests, max_portion),
@@ -128,37 +111,27 @@ class CacheManager:
                     self.groups.append(group)
                     by_need[need] = group
                 group.entries.append(entry)
-                k = v = None
-                if device is not None:
-                    # Zeroed once: a kernel may read a whole tile whose tail was never written.
-                    k = torch.zeros(key_page_shape(group.pool.num_pages, need.kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
-                    v = torch.zeros(value_page_shape(group.pool.num_pages, need.kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
-                self._bindings[entry] = PagedBinding(group.index, need, k, v, owned=True)
-            elif isinstance(need, StateNeed):
-                state = None
-                if device is not None:
-                    state = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
-                    self._state_tensors.append(state)
-                self._bindings[entry] = StateBinding(need, state, owned=True)
-            elif need is not None:
-                raise TypeError(f"run entry {entry} declares an unknown cache need {need!r}")
+                storage = need.allocate_pages(group.pool.num_pages, page_size, dtype, device) if device is not None else None
+                self._bindings[entry] = need.bind(group.index, storage, True)
+            else:
+                storage = need.allocate_slots(max_requests, dtype, device) if device is not None else None
+                if storage is not None:
+                    self._slot_storage.append((need, storage))
+                self._bindings[entry] = need.bind(None, storage, True)
         for entry, source in enumerate(reads):
             if source is None:
                 continue
             binding = self._bindings[source]
             if binding is None:
                 raise ValueError(f"run entry {entry} reads the cache of entry {source}, which has none")
-            if isinstance(binding, PagedBinding):
-                self._bindings[entry] = PagedBinding(binding.group, binding.need, binding.k, binding.v, owned=False)
-            else:
-                self._bindings[entry] = StateBinding(binding.need, binding.state, owned=False)
+            self._bindings[entry] = binding.shared()
 
     # ---- what the model sees -------------------------------------------------------------
     @property
     def has_state(self) -> bool:
         """Whether any run entry keeps per-request state of fixed size (which, unlike pages, a failed step cannot
         simply leave behind)."""
-        return any(isinstance(binding, StateBinding) and binding.owned for binding in self._bindings)
+        return any(binding is not None and not binding.need.paged and binding.owned for binding in self._bindings)
 
     def bindings(self) -> List[object]:
         return list(self._bindings)
@@ -168,8 +141,8 @@ class CacheManager:
         if request_id in self.requests:
             raise KeyError(f"request {request_id!r} is already open")
         slot = self.slots.take_one()
-        for state in self._state_tensors:
-            state[slot].zero_()
+        for need, storage in self._slot_storage:
+            need.zero_slot(storage, slot)
         request = RequestCache(request_id, slot, pages=[[] for _ in self.groups])
         self.requests[request_id] = request
         return request
@@ -269,8 +242,12 @@ class CacheManager:
         return [group.pool.num_held for group in self.groups]
 
     def bytes_per_page(self, group: CacheGroup) -> int:
-        element = torch.empty((), dtype=self.dtype).element_size()
-        return 2 * len(group.entries) * group.need.kv_heads * self.page_size * group.need.head_dim * element
+        return len(group.entries) * self.page_size * group.need.bytes_per_position(self.dtype)
+
+    def state_bytes(self) -> int:
+        """Bytes of the slots of every run entry that keeps per-request state, for all request slots."""
+        return sum(self.max_requests * binding.need.bytes_per_request(self.dtype) for binding in self._bindings
+                   if binding is not None and not binding.need.paged and binding.owned)
 
     def allocated_bytes(self) -> int:
         return sum(self.bytes_per_page(group) * group.pool.num_pages for group in self.groups)

@@ -193,6 +193,7 @@ def run(options: Dict[str, object]) -> int:
     from ..config import load_config
     from ..engine.benchmark import decode_throughput, prefill_throughput
     from ..engine.batch import StepEntry
+    from ..ops.transfers import on_host, reset_transfer_stats, transfer_stats
 
     tokens = integers(str(options["tokens"]), "--tokens")
     prompt_lengths = integers(str(options["prompt-lengths"]), "--prompt-lengths")
@@ -241,6 +242,16 @@ def run(options: Dict[str, object]) -> int:
               "kv_block_size": block_size, "kv_blocks": engine.cache.groups[0].pool.num_pages if engine.cache.groups else 0,
               "allocated_cache_bytes": engine.cache.allocated_bytes(), "weight_copies": engine.weight_copies}
     stop_tokens = tuple(integers(str(options["stop-tokens"]), "--stop-tokens"))
+
+    def measured_transfers() -> dict:
+        """Copies between host and device since the engine was loaded, warm-up runs included, under the reference's
+        keys (apps/hf_infer.cpp:1001-1012, 1407-1418)."""
+        moved = transfer_stats()
+        return {"measured_h2d_calls": moved.host_to_device_calls, "measured_h2d_bytes": moved.host_to_device_bytes,
+                "measured_d2h_calls": moved.device_to_host_calls, "measured_d2h_bytes": moved.device_to_host_bytes,
+                "measured_d2d_calls": moved.device_to_device_calls, "measured_d2d_bytes": moved.device_to_device_bytes}
+
+    reset_transfer_stats()
     params = GenerationConfig(max_new_tokens=new_tokens, temperature=float(options["temperature"]),
                               top_k=int(options["sample-top-k"]), seed=int(options["seed"]), stop_tokens=stop_tokens)
 
@@ -296,6 +307,7 @@ def run(options: Dict[str, object]) -> int:
             "kv_cache_byte_utilization": round(metrics.peak_held_pages / max(1, report["kv_blocks"]), 4),
             "generated": generated, "token_checksum": int(sum((i + 1) * t for g in generated for i, t in enumerate(g)) % (1 << 31)),
         })
+        report.update(measured_transfers())
         print(json.dumps(report), flush=True)
         return 0
 
@@ -332,7 +344,7 @@ def run(options: Dict[str, object]) -> int:
                 engine.close(request_id)
         report["prefill_ms"] = round(min(timings) * 1e3, 3)
         report["prefill_tokens_per_second"] = round(batch * len(tokens) / min(timings), 3)
-        last = logits[0].cpu().numpy()
+        last = on_host(logits[0]).numpy()
         top = np.argsort(-last, kind="stable")[:int(options["top-k"])]
         report["top_logits"] = [[int(index), float(last[index])] for index in top]
         if options["logits-output"]:
@@ -344,19 +356,19 @@ def run(options: Dict[str, object]) -> int:
         report["decode_ms_per_step"] = round(steady["ms_per_step"], 4)
     if options["workload"] == "both" and new_tokens > 0:
         from ..ops import kernels
-        on_host = options["batch-argmax-mode"] == "host"
+        argmax_on_host = options["batch-argmax-mode"] == "host"
 
         def engine_argmax(logits):
-            chosen = kernels.argmax(logits).tolist()
+            chosen = on_host(kernels.argmax(logits)).tolist()
             if min(chosen) < 0:
                 raise RuntimeError("a row of the logits is not finite")
             return chosen
 
         def first_maximum(logits):
             """Greedy choice per row, on the device or (--batch-argmax-mode host) from the rows copied out."""
-            if not on_host:
+            if not argmax_on_host:
                 return engine_argmax(logits)
-            rows = logits.cpu().numpy()
+            rows = on_host(logits).numpy()
             if not np.isfinite(rows).all():
                 raise RuntimeError("a row of the logits is not finite")
             return [int(np.argmax(row)) for row in rows]
@@ -400,7 +412,7 @@ def run(options: Dict[str, object]) -> int:
             return sequences, logits
 
         greedy = params.temperature == 0.0 or params.top_k == 1
-        explicit = not use_cache or options["cache-prefill-mode"] == "token" or options["cache-logits-output"] or on_host
+        explicit = not use_cache or options["cache-prefill-mode"] == "token" or options["cache-logits-output"] or argmax_on_host
         if explicit and not greedy:
             raise UsageError("--use-cache false, --cache-prefill-mode token, --batch-argmax-mode host and "
                              "--cache-logits-output are for greedy generation (--temperature 0)")
@@ -421,7 +433,7 @@ def run(options: Dict[str, object]) -> int:
                 raise RuntimeError("deterministic generation changed across steps")      # apps/hf_infer.cpp:1285-1287
             outputs = current
             if options["cache-logits-output"] and last_logits is not None:
-                last_logits.cpu().numpy().astype("<f4").tofile(str(options["cache-logits-output"]))   # apps/hf_infer.cpp:1297-1305
+                on_host(last_logits).numpy().astype("<f4").tofile(str(options["cache-logits-output"]))   # apps/hf_infer.cpp:1297-1305
         runs = max(1, int(options["steps"])) if options["decode-mode"] == "generation" else 1
         report["generated_tokens"] = outputs[0][len(tokens):]
         report["generation_ms"] = round(elapsed * 1e3, 3)
@@ -430,5 +442,6 @@ def run(options: Dict[str, object]) -> int:
                        "batch_argmax_mode": options["batch-argmax-mode"]})
     report["prefill_logits_mode"] = options["prefill-logits"]
     report["prompt_tokens"] = len(tokens)
+    report.update(measured_transfers())
     print(json.dumps(report), flush=True)
     return 0

@@ -15,6 +15,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, RELEASED, RequestCache
+from ..ops.transfers import copy_to_device, on_device
 
 
 @dataclass
@@ -137,7 +138,7 @@ class StepContext:
         if plan is None:
             arrays, values = planner.plan(self.host)
             device = self.tokens.device
-            plan = SimpleNamespace(**values, **{name: torch.from_numpy(np.ascontiguousarray(array, dtype=np.int32)).to(device)
+            plan = SimpleNamespace(**values, **{name: on_device(np.ascontiguousarray(array, dtype=np.int32), device)
                                                 for name, array in arrays.items()})
             self.planned[planner.key] = plan
         return plan
@@ -179,7 +180,7 @@ class BatchBuilder:
         if self._copied is not None:
             self._copied.synchronize()
         self._staging.numpy()[:count] = tokens
-        self._device_buffer[:count].copy_(self._staging[:count], non_blocking=True)
+        copy_to_device(self._device_buffer[:count], self._staging[:count], non_blocking=True)
         self._copied = torch.cuda.Event()
         self._copied.record()
 
@@ -293,7 +294,7 @@ class BatchBuilder:
         host = staging.numpy()
         for offset, piece in zip(offsets, pieces):
             host[offset:offset + piece.size] = piece
-        device_buffer[:cursor].copy_(staging[:cursor], non_blocking=True)
+        copy_to_device(device_buffer[:cursor], staging[:cursor], non_blocking=True)
         self._copied = torch.cuda.Event()
         self._copied.record()
 

@@ -12,7 +12,6 @@ from typing import Dict
 import numpy as np
 import torch
 
-from ..cache.manager import PagedBinding
 from ..parts.linear import Weight
 from ..sampling import Sampler, SamplingParams
 from .batch import StepEntry
@@ -21,9 +20,9 @@ from .engine import Engine
 
 def _fill_random(engine: Engine) -> None:
     for binding in engine.cache.bindings():
-        if isinstance(binding, PagedBinding) and binding.owned:
-            binding.k.normal_(0.0, 1.0)
-            binding.v.normal_(0.0, 1.0)
+        if binding is not None and binding.need.paged and binding.owned:
+            for tensor in binding.tensors():
+                tensor.normal_(0.0, 1.0)
 
 
 def decode_throughput(engine: Engine, batch: int, context: int, steps: int, warmup: int, seed: int = 0) -> Dict[str, float]:
@@ -110,31 +109,19 @@ def weight_bytes(engine: Engine) -> int:
 
 def step_bytes(engine: Engine, batch: int, context: int) -> int:
     """What a decode step has to read: every weight once, the cache of the live requests, one embedding row each."""
-    element = torch.empty((), dtype=engine.dtype).element_size()
     cache = 0
     for group in engine.cache.groups:
         visible = context if group.need.window is None else min(context, group.need.window)
-        cache += 2 * len(group.entries) * group.need.kv_heads * group.need.head_dim * visible * element
-    row = engine.spec.hidden_size * engine.model.embedding.table.element_size()
-    return weight_bytes(engine) + batch * (cache + row)
+        cache += len(group.entries) * visible * group.need.bytes_per_position(engine.dtype)
+    cache += engine.cache.state_bytes() // engine.cache.max_requests
+    return weight_bytes(engine) + batch * cache + engine.model.embedding.bytes_read(batch, context)
 
 
 def step_flops(engine: Engine, tokens: int) -> float:
     """Floating-point operations of one prompt of ``tokens`` ids: 2 per multiply-add of every matrix product over
     all tokens (the head for one row) and of causal attention (scores and values)."""
-    flops = 0.0
-    for block in engine.model.blocks:
-        for part in block.parts():
-            for name, value in vars(part).items():
-                if isinstance(value, Weight):
-                    flops += 2.0 * value.out_features * value.in_features * tokens
-        mixer = block.mixer
-        if hasattr(mixer, "heads"):
-            window = mixer.window or tokens
-            pairs = sum(min(position + 1, window) for position in range(tokens))
-            flops += 4.0 * mixer.heads * mixer.head_dim * pairs
-    flops += 2.0 * engine.model.head.weight.out_features * engine.model.head.weight.in_features
-    return flops
+    flops = sum(part.flops(tokens) for block in engine.model.blocks for part in block.parts())
+    return flops + engine.model.head.flops(tokens, wanted=1)
 
 
 def percentile(values, quantile: float) -> float:

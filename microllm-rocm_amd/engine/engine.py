@@ -10,7 +10,6 @@ with its own batch shape (src/model/model.cpp:1091-1135, 1263-1303, 1316-1354,
 from __future__ import annotations
 
 import os
-from collections import OrderedDict
 from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Union
 
 import torch
@@ -19,9 +18,11 @@ from ..cache.manager import CacheManager, RequestCache, pages_of_group
 from ..cache.pages import OutOfPages
 from ..config.registry import architecture_named, load_config
 from ..ops import kernels, library
+from ..ops.transfers import device_copy, on_device
 from ..parts import Model, ModelSpec, Runtime
 from ..weights import load_folder, place_all, random_tensors
 from .batch import BatchBuilder, FixedShape, HostBatch, StepContext, StepEntry
+from .graphs import GraphPolicy
 
 _DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": torch.bfloat16, "bf16": torch.bfloat16}
 
@@ -38,10 +39,13 @@ def parse_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
 
 MAX_GRAPH_REQUESTS = 256
 MIN_GRAPH_WIDTH = 16
-MAX_GRAPHS = 48     # captured steps kept at a time; the one replayed longest ago goes first
+DECODE_GRAPHS = 32          # captured steps of single tokens kept at a time; the one replayed longest ago goes first
+MIXED_GRAPHS = 16           # and captured mixed steps, which have a budget of their own (engine/graphs.py)
+GRAPH_LOGITS_BYTES = 2 << 30    # what the kept graphs' logits may hold together
 MAX_GRAPH_TOKENS = 4096     # mixed steps of more tokens run eagerly: their launches no longer cost more than their kernels
 MAX_GRAPH_WANTED = 256
 SHAPE_SEEN_TWICE = 2        # a mixed step's shape is captured when it comes for the second time
+WANTED_ROWS = (1, 2, 4, 8, 16, 32, 40, 48, 64, 128, 256)    # what the wanted rows of a mixed step are padded to
 
 
 def _power_of_two(value: int, least: int = 1) -> int:
@@ -49,10 +53,19 @@ def _power_of_two(value: int, least: int = 1) -> int:
 
 
 def _token_rows(tokens: int) -> int:
-    """Rows a mixed step of ``tokens`` tokens is padded to: steps of 16 up to 128, of 64 up to 1024, then of 256
-    (at most an eighth more rows than tokens from 128 on)."""
+    """Rows a mixed step of ``tokens`` tokens is padded to: steps of 16 up to 128 (and 40), of 64 up to 1024, then
+    of 256 (at most an eighth more rows than tokens from 128 on). No padded count lies on the other side of a row
+    count at which a product changes its kernel (16, 40, 48, 64; ``parts.linear``) than the count itself: the
+    padded step then gives the bits of the step run as it is."""
+    if 32 < tokens <= 40:
+        return 40
     step = 16 if tokens <= 128 else (64 if tokens <= 1024 else 256)
     return -(-tokens // step) * step
+
+
+def _wanted_rows(wanted: int) -> int:
+    """Rows the head's product is padded to in a mixed step; the same rule about kernels' row counts."""
+    return next(rows for rows in WANTED_ROWS if rows >= max(wanted, 1))
 
 
 class _DecodeGraph:
@@ -63,6 +76,7 @@ class _DecodeGraph:
         self.width = width
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
+        self.held_bytes = 0         # of its logits, once captured
 
 
 class _BuiltAhead:
@@ -107,6 +121,7 @@ class Engine:
         self.device = torch.device(device)
         torch.cuda.set_device(self.device)
         self.spec = spec
+        self._policy = GraphPolicy(DECODE_GRAPHS, MIXED_GRAPHS, GRAPH_LOGITS_BYTES, SHAPE_SEEN_TWICE)
         if num_pages is None:
             if max_tokens is None:
                 raise ValueError("give max_tokens or num_pages: the cache pool is sized once")
@@ -137,10 +152,9 @@ class Engine:
         self.use_graphs = use_graphs and all(part.graph_safe for part in self.model.parts())
         self._graphs_allowed = self.use_graphs
         # All captures share one memory pool: a graph's activations live only while it runs, so the next graph may
-        # have them; what a graph hands out (its logits) stays its own while the graph is kept. At most
-        # MAX_GRAPHS are kept (continuous batching walks through many numbers of requests): each holds its
-        # logits [requests, vocabulary] in float32 and its metadata buffers.
-        self._graphs: "OrderedDict[tuple, _DecodeGraph]" = OrderedDict()
+        # have them; what a graph hands out (its logits) stays its own while the graph is kept. How many are kept,
+        # and of which kind, is the policy's business (continuous batching walks through many numbers of
+        # requests): each holds its logits [rows, vocabulary] in float32 and its metadata buffers.
         self._graph_pool = None
         self.graph_replays = 0
         self.graphs_captured = 0
@@ -148,7 +162,6 @@ class Engine:
         # from graphs too, once a shape has come twice: for small models such a step's launches cost the host
         # more time than its kernels cost the GPU.
         self.graph_mixed_steps = graph_mixed_steps
-        self._shape_seen: Dict[tuple, int] = {}
         self.mixed_graph_replays = 0
 
     def _two_copies_fit(self, model: Model, decls, num_pages: int, page_size: int, max_requests: int,
@@ -156,15 +169,20 @@ class Engine:
         """Whether the weights as stored, their packed copies and the cache pool fit the GPU with a tenth to spare."""
         if self.dtype != torch.bfloat16:
             return True     # a float32 engine has no packed copies
-        element = 2
-        weights = sum(element * int(torch.Size(decl.shape).numel()) for decl in decls.values())
+        weights = sum(2 * int(torch.Size(decl.shape).numel()) for decl in decls.values())
         cache = 0
         for need in model.cache_needs():
-            if need is not None and hasattr(need, "kv_heads"):
-                pages = pages_of_group(need, num_pages, page_size, max_requests, max_portion)
-                cache += 2 * pages * page_size * need.kv_heads * need.head_dim * element
+            if need is None:
+                continue
+            if need.paged:
+                cache += pages_of_group(need, num_pages, page_size, max_requests, max_portion) * page_size * need.bytes_per_position(self.dtype)
+            else:
+                cache += max_requests * need.bytes_per_request(self.dtype)
+        # What graphs keep: their logits up to the policy's bound, and one pool with the activations of the largest
+        # captured step (a few dozen float32 rows of the stream's width per token covers every part here).
+        graphs = self._policy.most_bytes + MAX_GRAPH_TOKENS * model.spec.hidden_size * 64
         total = torch.cuda.get_device_properties(self.device).total_memory
-        return 2 * weights + cache <= 0.9 * total
+        return 2 * weights + cache + graphs <= 0.9 * total
 
     # ---- construction --------------------------------------------------------------------
     @classmethod
@@ -203,19 +221,21 @@ class Engine:
     def is_open(self, request_id: Hashable) -> bool:
         return request_id in self.cache.requests
 
+    @property
+    def kept_graphs(self) -> int:
+        """Captured steps held at the moment, of both kinds."""
+        return len(self._policy)
+
     # ---- decode steps from graphs ---------------------------------------------------------
     def _graph_step(self, requests: List[RequestCache], entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         n = len(entries)
         widest = -(-(max(request.num_tokens for request in requests) + 1) // self.cache.page_size)
         width = max(MIN_GRAPH_WIDTH, 1 << (max(widest, 1) - 1).bit_length())
         key = (n, width)
-        state = self._graphs.get(key)
+        state = self._policy.decode.get(key)
         if state is None:
-            while len(self._graphs) >= MAX_GRAPHS:
-                self._graphs.popitem(last=False)
-            state = self._graphs[key] = _DecodeGraph(self, width)
-        else:
-            self._graphs.move_to_end(key)
+            state = _DecodeGraph(self, width)
+            self._policy.decode.put(key, state)
         every_row = [[0]] * n   # the graph computes the logits of every row; the wanted ones are picked after
         ahead, self._ahead = self._ahead, None
         if ahead is not None and state.graph is not None and ahead.holds_for(state, requests):
@@ -227,14 +247,15 @@ class Engine:
         self._last_graph = state
         if state.graph is None:
             self._capture(state, ctx)
+            self._policy.decode.trim(keep=key)
         state.graph.replay()
         self.graph_replays += 1
         wanted = [index for index, entry in enumerate(entries) if len(entry.want) > 0]
         if not wanted:
             return None
         if len(wanted) == n:
-            return state.logits if self._borrow else state.logits.clone()
-        return state.logits[torch.tensor(wanted, device=self.device)]
+            return state.logits if self._borrow else device_copy(state.logits)
+        return state.logits[on_device(wanted, self.device, dtype=torch.int64)]
 
     # ---- mixed steps from graphs -----------------------------------------------------------
     def _fixed_shape(self, batch: HostBatch) -> Optional[FixedShape]:
@@ -245,28 +266,21 @@ class Engine:
         if step.n_tokens > MAX_GRAPH_TOKENS or step.n_seqs > MAX_GRAPH_REQUESTS or wanted > MAX_GRAPH_WANTED:
             return None
         shape = FixedShape(tokens=_token_rows(step.n_tokens), requests=_power_of_two(step.n_seqs),
-                           wanted=_power_of_two(wanted), width=_power_of_two(batch.blocks_needed, MIN_GRAPH_WIDTH),
+                           wanted=_wanted_rows(wanted), width=_power_of_two(batch.blocks_needed, MIN_GRAPH_WIDTH),
                            planned={name: _power_of_two(rows) for name, rows in batch.planned_rows().items()})
-        key = shape.key()
-        if key in self._graphs:
-            return shape
-        if len(self._shape_seen) > 4096:
-            self._shape_seen.clear()
-        seen = self._shape_seen[key] = self._shape_seen.get(key, 0) + 1
-        return shape if seen >= SHAPE_SEEN_TWICE else None
+        return shape if self._policy.wants_mixed(shape.key()) else None
 
     def _mixed_graph_step(self, shape: FixedShape, batch: HostBatch) -> Optional[torch.Tensor]:
         key = shape.key()
-        state = self._graphs.get(key)
+        state = self._policy.mixed.get(key)
         if state is None:
-            while len(self._graphs) >= MAX_GRAPHS:
-                self._graphs.popitem(last=False)
-            state = self._graphs[key] = _DecodeGraph(self, shape.width)
-        else:
-            self._graphs.move_to_end(key)
+            state = _DecodeGraph(self, shape.width)
+            self._policy.mixed.put(key, state, self._policy.evicted_mixed)
         ctx = state.builder.upload(batch, fixed=shape)
         if state.graph is None:
             self._capture(state, ctx)
+            self._policy.captured_mixed(key)
+            self._policy.mixed.trim(self._policy.evicted_mixed, keep=key)
         state.graph.replay()
         self.graph_replays += 1
         self.mixed_graph_replays += 1
@@ -274,7 +288,7 @@ class Engine:
         if wanted == 0:
             return None
         logits = state.logits[:wanted]
-        return logits if self._borrow else logits.clone()
+        return logits if self._borrow else device_copy(logits)
 
     def _capture(self, state: "_DecodeGraph", ctx: StepContext) -> None:
         """Once eagerly (libraries create their handles and workspaces), then the capture. The step writes the same
@@ -288,6 +302,7 @@ class Engine:
         with torch.cuda.graph(graph, pool=self._graph_pool):
             state.logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
         state.graph = graph
+        state.held_bytes = state.logits.numel() * state.logits.element_size() if state.logits is not None else 0
         self.graphs_captured += 1
 
     # ---- the step ------------------------------------------------------------------------

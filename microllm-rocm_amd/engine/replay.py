@@ -17,6 +17,7 @@ from typing import IO, Optional
 import numpy as np
 import torch
 
+from ..ops.transfers import on_host
 from .batch import StepEntry
 from .engine import Engine
 
@@ -49,14 +50,14 @@ def replay(engine: Engine, lines: IO[str], out_dir: str, report: Optional[IO[str
         streams.clear()
         logits = engine.step(entries) if entries else None
         if logits is not None:
-            array = logits.detach().to("cpu").numpy().astype("<f4", copy=False)
+            array = on_host(logits).numpy().astype("<f4", copy=False)
             array.tofile(os.path.join(out_dir, f"{step}.f32"))
             if dump_layers:
                 rows, first = [], 0
                 for entry in entries:
                     rows += [first + place for place in entry.want]
                     first += len(entry.tokens)
-                wanted = torch.stack(streams)[:, rows].to("cpu").numpy().astype("<f4", copy=False)
+                wanted = on_host(torch.stack(streams)[:, rows]).numpy().astype("<f4", copy=False)
                 wanted.tofile(os.path.join(out_dir, f"{step}.layers.f32"))
         for request_id in record.get("end", []):
             if engine.is_open(request_id):

@@ -124,6 +124,12 @@ class PagedAttention(Mixer):
             return None
         return PagedKVNeed(self.kv_heads, self.head_dim, self.window)
 
+    def flops(self, tokens: int) -> float:
+        """The projections', and 4 per (query, visible key, head, dim): scores and weighted values."""
+        window = self.window or tokens
+        pairs = sum(min(position + 1, window) for position in range(tokens))
+        return super().flops(tokens) + 4.0 * self.heads * self.head_dim * pairs
+
     # ---- forward -------------------------------------------------------------------------
     def takes_unscaled(self, rows: int) -> bool:
         return self.qkv_weight.row_order is not None and takes_unscaled(self.qkv_weight, rows)

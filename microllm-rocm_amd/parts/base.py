@@ -12,6 +12,7 @@ from typing import Dict, Mapping, Optional, Sequence, Tuple, Union
 
 import torch
 
+from ..cache.needs import CacheNeed, PagedKVNeed, StateNeed
 from .spec import PartSpec
 
 MATRIX = "matrix"   # a float matrix or table: float32 stays float32, bfloat16 stays bfloat16 in a bfloat16 engine
@@ -33,24 +34,6 @@ class Runtime:
     dtype: torch.dtype
     device: torch.device
     keep_plain_weights: bool = True
-
-
-@dataclass(frozen=True)
-class PagedKVNeed:
-    """Keys and values in pages; ``window`` is None when every key stays needed."""
-    kv_heads: int
-    head_dim: int
-    window: Optional[int] = None
-
-
-@dataclass(frozen=True)
-class StateNeed:
-    """Per-request state of fixed size: one slot of ``shape`` and ``dtype`` per live request."""
-    shape: Tuple[int, ...]
-    dtype: torch.dtype = torch.float32
-
-
-CacheNeed = Union[PagedKVNeed, StateNeed, None]
 
 
 class Part:
@@ -82,6 +65,12 @@ class Part:
         the step's other metadata; None otherwise. ``ctx.plan_of(planner)`` gives the plan in ``forward``."""
         return None
 
+    def flops(self, tokens: int) -> float:
+        """Floating-point operations of this part over one request's prompt of ``tokens`` ids (2 per multiply-add);
+        by default those of its matrix products, found as attributes with ``out_features`` and ``in_features``."""
+        return sum(2.0 * value.out_features * value.in_features * tokens for value in vars(self).values()
+                   if hasattr(value, "out_features") and hasattr(value, "in_features"))
+
     def name(self, role: str) -> str:
         try:
             return self.spec.names[role]
@@ -97,7 +86,9 @@ class Mixer(Part):
     def takes_unscaled(self, rows: int) -> bool:
         return False
 
-    def cache_need(self) -> CacheNeed:
+    def cache_need(self) -> Optional[CacheNeed]:
+        """What this mixer keeps between steps (``cache.needs``): ``PagedKVNeed``, ``StateNeed``, a need class of
+        its own, or None."""
         return None
 
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:

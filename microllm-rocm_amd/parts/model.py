@@ -20,7 +20,8 @@ from .spec import ModelSpec, PartSpec
 
 
 class TokenEmbedding(Part):
-    """``h0[t] = E[id_t]`` widened to float32 (src/model/model.cpp:1111)."""
+    """``h0[t] = E[id_t]`` widened to float32 (src/model/model.cpp:1111). An embedding part is handed the whole
+    step, so that one which also needs positions or requests (learned positions, token types) finds them."""
     category = "embedding"
     graph_safe = True
 
@@ -36,8 +37,11 @@ class TokenEmbedding(Part):
     def bind(self, tensors):
         self.table = tensors[self.name("weight")]
 
-    def forward(self, ids: torch.Tensor) -> torch.Tensor:
-        return kernels.embedding(self.table, ids)
+    def forward(self, ctx) -> torch.Tensor:
+        return kernels.embedding(self.table, ctx.tokens)
+
+    def bytes_read(self, rows: int, context: int) -> int:
+        return rows * self.width * self.table.element_size()     # a row per token, not the table
 
 
 class LMHead(Part):
@@ -60,6 +64,9 @@ class LMHead(Part):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return linear(x, self.weight, out_dtype=torch.float32)
+
+    def flops(self, tokens: int, wanted: int = 1) -> float:
+        return 2.0 * self.vocab * self.width * wanted     # logits at the wanted rows only
 
 
 register_part("embedding", "token_embedding", TokenEmbedding)
@@ -151,9 +158,9 @@ class Model:
                 planners.append(planner)
         return planners
 
-    def cache_needs(self) -> List[CacheNeed]:
+    def cache_needs(self) -> List[Optional[CacheNeed]]:
         """The cache need of every run entry; None for an entry that owns none."""
-        needs: List[CacheNeed] = []
+        needs: List[Optional[CacheNeed]] = []
         for entry in self.spec.order:
             need = self.blocks[entry.layer].mixer.cache_need()
             needs.append(None if entry.reads_cache_of is not None else need)
@@ -166,7 +173,7 @@ class Model:
         ``caches[i]`` is the cache binding of run entry ``i`` (its own, or the one it reads).
         ``want_rows`` indexes the step's flat token list; None or empty skips the head.
         """
-        h = self.embedding.forward(ctx.tokens)
+        h = self.embedding.forward(ctx)
         pending = None
         order = self.spec.order
         for index, entry in enumerate(order):

@@ -20,6 +20,7 @@ import numpy as np
 import torch
 
 from ..ops import kernels
+from ..ops.transfers import on_device, on_host
 
 _MASK = (1 << 64) - 1
 
@@ -78,12 +79,12 @@ class Sampler:
             packed[0] = [0.0 if p.greedy else p.temperature for p in params]
             packed[1].view(np.int32)[:] = [p.top_k for p in params]
             packed[2] = [uniform_for(p.seed, d) for p, d in zip(params, draws)]
-            on_device = torch.from_numpy(packed).to(logits.device)
-            temperature, top_k, uniform = on_device[0], on_device[1].view(torch.int32), on_device[2]
+            values = on_device(packed, logits.device)
+            temperature, top_k, uniform = values[0], values[1].view(torch.int32), values[2]
             if all(p.top_k == 0 for p in params):
                 top_k = None      # no row is restricted: the kernel leaves its search for the k-th value out
             chosen = kernels.sample(logits, temperature, top_k, uniform)
-        tokens = chosen.tolist()
+        tokens = on_host(chosen).tolist()
         for row, token in enumerate(tokens):
             if token < 0:
                 raise NonFiniteLogits(f"row {row} of the logits is not finite")

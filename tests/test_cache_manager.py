@@ -114,6 +114,48 @@ def test_state_slots_and_shared_caches():
         CacheManager([None, None], [None, 0], 16, 4, 2, device=None)
 
 
+def test_a_need_class_from_outside_is_grouped_sized_and_counted_like_the_package_s_own():
+    """The manager asks a need how it lives (pages or slots), what a position costs and what to hand the mixer;
+    it lists no kinds. Something that is no need at all is refused by name."""
+    from dataclasses import dataclass
+    from typing import Optional
+    from microllm_rocm_amd.cache import Binding, CacheNeed
+
+    @dataclass(frozen=True)
+    class LatentNeed(CacheNeed):
+        width: int
+        window: Optional[int] = None
+        paged = True
+
+        def bytes_per_position(self, dtype):
+            return 2 * self.width
+
+        def bind(self, group, storage, owned):
+            return LatentBinding(self, owned, group)
+
+    @dataclass
+    class LatentBinding(Binding):
+        group: int = 0
+
+    latent, windowed = LatentNeed(24), LatentNeed(24, window=20)
+    cache = CacheManager([latent, FULL, windowed, latent, None], [None, None, None, None, 0], 16, 8, 2, device=None, max_portion=8)
+    assert [type(group.need).__name__ for group in cache.groups] == ["LatentNeed", "PagedKVNeed", "LatentNeed"]
+    assert cache.groups[0].entries == [0, 3] and cache.groups[2].need.window == 20
+    assert cache.groups[2].pool.num_pages == 2 * 3, "a windowed group of any payload is sized by its window"
+    bindings = cache.bindings()
+    assert isinstance(bindings[0], LatentBinding) and bindings[3].group == bindings[0].group
+    assert bindings[4].group == bindings[0].group and not bindings[4].owned
+    assert cache.bytes_per_page(cache.groups[0]) == 2 * 16 * 48 and not cache.has_state
+    request = cache.open("a")
+    cache.reserve(request, 40)
+    cache.commit(request, 40)
+    assert cache.held_pages() == [3, 3, 2], "the window has passed the first page of its group"
+    cache.close("a")
+    cache.check()
+    with pytest.raises(TypeError, match="unknown cache need"):
+        CacheManager([("keys", 4)], [None], 16, 8, 2, device=None)
+
+
 def test_exact_byte_accounting():
     # the style of tests/inference/scheduler_test.cpp:419-422: bytes are an exact formula of the sizes
     cache = manager(needs=(FULL, FULL, WINDOW), num_pages=8)

@@ -120,7 +120,7 @@ def test_every_replay_of_a_decode_graph_equals_the_eager_step(tmp_path, dtype):
     # most replays found their metadata built while the step before ran (not the first of a graph, not those at a
     # page's edge or after another kind of step), and none took what was built for other requests
     assert replays // 2 < graphs.steps_built_ahead < replays
-    assert len(graphs._graphs) >= 2, "more than one graph was captured (two and three requests)"
+    assert graphs.kept_graphs >= 2, "more than one graph was captured (two and three requests)"
     for engine in (graphs, eager):
         engine.cache.check()
 
@@ -493,3 +493,41 @@ def test_mixed_steps_replayed_from_graphs_equal_eager_steps(tmp_path, dtype, whi
     assert graphs.mixed_graph_replays >= 15 and eager.graph_replays == 0
     pool = graphs.cache.groups[0].pool
     assert pool.total_taken > pool.num_pages, "pages were used again"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_step_copies_its_metadata_once_and_nothing_back(tmp_path, dtype):
+    """The copies between host and device that the engine makes are counted: a step moves one packed buffer of
+    metadata to the device and nothing to the host (a decode step from a graph: its tokens, and the next step's
+    metadata built ahead); selecting tokens moves the chosen ids back, one copy a step. The reference holds a
+    forward to no copy to the host the same way (tests/inference/hip_shape_matrix_test.cpp:101-136)."""
+    from microllm_rocm_amd import GenerationConfig, generate
+    from microllm_rocm_amd.engine import StepEntry
+    from microllm_rocm_amd.ops.transfers import reset_transfer_stats, transfer_stats
+    folder = make_folder(tmp_path, "B", SHARP)
+    config = CONFIGS["B"]
+    engine = engine_for(folder, dtype)
+    prompts = {name: random_tokens(60 + index, length, config.vocab_size) for index, (name, length) in enumerate((("a", 40), ("b", 9), ("c", 21)))}
+    for name in prompts:
+        engine.open(name)
+    reset_transfer_stats()
+    logits = engine.step([StepEntry("a", prompts["a"], [39]), StepEntry("b", prompts["b"][:5], [])])      # portions of prompts
+    moved = transfer_stats()
+    assert (moved.host_to_device_calls, moved.device_to_host_calls) == (1, 0) and 0 < moved.host_to_device_bytes < 4096
+    engine.step([StepEntry("a", [3], [0]), StepEntry("b", prompts["b"][5:], [3]), StepEntry("c", prompts["c"], [])])   # mixed
+    moved = transfer_stats()
+    assert (moved.host_to_device_calls, moved.device_to_host_calls) == (2, 0)
+    for _ in range(4):                                                                                        # single tokens
+        before = transfer_stats()
+        logits = engine.step([StepEntry(name, [5], [0]) for name in prompts], borrow_logits=True)
+        moved = transfer_stats()
+        assert moved.device_to_host_calls == 0 and 1 <= moved.host_to_device_calls - before.host_to_device_calls <= 2
+    assert engine.graph_replays == 4 and engine.steps_built_ahead >= 2
+    torch.cuda.synchronize()
+    assert torch.isfinite(logits).all()
+    for name in prompts:
+        engine.close(name)
+    reset_transfer_stats()
+    generate(engine, [prompts["b"]], GenerationConfig(max_new_tokens=6, temperature=0.0))
+    moved = transfer_stats()
+    assert moved.device_to_host_calls == 6 and moved.device_to_host_bytes == 6 * 4, "the chosen id of every step, nothing else"

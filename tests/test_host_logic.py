@@ -124,3 +124,62 @@ def test_percentile_interpolates_between_the_two_nearest_sorted_values():
     assert percentile([1, 2, 3, 4, 5], 0.95) == pytest.approx(4.8) and percentile([5, 1], 0.0) == 1 and percentile([5, 1], 1.0) == 5
     with pytest.raises(ValueError):
         percentile([], 0.5)
+
+
+def test_padding_a_step_to_a_graph_shape_never_changes_the_kernel_a_product_takes():
+    """A mixed step is padded to fixed numbers of token rows and of wanted rows before it is replayed from a graph;
+    the padded count must take the same product as the real one, for every kind of weight, or the replayed step
+    would give other bits than the same step run eagerly."""
+    from microllm_rocm_amd.engine.engine import MAX_GRAPH_TOKENS, MAX_GRAPH_WANTED, _token_rows, _wanted_rows
+    narrow = Weight(torch.zeros((64, 32), dtype=torch.bfloat16), pack=False)
+    narrow.packed = torch.zeros((4, 1, 4, 16, 8), dtype=torch.bfloat16)
+    wide = Weight(torch.zeros((16, 8), dtype=torch.bfloat16), pack=False)
+    wide.packed, wide.out_features = narrow.packed, 2048 * 16
+
+    def kernel_of(weight, rows, gated):
+        return (rows <= SKINNY_ROWS, takes_unscaled(weight, rows), takes_packed(weight, rows, gated), rows <= MEDIUM_ROWS)
+
+    for pad, most in ((_token_rows, MAX_GRAPH_TOKENS), (_wanted_rows, MAX_GRAPH_WANTED)):
+        for rows in range(1, most + 1):
+            padded = pad(rows)
+            assert rows <= padded <= max(16, 2 * rows)
+            for weight in (narrow, wide):
+                for gated in (False, True):
+                    assert kernel_of(weight, rows, gated) == kernel_of(weight, padded, gated), (pad.__name__, rows, padded)
+
+
+def test_kept_graphs_stay_bounded_and_mixed_shapes_never_push_decode_graphs_out():
+    """More recurring shapes than the budget holds: captures stay bounded (a shape that was captured and evicted
+    twice runs eagerly from then on), decode graphs are not evicted by mixed ones, and both budgets hold in bytes."""
+    from types import SimpleNamespace
+    from microllm_rocm_amd.engine.graphs import MAX_CAPTURES_A_SHAPE, GraphPolicy
+    policy = GraphPolicy(decode_graphs=4, mixed_graphs=3, most_bytes=1000, seen_before_capture=2)
+    captures = 0
+    for key in range(4):                                   # four decode shapes, captured once each
+        policy.decode.put(("decode", key), SimpleNamespace(held_bytes=100))
+    assert len(policy.decode) == 4
+    shapes = [("mixed", index) for index in range(10)]      # ten mixed shapes that keep coming round
+    for round_number in range(40):
+        for key in shapes:
+            if not policy.wants_mixed(key):
+                continue
+            if policy.mixed.get(key) is None:
+                state = SimpleNamespace(held_bytes=0)
+                policy.mixed.put(key, state, policy.evicted_mixed)
+                state.held_bytes = 100                      # the capture
+                captures += 1
+                policy.captured_mixed(key)
+                policy.mixed.trim(policy.evicted_mixed, keep=key)
+            assert len(policy.mixed) <= 3 and policy.mixed.held_bytes() <= 500
+    assert captures <= MAX_CAPTURES_A_SHAPE * len(shapes), "no shape is captured over and over"
+    assert len(policy.decode) == 4 and all(("decode", key) in policy.decode for key in range(4))
+    assert all(not policy.wants_mixed(key) or key in policy.mixed for key in shapes), "evicted twice: eagerly for good"
+    # a shape seen once is not captured; the second time it is
+    fresh = GraphPolicy(seen_before_capture=2)
+    assert not fresh.wants_mixed("s") and fresh.wants_mixed("s")
+    # the budget in bytes: a graph of large logits pushes older ones out, the one in use stays
+    small = GraphPolicy(decode_graphs=8, mixed_graphs=8, most_bytes=600)
+    for key in range(3):
+        small.decode.put(key, SimpleNamespace(held_bytes=100))
+    small.decode.put("large", SimpleNamespace(held_bytes=250))
+    assert "large" in small.decode and small.decode.held_bytes() <= 300 and 0 not in small.decode

@@ -313,7 +313,8 @@ def test_position_embedding_and_head_parts_alone():
     embedding.bind(tensors)
     head.bind(tensors)
     ids = torch.tensor([3, 330, 0], dtype=torch.int32, device=DEVICE)
-    rows = embedding.forward(ids)
+    from types import SimpleNamespace
+    rows = embedding.forward(SimpleNamespace(tokens=ids))       # an embedding part is handed the step
     assert rows.dtype == torch.float32 and torch.equal(rows.cpu(), table[[3, 330, 0]].float())
     x = bf16_exact(rng.normal(size=(5, 72)))
     logits = head.forward(x.to(DEVICE))

@@ -31,11 +31,19 @@ def both(lib, logits):
     got = torch.full((rows,), -7, dtype=torch.int32, device=DEVICE)
     expected = torch.full((rows,), -7, dtype=torch.int32, device=DEVICE)
     parts = torch.empty((rows, lib.mll_argmax_slices(vocab), 4), dtype=torch.int32, device=DEVICE)
-    torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # The first call on a GPU asks for the static array's address; from then on a call must leave the device's
+    # free memory as it found it. ``mem_get_info`` is the driver's own count, so it also sees what a library
+    # would take or give back behind torch's allocator (which ``memory_allocated`` does not).
     status = lib.mll_argmax_static(logits.data_ptr(), got.data_ptr(), rows, vocab, stream)
     assert status == 0, lib.mll_last_error().decode()
-    assert torch.cuda.memory_allocated() == before
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    allocated_before = torch.cuda.memory_allocated()
+    got.fill_(-7)
+    status = lib.mll_argmax_static(logits.data_ptr(), got.data_ptr(), rows, vocab, stream)
+    assert status == 0, lib.mll_last_error().decode()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before and torch.cuda.memory_allocated() == allocated_before
     status = lib.mll_argmax(logits.data_ptr(), expected.data_ptr(), parts.data_ptr(), rows, vocab, stream)
     assert status == 0, lib.mll_last_error().decode()
     torch.cuda.synchronize()
