@@ -1,66 +1,119 @@
-// The float32 matrix product of the true 32-bit path: C = A * W^T (+ bias), 64x64 tiles staged
-// through LDS, a 4x4 block of outputs per thread. Every output element is summed by one thread
-// in ascending k, so a row's result is the same whatever other rows the call holds.
+// The float32 matrix product of the true 32-bit path: C = A * W^T (+ bias), tiles staged through LDS.
+// Every output element is summed by one thread in ascending k, so a row's result is the same whatever
+// other rows the call holds and whichever of the kernels here computes it.
 #include "common.h"
 #include "microllm_hip.h"
 
 namespace mll {
 
-constexpr int kTile = 64;
-constexpr int kDepth = 16;
+// The reduction may be cut into parts of k_split terms, one a blockIdx.z: part z sums k in [z * k_split, (z + 1) *
+// k_split) in ascending order into C[z] (its own [m, n] array), the bias goes to part 0, and whoever reads the result
+// adds the parts in order. The cut depends on the weight's shape alone (mll_gemm_f32_splits), never on the rows of the
+// call, so a row's bits stay what they are under every batch. Inside a kernel `k` then is the part's end, and sums
+// start at k_lo.
+#define MLL_F32_SPLIT_RANGE                                                          \
+    const int ld = k; /* elements from one row of A or W to the next */              \
+    const int k_lo = blockIdx.z * k_split;                                           \
+    k = min(k, k_lo + k_split);                                                      \
+    c += static_cast<int64_t>(blockIdx.z) * m * n;                                   \
+    if (blockIdx.z != 0) bias = nullptr;
 
-__global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__ a, const float* __restrict__ w,
-                                                       const float* __restrict__ bias, float* __restrict__ c,
-                                                       int m, int n, int k) {
-    __shared__ float a_tile[kDepth][kTile + 4];
-    __shared__ float w_tile[kDepth][kTile + 4];
-    const int row0 = blockIdx.y * kTile;
-    const int col0 = blockIdx.x * kTile;
-    const int tx = threadIdx.x % 16;  // 4 output columns each
-    const int ty = threadIdx.x / 16;  // 4 output rows each
-    const int load_row = threadIdx.x / 4;        // 0..63
-    const int load_k = (threadIdx.x % 4) * 4;    // 0,4,8,12
-
-    float acc[4][4];
+// Tiles for more than 16 rows. A workgroup of THREADS threads takes (THREADS / 16) * TR rows and 16 * TC columns of
+// C; a thread TR x TC elements (rows r + (THREADS / 16) * i, columns c + 16 * j), each summed by that thread alone in
+// ascending k with one fused multiply-add a term: the bits of the kernels for few rows below. Both operands come in
+// chunks of DEPTH of k with 16-byte loads of whole rows (the next chunk is on its way while this one is summed) and lie
+// in LDS as [row][k] with rows four banks apart, so that a thread's four consecutive k are one read and the rows a
+// wave reads at one k fall on different banks. Two shapes are used: 64 x 64 with 4 x 4 elements a thread (one read
+// from LDS for eight multiply-adds) wherever that gives the GPU enough workgroups (prompts; weights of many rows), and
+// 16 x 32 with 2 x 2 (one for four) where C is small: 64 rows of a weight of 3584 are 224 tiles of 64 x 64 but 896
+// of 16 x 32.
+template <int THREADS, int TR, int TC, int DEPTH, bool VECTOR>
+__global__ __launch_bounds__(THREADS) void gemm_f32_tile_kernel(const float* __restrict__ a, const float* __restrict__ w,
+                                                                const float* __restrict__ bias, float* __restrict__ c,
+                                                                int m, int n, int k, int k_split) {
+    MLL_F32_SPLIT_RANGE
+    constexpr int ROW_STEP = THREADS / 16;
+    constexpr int ROWS = ROW_STEP * TR;
+    constexpr int COLUMNS = 16 * TC;
+    constexpr int QUADS = DEPTH / 4;                       // float4 in a row of a chunk
+    constexpr int LOADS_A = ROWS * QUADS / THREADS;
+    constexpr int LOADS_W = COLUMNS * QUADS / THREADS;
+    static_assert(ROWS * QUADS % THREADS == 0 && COLUMNS * QUADS % THREADS == 0, "a chunk is dealt evenly to the threads");
+    __shared__ __align__(16) float a_tile[ROWS][DEPTH + 4];
+    __shared__ __align__(16) float w_tile[COLUMNS][DEPTH + 4];
+    const int row0 = blockIdx.y * ROWS;
+    const int col0 = blockIdx.x * COLUMNS;
+    const int column = threadIdx.x % 16;
+    const int row = threadIdx.x / 16;
+    auto load4 = [&](const float* matrix, int rows, int first_row, int index, int k0) {
+        const int r = index / QUADS, kk = k0 + (index % QUADS) * 4;
+        const bool live = first_row + r < rows;
+        const float* source = matrix + static_cast<int64_t>(live ? first_row + r : 0) * ld + kk;
+        if (VECTOR) return (live && kk < k) ? *reinterpret_cast<const float4*>(source) : make_float4(0.f, 0.f, 0.f, 0.f);
+        float v[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+        for (int e = 0; e < 4; ++e) v[e] = (live && kk + e < k) ? source[e] : 0.0f;
+        return make_float4(v[0], v[1], v[2], v[3]);
+    };
+    float4 a_next[LOADS_A], w_next[LOADS_W];
+    auto fetch = [&](int k0) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = 0.0f;
-
-    for (int k0 = 0; k0 < k; k0 += kDepth) {
+        for (int j = 0; j < LOADS_A; ++j) a_next[j] = load4(a, m, row0, threadIdx.x + j * THREADS, k0);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int kk = k0 + load_k + e;
-            const int ar = row0 + load_row;
-            const int wr = col0 + load_row;
-            a_tile[load_k + e][load_row] = (ar < m && kk < k) ? a[static_cast<int64_t>(ar) * k + kk] : 0.0f;
-            w_tile[load_k + e][load_row] = (wr < n && kk < k) ? w[static_cast<int64_t>(wr) * k + kk] : 0.0f;
+        for (int j = 0; j < LOADS_W; ++j) w_next[j] = load4(w, n, col0, threadIdx.x + j * THREADS, k0);
+    };
+    float acc[TR][TC];
+#pragma unroll
+    for (int i = 0; i < TR; ++i)
+#pragma unroll
+        for (int j = 0; j < TC; ++j) acc[i][j] = 0.0f;
+    fetch(k_lo);
+    for (int k0 = k_lo; k0 < k; k0 += DEPTH) {
+#pragma unroll
+        for (int j = 0; j < LOADS_A; ++j) {
+            const int index = threadIdx.x + j * THREADS;
+            *reinterpret_cast<float4*>(&a_tile[index / QUADS][(index % QUADS) * 4]) = a_next[j];
+        }
+#pragma unroll
+        for (int j = 0; j < LOADS_W; ++j) {
+            const int index = threadIdx.x + j * THREADS;
+            *reinterpret_cast<float4*>(&w_tile[index / QUADS][(index % QUADS) * 4]) = w_next[j];
         }
         __syncthreads();
+        if (k0 + DEPTH < k) fetch(k0 + DEPTH);
 #pragma unroll
-        for (int kk = 0; kk < kDepth; ++kk) {
-            float av[4], wv[4];
+        for (int kk = 0; kk < DEPTH; kk += 4) {
+            float4 av[TR], wv[TC];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) av[i] = a_tile[kk][ty * 4 + i];
+            for (int i = 0; i < TR; ++i) av[i] = *reinterpret_cast<const float4*>(&a_tile[row + ROW_STEP * i][kk]);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) wv[j] = w_tile[kk][tx * 4 + j];
+            for (int j = 0; j < TC; ++j) wv[j] = *reinterpret_cast<const float4*>(&w_tile[column + 16 * j][kk]);
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < TR; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+                for (int j = 0; j < TC; ++j) acc[i][j] = fmaf(av[i].x, wv[j].x, acc[i][j]);
+#pragma unroll
+            for (int i = 0; i < TR; ++i)
+#pragma unroll
+                for (int j = 0; j < TC; ++j) acc[i][j] = fmaf(av[i].y, wv[j].y, acc[i][j]);
+#pragma unroll
+            for (int i = 0; i < TR; ++i)
+#pragma unroll
+                for (int j = 0; j < TC; ++j) acc[i][j] = fmaf(av[i].z, wv[j].z, acc[i][j]);
+#pragma unroll
+            for (int i = 0; i < TR; ++i)
+#pragma unroll
+                for (int j = 0; j < TC; ++j) acc[i][j] = fmaf(av[i].w, wv[j].w, acc[i][j]);
         }
         __syncthreads();
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int row = row0 + ty * 4 + i;
-        if (row >= m) continue;
+    for (int i = 0; i < TR; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int col = col0 + tx * 4 + j;
-            if (col < n) c[static_cast<int64_t>(row) * n + col] = acc[i][j] + (bias ? bias[col] : 0.0f);
+        for (int j = 0; j < TC; ++j) {
+            const int r = row0 + row + ROW_STEP * i, col = col0 + column + 16 * j;
+            if (r < m && col < n) c[static_cast<int64_t>(r) * n + col] = acc[i][j] + (bias ? bias[col] : 0.0f);
         }
-    }
 }
 
 // The same product for at most 16 rows (decoding): a workgroup takes 16 columns of C, so that a weight of a few
@@ -76,7 +129,8 @@ constexpr int kSmallParts = kSmallDepth / 64;
 template <bool VECTOR>
 __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float* __restrict__ a, const float* __restrict__ w,
                                                              const float* __restrict__ bias, float* __restrict__ c,
-                                                             int m, int n, int k) {
+                                                             int m, int n, int k, int k_split) {
+    MLL_F32_SPLIT_RANGE
     // Rows of kSmallDepth + 4 floats: 16-byte aligned, so that four consecutive k are one read, and four banks on
     // from row to row, so that the 16 rows (or columns) that a wave reads at one k fall on different banks.
     __shared__ __align__(16) float a_tile[16][kSmallDepth + 4];
@@ -89,8 +143,8 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float* __rest
     const int load_row = threadIdx.x / 16;
     const int load_k = (threadIdx.x % 16) * 4;
     const bool a_live = load_row < m, w_live = col0 + load_row < n;
-    const float* a_row = a + static_cast<int64_t>(a_live ? load_row : 0) * k;
-    const float* w_row = w + static_cast<int64_t>(w_live ? col0 + load_row : 0) * k;
+    const float* a_row = a + static_cast<int64_t>(a_live ? load_row : 0) * ld;
+    const float* w_row = w + static_cast<int64_t>(w_live ? col0 + load_row : 0) * ld;
     float4 a_next[kSmallParts], w_next[kSmallParts];
     auto fetch = [&](int k0) {
 #pragma unroll
@@ -112,8 +166,8 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float* __rest
         }
     };
     float acc = 0.0f;
-    fetch(0);
-    for (int k0 = 0; k0 < k; k0 += kSmallDepth) {
+    fetch(k_lo);
+    for (int k0 = k_lo; k0 < k; k0 += kSmallDepth) {
 #pragma unroll
         for (int part = 0; part < kSmallParts; ++part) {
             const int at = 64 * part + load_k;
@@ -157,7 +211,8 @@ constexpr int kWideFrom = 16384;                     // columns of C from which 
 template <bool VECTOR>
 __global__ __launch_bounds__(kWideThreads) void gemm_f32_small_wide_kernel(const float* __restrict__ a, const float* __restrict__ w,
                                                                            const float* __restrict__ bias, float* __restrict__ c,
-                                                                           int m, int n, int k) {
+                                                                           int m, int n, int k, int k_split) {
+    MLL_F32_SPLIT_RANGE
     __shared__ __align__(16) float a_tile[16][kWideDepth + 4];
     __shared__ __align__(16) float w_tile[kWideColumns][kWideDepth + 4];
     const int col0 = blockIdx.x * kWideColumns;
@@ -168,7 +223,7 @@ __global__ __launch_bounds__(kWideThreads) void gemm_f32_small_wide_kernel(const
     auto load4 = [&](const float* matrix, int rows, int first_row, int index, int k0) {
         const int r = index / kWideQuads, kk = k0 + (index % kWideQuads) * 4;
         const bool live = first_row + r < rows;
-        const float* source = matrix + static_cast<int64_t>(live ? first_row + r : 0) * k + kk;
+        const float* source = matrix + static_cast<int64_t>(live ? first_row + r : 0) * ld + kk;
         if (VECTOR) return (live && kk < k) ? *reinterpret_cast<const float4*>(source) : make_float4(0.f, 0.f, 0.f, 0.f);
         float v[4];
 #pragma unroll
@@ -183,8 +238,8 @@ __global__ __launch_bounds__(kWideThreads) void gemm_f32_small_wide_kernel(const
         for (int j = 0; j < kWideLoadsW; ++j) w_next[j] = load4(w, n, col0, threadIdx.x + j * kWideThreads, k0);
     };
     float acc[2][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}};
-    fetch(0);
-    for (int k0 = 0; k0 < k; k0 += kWideDepth) {
+    fetch(k_lo);
+    for (int k0 = k_lo; k0 < k; k0 += kWideDepth) {
 #pragma unroll
         for (int j = 0; j < kWideLoadsA; ++j) {
             const int index = threadIdx.x + j * kWideThreads;
@@ -228,25 +283,55 @@ __global__ __launch_bounds__(kWideThreads) void gemm_f32_small_wide_kernel(const
 
 using namespace mll;
 
+// Into how many parts the reduction over k is cut for a weight [n, k]: a function of the weight's shape alone. A
+// weight with few rows of its own (q/k/v, o, down) gives the GPU too few tiles of C; its parts go to workgroups of
+// their own. Parts are at least 512 terms long and at most 8.
+extern "C" int mll_gemm_f32_splits(int n, int k) {
+    if (n >= kWideFrom) return 1;
+    int splits = 1;
+    while (splits < 8 && (n / kSmallColumns) * splits < 1024 && k / (2 * splits) >= 512) splits *= 2;
+    return splits;
+}
+
+// C[splits][m][n]; splits is 1 or mll_gemm_f32_splits(n, k).
 extern "C" int mll_gemm_f32(const float* a, const float* w, const float* bias, float* c,
-                            int m, int n, int k, hipStream_t stream) {
+                            int m, int n, int k, int splits, hipStream_t stream) {
     MLL_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm_f32: sizes must be positive");
+    MLL_REQUIRE(splits == 1 || splits == mll_gemm_f32_splits(n, k), "gemm_f32: the reduction is cut as mll_gemm_f32_splits says, or not at all");
     if (m == 0) return 0;
+    const int k_split = splits == 1 ? k : ((k + splits - 1) / splits + 3) / 4 * 4;
+    MLL_REQUIRE(static_cast<int64_t>(k_split) * (splits - 1) < k, "gemm_f32: a part of the reduction would be empty");
+    const unsigned parts = static_cast<unsigned>(splits);
+    const bool vector = k % 4 == 0 && reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
     if (m <= 16) {
-        const bool vector = k % 4 == 0 && reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
         if (n >= kWideFrom) {
-            const int groups = (n + kWideColumns - 1) / kWideColumns;
-            if (vector) gemm_f32_small_wide_kernel<true><<<groups, kWideThreads, 0, stream>>>(a, w, bias, c, m, n, k);
-            else gemm_f32_small_wide_kernel<false><<<groups, kWideThreads, 0, stream>>>(a, w, bias, c, m, n, k);
+            const dim3 grid((n + kWideColumns - 1) / kWideColumns, 1, parts);
+            if (vector) gemm_f32_small_wide_kernel<true><<<grid, kWideThreads, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
+            else gemm_f32_small_wide_kernel<false><<<grid, kWideThreads, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
             return check_launch("gemm_f32");
         }
-        const int groups = (n + kSmallColumns - 1) / kSmallColumns;
-        if (vector) gemm_f32_small_kernel<true><<<groups, 256, 0, stream>>>(a, w, bias, c, m, n, k);
-        else gemm_f32_small_kernel<false><<<groups, 256, 0, stream>>>(a, w, bias, c, m, n, k);
+        const dim3 grid((n + kSmallColumns - 1) / kSmallColumns, 1, parts);
+        if (vector) gemm_f32_small_kernel<true><<<grid, 256, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
+        else gemm_f32_small_kernel<false><<<grid, 256, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
         return check_launch("gemm_f32");
     }
-    const dim3 grid((n + kTile - 1) / kTile, (m + kTile - 1) / kTile);
-    MLL_REQUIRE(grid.y <= 65535, "gemm_f32: too many rows for one call");
-    gemm_f32_kernel<<<grid, 256, 0, stream>>>(a, w, bias, c, m, n, k);
+    // Tiles of 64 x 64 wherever they are enough workgroups for the GPU; for at most 32 rows of a weight with many rows
+    // tiles of 32 x 64 (the same 4 x 4 elements a thread: the head at 17 to 32 rows 940 -> 640 us); else tiles of 16 x 32.
+    const int64_t column_tiles = (n + 63) / 64;
+    if (m > 32 && column_tiles * ((m + 63) / 64) * splits >= 384) {
+        const dim3 grid(column_tiles, (m + 63) / 64, parts);
+        MLL_REQUIRE(grid.y <= 65535, "gemm_f32: too many rows for one call");
+        if (vector) gemm_f32_tile_kernel<256, 4, 4, 32, true><<<grid, 256, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
+        else gemm_f32_tile_kernel<256, 4, 4, 32, false><<<grid, 256, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
+    } else if (m <= 32 && n >= kWideFrom) {
+        const dim3 grid(column_tiles, (m + 31) / 32, parts);
+        if (vector) gemm_f32_tile_kernel<128, 4, 4, 32, true><<<grid, 128, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
+        else gemm_f32_tile_kernel<128, 4, 4, 32, false><<<grid, 128, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
+    } else {
+        const dim3 grid((n + 31) / 32, (m + 15) / 16, parts);
+        MLL_REQUIRE(grid.y <= 65535, "gemm_f32: too many rows for one call");
+        if (vector) gemm_f32_tile_kernel<128, 2, 2, 128, true><<<grid, 128, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
+        else gemm_f32_tile_kernel<128, 2, 2, 128, false><<<grid, 128, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
+    }
     return check_launch("gemm_f32");
 }

@@ -85,9 +85,12 @@ int mll_silu_mul(const void* gate, const void* up, int64_t in_stride, void* out,
                  int n_tokens, int width, hipStream_t stream);
 
 // C[m, n] = sum_k A[m, k] * W[n, k] (+ bias[n]), all float32, k summed in ascending order by one
-// thread per output element, so a row's result does not depend on the other rows.
+// thread per output element, so a row's result does not depend on the other rows. With splits > 1
+// (only the number mll_gemm_f32_splits gives for the weight's shape) C is [splits, m, n]: sums over
+// consecutive ranges of k, the bias in the first, for the reader to add in order.
+int mll_gemm_f32_splits(int n, int k);
 int mll_gemm_f32(const float* a, const float* w, const float* bias, float* c,
-                 int m, int n, int k, hipStream_t stream);
+                 int m, int n, int k, int splits, hipStream_t stream);
 
 // C = A . W^T for bfloat16 A [m <= 64, k] and a weight packed as [n/16][k/32][4][16][8] (zero padded):
 // element (row, col) of W sits at piece (row / 16, col / 32), position ((col % 32) / 8, row % 16, col % 8).

@@ -392,9 +392,17 @@ def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
     return out
 
 
+def f32_splits(n: int, k: int) -> int:
+    """Into how many parts ``gemm_f32`` may cut the reduction of a weight ``[n, k]``: the weight's shape decides,
+    never the rows of a call, so that a row's bits are the same in every batch."""
+    return int(library.load().mll_gemm_f32_splits(int(n), int(k)))
+
+
 def gemm_f32(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-             out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``a @ weight.T (+ bias)`` in true float32 with a fixed order of additions per element."""
+             out: Optional[torch.Tensor] = None, partials: bool = False) -> torch.Tensor:
+    """``a @ weight.T (+ bias)`` in true float32 with a fixed order of additions per element. With ``partials``
+    the result may come as ``[parts, m, n]`` (``f32_splits`` parts): sums over consecutive ranges of k, which the
+    caller adds in order."""
     lib = library.load()
     _device_tensor(a, "gemm input", torch.float32)
     _device_tensor(weight, "gemm weight", torch.float32)
@@ -405,15 +413,17 @@ def gemm_f32(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]
     if bias is not None:
         _device_tensor(bias, "gemm bias", torch.float32)
         _need(tuple(bias.shape) == (n,), "gemm bias has the wrong size")
+    step = 65535 * 16
+    splits = f32_splits(n, k) if partials and m <= step else 1
+    shape = (m, n) if splits == 1 else (splits, m, n)
     if out is None:
-        out = torch.empty((m, n), dtype=torch.float32, device=a.device)
+        out = torch.empty(shape, dtype=torch.float32, device=a.device)
     _device_tensor(out, "gemm output", torch.float32)
-    _need(tuple(out.shape) == (m, n), "gemm output has the wrong shape")
-    step = 65535 * 64
+    _need(tuple(out.shape) == shape, "gemm output has the wrong shape")
     for start in range(0, max(m, 1), step):
         count = min(step, m - start)
         _check(lib.mll_gemm_f32(ctypes.c_void_p(a.data_ptr() + start * k * 4), _ptr(weight), _ptr(bias),
-                                ctypes.c_void_p(out.data_ptr() + start * n * 4), count, n, k, _stream()), lib)
+                                ctypes.c_void_p(out.data_ptr() + start * n * 4), count, n, k, splits, _stream()), lib)
     return out
 
 

@@ -121,7 +121,7 @@ def linear(x: Union[torch.Tensor, UnscaledRows], weight, out_dtype: Optional[tor
     if weight.dtype == torch.float32:
         # True 32-bit product, also for a 32-bit weight inside a bfloat16 engine.
         a = x if x.dtype == torch.float32 else x.to(torch.float32)
-        y = kernels.gemm_f32(a, w)
+        y = kernels.gemm_f32(a, w, partials=partials and not gated and out_dtype == torch.float32)
         if gated:
             return kernels.silu_mul(y if x.dtype == torch.float32 else y.to(x.dtype))
         return y if out_dtype == torch.float32 else y.to(out_dtype)
