@@ -82,6 +82,9 @@ def main() -> int:
                              "portions of 512 (--steps whole runs timed after --warmup untimed ones); meant for --size 0.5b")
     parser.add_argument("--serve-requests", type=int, default=64)
     parser.add_argument("--no-mixed-graphs", action="store_true", help="run steps that mix portions and single tokens eagerly")
+    parser.add_argument("--no-extras", action="store_true",
+                        help="leave out what the default run adds to its line after the main figures: decoding on the 32-bit path "
+                             "at batch 8 and the continuous-batching workload at Qwen2-0.5B sizes")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
@@ -147,7 +150,10 @@ def main() -> int:
         flops = step_flops(engine, args.prefill_tokens)
         line["prefill"] = {"value": round(prefill["tokens_per_second"], 1), "tokens": args.prefill_tokens,
                            "ms": round(prefill["ms"], 3),
-                           "frac": round(flops / (prefill["ms"] * 1e-3) / peak_flops, 4)}
+                           "frac": round(flops / (prefill["ms"] * 1e-3) / peak_flops, 4),
+                           "runs": "best of 3 (value, ms, frac); their mean beside it",
+                           "mean_ms": round(prefill["mean_ms"], 3), "mean_value": round(prefill["mean_tokens_per_second"], 1),
+                           "mean_frac": round(flops / (prefill["mean_ms"] * 1e-3) / peak_flops, 4), "all_ms": prefill["all_ms"]}
     if not args.no_calibration and args.dtype == "bfloat16":
         # What kernels that do nothing but read memory, or nothing but bfloat16 MFMAs, reach on this GPU: the
         # fractions of these stand beside the fractions of the published peaks.
@@ -157,6 +163,37 @@ def main() -> int:
         line["roofline"]["frac_of_measured"] = round(achieved / measured["hbm_read_GBps"], 4)
         if "prefill" in line:
             line["prefill"]["frac_of_measured"] = round(flops / (prefill["ms"] * 1e-3) / (measured["mfma_bf16_TFLOPs"] * 1e12), 4)
+    extras = not args.no_extras and args.size == "7b" and args.dtype == "bfloat16" and args.layers == full_layers
+    if extras:
+        # Two more figures of the same program on the same GPU, each on an engine of its own after the main one is
+        # gone: decoding on the true 32-bit path, and the continuous-batching workload at the smallest model's sizes.
+        del engine
+        torch.cuda.empty_cache()
+        exact = Engine.from_random(config, seed=0, dtype="float32", device="cuda:0", on_device=True, page_size=page_size,
+                                   max_tokens=8 * (args.context + 8 + 2 * page_size), max_requests=8)
+        fp32 = decode_throughput(exact, 8, args.context, steps=5, warmup=1, seed=8)
+        fp32_bytes = step_bytes(exact, 8, args.context + 3)
+        line["points"]["fp32_decode_b8"] = round(fp32["tokens_per_second"], 2)
+        line["fp32"] = {"config": "the same model and context on the true 32-bit path, batch 8, 5 steps after 1", "dtype": "fp32",
+                        "value": round(fp32["tokens_per_second"], 2), "ms_per_step": round(fp32["ms_per_step"], 3),
+                        "roofline_frac": round(fp32_bytes / (fp32["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+        del exact
+        torch.cuda.empty_cache()
+        from microllm_rocm_amd.engine.benchmark import serving_throughput
+        small_sizes = dict(SIZES["0.5b"])
+        small = Qwen2Config(max_position_embeddings=32768, rope_theta=1e6, rms_norm_eps=1e-6, **small_sizes)
+        requests, longest, new_tokens, chunk, budget = 64, 2048, 256, 512, 2048
+        server = Engine.from_random(small, seed=0, dtype="bfloat16", device="cuda:0", on_device=True, page_size=page_size,
+                                    max_tokens=requests * (-(-(longest + new_tokens) // page_size) + 1) * page_size,
+                                    max_requests=requests, max_portion=chunk)
+        served = serving_throughput(server, requests=requests, prompt_range=(128, longest), new_tokens=new_tokens,
+                                    prefill_chunk=chunk, max_batched_tokens=budget, runs=3, warmup=1)
+        line["serve"] = {"config": "Qwen2-0.5B size, bf16, 64 requests, prompts uniform 128..2048, 256 new tokens each, "
+                                   "portions of 512, 2048 tokens a step, 3 runs after 1",
+                         "value": round(served["tokens_per_second"], 1), "unit": "generated tok/s",
+                         "ttft_p50_ms": round(served["ttft_p50_ms"], 1), "ttft_p95_ms": round(served["ttft_p95_ms"], 1),
+                         "completion_p95_ms": round(served["completion_p95_ms"], 1), "preemptions": served["preemptions"],
+                         "scheduler_steps": served["scheduler_steps"]}
     print(json.dumps(line), flush=True)
     return 0
 

@@ -318,7 +318,12 @@ extern "C" int mll_gemm_f32(const float* a, const float* w, const float* bias, f
     // Tiles of 64 x 64 wherever they are enough workgroups for the GPU; for at most 32 rows of a weight with many rows
     // tiles of 32 x 64 (the same 4 x 4 elements a thread: the head at 17 to 32 rows 940 -> 640 us); else tiles of 16 x 32.
     const int64_t column_tiles = (n + 63) / 64;
-    if (m > 32 && column_tiles * ((m + 63) / 64) * splits >= 384) {
+    if (m >= 512 && column_tiles * ((m + 127) / 128) * splits >= 512) {
+        const dim3 grid(column_tiles, (m + 127) / 128, parts);
+        MLL_REQUIRE(grid.y <= 65535, "gemm_f32: too many rows for one call");
+        if (vector) gemm_f32_tile_kernel<256, 8, 4, 32, true><<<grid, 256, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
+        else gemm_f32_tile_kernel<256, 8, 4, 32, false><<<grid, 256, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
+    } else if (m > 32 && column_tiles * ((m + 63) / 64) * splits >= 384) {
         const dim3 grid(column_tiles, (m + 63) / 64, parts);
         MLL_REQUIRE(grid.y <= 65535, "gemm_f32: too many rows for one call");
         if (vector) gemm_f32_tile_kernel<256, 4, 4, 32, true><<<grid, 256, 0, stream>>>(a, w, bias, c, m, n, k, k_split);

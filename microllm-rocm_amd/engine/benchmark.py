@@ -58,11 +58,14 @@ def decode_throughput(engine: Engine, batch: int, context: int, steps: int, warm
 
 
 def prefill_throughput(engine: Engine, tokens: int, repeats: int = 3, seed: int = 0) -> Dict[str, float]:
-    """One request's prompt of ``tokens`` ids in one step, logits at its last position; the best of ``repeats``."""
+    """One request's prompt of ``tokens`` ids in one step, logits at its last position, ``repeats`` times after
+    two runs that warm up (the library, where it is tuned, settles its choice of algorithm over the first calls of
+    a shape): the best run (``ms``, ``tokens_per_second``) and the mean of the runs (``mean_ms``)."""
     rng = np.random.default_rng(seed)
     prompt = rng.integers(0, engine.spec.vocab_size, size=tokens).tolist()
-    best = float("inf")
-    for repeat in range(repeats + 1):   # the first run warms up
+    times = []
+    warmup = 2
+    for repeat in range(repeats + warmup):
         request_id = ("prefill", repeat)
         engine.open(request_id)
         torch.cuda.synchronize()
@@ -72,9 +75,11 @@ def prefill_throughput(engine: Engine, tokens: int, repeats: int = 3, seed: int 
         elapsed = time.perf_counter() - started
         engine.close(request_id)
         assert torch.isfinite(logits).all()
-        if repeat > 0:
-            best = min(best, elapsed)
-    return {"tokens_per_second": tokens / best, "ms": best * 1e3}
+        if repeat >= warmup:
+            times.append(elapsed)
+    best, mean = min(times), sum(times) / len(times)
+    return {"tokens_per_second": tokens / best, "ms": best * 1e3, "mean_ms": mean * 1e3, "mean_tokens_per_second": tokens / mean,
+            "all_ms": [round(elapsed * 1e3, 3) for elapsed in times]}
 
 
 def weight_bytes(engine: Engine) -> int:

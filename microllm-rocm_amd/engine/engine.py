@@ -40,7 +40,7 @@ def parse_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
 MAX_GRAPH_REQUESTS = 256
 MIN_GRAPH_WIDTH = 16
 DECODE_GRAPHS = 32          # captured steps of single tokens kept at a time; the one replayed longest ago goes first
-MIXED_GRAPHS = 16           # and captured mixed steps, which have a budget of their own (engine/graphs.py)
+MIXED_GRAPHS = 48           # and captured mixed steps, which have a budget of their own (engine/graphs.py)
 GRAPH_LOGITS_BYTES = 2 << 30    # what the kept graphs' logits may hold together
 MAX_GRAPH_TOKENS = 4096     # mixed steps of more tokens run eagerly: their launches no longer cost more than their kernels
 MAX_GRAPH_WANTED = 256
@@ -259,16 +259,25 @@ class Engine:
 
     # ---- mixed steps from graphs -----------------------------------------------------------
     def _fixed_shape(self, batch: HostBatch) -> Optional[FixedShape]:
-        """The shape this step is padded to for a graph, or None if it runs eagerly: too large, or a shape that
-        has not come before (most shapes of a changing workload come once)."""
+        """The shape a mixed step is padded to, or None if it is too large for that and runs as it is. Whether
+        the padded step is then replayed from a graph or run eagerly is the policy's choice (most shapes of a
+        changing workload come once); it is padded either way, so that the kernels' choices that follow the number
+        of rows (which product, how a reduction is cut) are the same both times and a step gives the same bits
+        whether its shape happens to be captured or not."""
         step = batch.step
         wanted = int(batch.want_rows.size)
         if step.n_tokens > MAX_GRAPH_TOKENS or step.n_seqs > MAX_GRAPH_REQUESTS or wanted > MAX_GRAPH_WANTED:
             return None
-        shape = FixedShape(tokens=_token_rows(step.n_tokens), requests=_power_of_two(step.n_seqs),
-                           wanted=_wanted_rows(wanted), width=_power_of_two(batch.blocks_needed, MIN_GRAPH_WIDTH),
-                           planned={name: _power_of_two(rows) for name, rows in batch.planned_rows().items()})
-        return shape if self._policy.wants_mixed(shape.key()) else None
+        return FixedShape(tokens=_token_rows(step.n_tokens), requests=_power_of_two(step.n_seqs),
+                          wanted=_wanted_rows(wanted), width=_power_of_two(batch.blocks_needed, MIN_GRAPH_WIDTH),
+                          planned={name: _power_of_two(rows) for name, rows in batch.planned_rows().items()})
+
+    def _padded_step(self, shape: FixedShape, batch: HostBatch) -> Optional[torch.Tensor]:
+        """The step in its fixed shape, run eagerly."""
+        ctx = self._builder.upload(batch, fixed=shape)
+        logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
+        wanted = int(batch.want_rows.size)
+        return logits[:wanted] if wanted else None
 
     def _mixed_graph_step(self, shape: FixedShape, batch: HostBatch) -> Optional[torch.Tensor]:
         key = shape.key()
@@ -369,8 +378,10 @@ class Engine:
                 self._last_graph = None
                 batch = self._builder.prepare(requests, [entry.tokens for entry in entries], [entry.want for entry in entries])
                 shape = self._fixed_shape(batch) if self.use_graphs and self.graph_mixed_steps else None
-                if shape is not None:
+                if shape is not None and self._policy.wants_mixed(shape.key()):
                     logits = self._mixed_graph_step(shape, batch)
+                elif shape is not None:
+                    logits = self._padded_step(shape, batch)
                 else:
                     ctx = self._builder.upload(batch)
                     logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
