@@ -285,11 +285,11 @@ using namespace mll;
 
 // Into how many parts the reduction over k is cut for a weight [n, k]: a function of the weight's shape alone. A
 // weight with few rows of its own (q/k/v, o, down) gives the GPU too few tiles of C; its parts go to workgroups of
-// their own. Parts are at least 512 terms long and at most 8.
+// their own. Parts are at least 448 terms long and at most 8.
 extern "C" int mll_gemm_f32_splits(int n, int k) {
     if (n >= kWideFrom) return 1;
     int splits = 1;
-    while (splits < 8 && (n / kSmallColumns) * splits < 1024 && k / (2 * splits) >= 512) splits *= 2;
+    while (splits < 8 && (n / kSmallColumns) * splits < 2048 && k / (2 * splits) >= 448) splits *= 2;
     return splits;
 }
 
@@ -304,7 +304,7 @@ extern "C" int mll_gemm_f32(const float* a, const float* w, const float* bias, f
     const unsigned parts = static_cast<unsigned>(splits);
     const bool vector = k % 4 == 0 && reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
     if (m <= 16) {
-        if (n >= kWideFrom) {
+        if (n >= kWideFrom || static_cast<int64_t>((n + kWideColumns - 1) / kWideColumns) * splits >= 512) {
             const dim3 grid((n + kWideColumns - 1) / kWideColumns, 1, parts);
             if (vector) gemm_f32_small_wide_kernel<true><<<grid, kWideThreads, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
             else gemm_f32_small_wide_kernel<false><<<grid, kWideThreads, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
