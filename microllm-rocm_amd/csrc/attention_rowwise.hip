@@ -9,6 +9,8 @@
 // (steps with many rows: portions of prompts), or one wave per chunk leaves its result in a workspace and a
 // second kernel merges them (steps with few rows, whose keys would otherwise be walked by a handful of waves).
 // Sums that decide bits are written with explicit fused multiply-adds, so that both kernels round alike.
+#include <type_traits>
+
 #include "cache_layout.h"
 #include "common.h"
 #include "microllm_hip.h"
@@ -17,6 +19,10 @@ namespace mll {
 
 constexpr int kRowwiseMaxHeadDim = 512;
 constexpr int kRowwiseChunk = 128;      // keys; a multiple of the tiles of 64
+// Rows of (token, wave's heads) a step must still have when a wave takes several query heads of a kv head: 64, e.g. 16
+// requests of 4 kv heads (measured at 7B sizes and 4096 keys: 16 requests 159 -> 146 us, 64 requests 544 -> 413; 8
+// requests 89 -> 130). mll_rowwise_heads_from sets it: tests force either way with it.
+static int64_t grouped_from_rows = 64;
 
 __device__ inline void load_eight(const float* from, float (&to)[8]) {
     const float4 low = *reinterpret_cast<const float4*>(from);
@@ -209,6 +215,144 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_kernel(
     }
 }
 
+// MODE 1 for GW query heads of one kv head in one wave: a chunk's keys and values are read once and used for all of
+// them (with 7 query heads a kv head the plain kernel reads every key 7 times, and it is those reads that bound it
+// when a step has many rows of long requests). Head by head the operations and their order are those of
+// attend_chunk: the dot products in ascending dims, the tile's maximum and sum over the wave, the values in the
+// order of the keys; only what is independent of the head (addresses, loads) is done once. Writes what MODE 1 writes,
+// bit for bit. Head sizes up to 64 * DIMS <= 128.
+template <typename T, int DIMS, int GW>
+__global__ __launch_bounds__(kWave) void paged_attention_rowwise_heads_kernel(
+    const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ seq_of_token,
+    const int32_t* __restrict__ positions, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks,
+    float scale, int window, int heads, int kv_heads, int head_dim, int page_size) {
+    __shared__ float q_shared[GW][64 * DIMS];
+    __shared__ float p_shared[GW][kWave];
+    __shared__ int64_t v_shared[2][kWave];
+    const CacheLayout layout(kv_heads, page_size, head_dim);
+    const int token = blockIdx.x;
+    const int lane = threadIdx.x;
+    const int group = heads / kv_heads;
+    const int waves_of_group = group / GW;                       // GW divides the group
+    const int kv_head = blockIdx.y / waves_of_group;
+    const int first_head = kv_head * group + (blockIdx.y % waves_of_group) * GW;
+    const int seq = seq_of_token[token];
+    if (seq < 0) return;
+    const int position = positions[token];
+    const int low = window > 0 ? max(0, position - window + 1) : 0;
+    const int first_chunk = low / kRowwiseChunk, last_chunk = position / kRowwiseChunk;
+    if (first_chunk + static_cast<int>(blockIdx.z) > last_chunk) return;
+    const int32_t* table = block_table + static_cast<int64_t>(seq) * table_width;
+#pragma unroll
+    for (int g = 0; g < GW; ++g) {
+        const T* q_row = q + (static_cast<int64_t>(token) * heads + first_head + g) * head_dim;
+        for (int d = lane; d < head_dim; d += kWave) q_shared[g][d] = to_float(q_row[d]);
+    }
+    __syncthreads();
+
+    const int chunk = first_chunk + blockIdx.z;
+    const int first = max(low, chunk * kRowwiseChunk), last = min(position, chunk * kRowwiseChunk + kRowwiseChunk - 1);
+    float acc[GW][DIMS], chunk_max[GW], chunk_sum[GW];
+#pragma unroll
+    for (int g = 0; g < GW; ++g) {
+        chunk_max[g] = -INFINITY;
+        chunk_sum[g] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < DIMS; ++i) acc[g][i] = 0.0f;
+    }
+    for (int tile = (first / kWave) * kWave; tile <= last; tile += kWave) {
+        const int key = tile + lane;
+        const bool visible = key >= first && key <= last;
+        float dot[GW];
+#pragma unroll
+        for (int g = 0; g < GW; ++g) dot[g] = 0.0f;
+        int64_t v_place = 0, v_place_last = 0;
+        if (visible) {
+            const int64_t page = table[key / page_size];
+            const int offset = key % page_size;
+            const T* k_tile = k_cache + layout.k_tile(page, kv_head, offset / 16) + (offset % 16) * 8;
+            const int64_t v_tile = layout.v_tile(page, kv_head, offset / 16);
+            v_place = v_tile + ((offset % 16) / 8) * 256;
+            v_place_last = v_tile + ((offset % 16) / 8) * 128;
+            const int whole = head_dim / 8 * 8;
+            for (int d = 0; d < whole; d += 8) {
+                float k[8];
+                load_eight(k_tile + (d / 8) * 128, k);
+#pragma unroll
+                for (int g = 0; g < GW; ++g)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) dot[g] = __fmaf_rn(q_shared[g][d + i], k[i], dot[g]);
+            }
+            for (int d = whole; d < head_dim; ++d) {
+                const float k = to_float(k_tile[(d / 8) * 128 + d % 8]);
+#pragma unroll
+                for (int g = 0; g < GW; ++g) dot[g] = __fmaf_rn(q_shared[g][d], k, dot[g]);
+            }
+        }
+        float rescale[GW];
+        __syncthreads();      // the previous tile's readers are done
+#pragma unroll
+        for (int g = 0; g < GW; ++g) {
+            const float score = visible ? __fmul_rn(dot[g], scale) : -INFINITY;
+            const float new_max = fmaxf(chunk_max[g], wave_max(score));
+            const float p = visible ? expf(score - new_max) : 0.0f;
+            rescale[g] = expf(chunk_max[g] - new_max);
+            chunk_sum[g] = __fmaf_rn(chunk_sum[g], rescale[g], wave_sum(p));
+            chunk_max[g] = new_max;
+            p_shared[g][lane] = p;
+        }
+        v_shared[0][lane] = v_place;
+        v_shared[1][lane] = v_place_last;
+        __syncthreads();
+        const int begin = max(first - tile, 0);
+        const int end = min(last - tile, kWave - 1);
+#pragma unroll
+        for (int i = 0; i < DIMS; ++i) {
+            const int d = lane + i * kWave;
+            if (d < head_dim) {
+                const int of_dim = layout.v_in_tile(0, d);
+                const int64_t* places = v_shared[layout.v_in_tile(8, d) - of_dim == 256 ? 0 : 1];
+                float value[GW];
+#pragma unroll
+                for (int g = 0; g < GW; ++g) value[g] = __fmul_rn(acc[g][i], rescale[g]);
+                for (int eight = begin / 8; eight <= end / 8; ++eight) {
+                    const int from = max(begin, 8 * eight), to = min(end, 8 * eight + 7);
+                    float v[8];
+                    load_eight(v_cache + places[from] + of_dim, v);
+#pragma unroll
+                    for (int g = 0; g < GW; ++g)
+#pragma unroll
+                        for (int r = 0; r < 8; ++r)
+                            if (8 * eight + r >= from && 8 * eight + r <= to) value[g] = __fmaf_rn(p_shared[g][8 * eight + r], v[r], value[g]);
+                }
+#pragma unroll
+                for (int g = 0; g < GW; ++g) acc[g][i] = value[g];
+            }
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < GW; ++g) {
+        const int64_t slot = (static_cast<int64_t>(token) * heads + first_head + g) * max_chunks + blockIdx.z;
+#pragma unroll
+        for (int i = 0; i < DIMS; ++i) {
+            const int d = lane + i * kWave;
+            if (d < head_dim) part_o[slot * head_dim + d] = acc[g][i];
+        }
+        if (lane == 0) {
+            part_ml[slot * 2] = chunk_max[g];
+            part_ml[slot * 2 + 1] = chunk_sum[g];
+        }
+    }
+}
+
+// The most query heads of a kv head that one wave of the kernel above takes: the largest divisor of the group up to 8.
+static int heads_a_wave(int group) {
+    for (int count = group < 8 ? group : 8; count >= 2; --count)
+        if (group % count == 0) return count;
+    return 1;
+}
+
 // Merges what MODE 1 left, in the order and with the arithmetic of MODE 0. One wave per (token, head).
 template <typename T, int DIMS>
 __global__ __launch_bounds__(kWave) void paged_attention_rowwise_merge_kernel(
@@ -260,10 +404,35 @@ static int launch_rowwise_dims(const void* q, const void* k_cache, const void* v
             kv_heads, head_dim, page_size);
         return check_launch("paged_attention_rowwise");
     }
-    paged_attention_rowwise_kernel<T, 1, DIMS><<<dim3(n_tokens, heads, max_chunks), kWave, 0, stream>>>(
-        static_cast<const T*>(q), static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), block_table,
-        table_width, seq_of_token, positions, static_cast<T*>(out), part_o, part_ml, max_chunks, scale, window, heads,
-        kv_heads, head_dim, page_size);
+    // Several query heads of a kv head in one wave where the step still has rows enough for the GPU that way
+    // (float32, head sizes up to 128: the path of the 32-bit engine; 64 requests of 4096 keys at 7B sizes).
+    const int gw = (std::is_same<T, float>::value && DIMS <= 2) ? heads_a_wave(heads / kv_heads) : 1;
+    const int64_t grouped_rows = static_cast<int64_t>(n_tokens) * (heads / gw);
+    bool grouped = false;
+    if constexpr (std::is_same<T, float>::value && DIMS <= 2) {
+        if (gw >= 2 && grouped_rows >= grouped_from_rows) {
+            grouped = true;
+            const dim3 grid(n_tokens, heads / gw, max_chunks);
+#define MLL_ROWWISE_HEADS(GW)                                                                                          \
+    case GW:                                                                                                           \
+        paged_attention_rowwise_heads_kernel<T, DIMS, GW><<<grid, kWave, 0, stream>>>(                                 \
+            static_cast<const T*>(q), static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), block_table,    \
+            table_width, seq_of_token, positions, part_o, part_ml, max_chunks, scale, window, heads, kv_heads,        \
+            head_dim, page_size);                                                                                      \
+        break;
+            switch (gw) {
+                MLL_ROWWISE_HEADS(2) MLL_ROWWISE_HEADS(3) MLL_ROWWISE_HEADS(4) MLL_ROWWISE_HEADS(5)
+                MLL_ROWWISE_HEADS(6) MLL_ROWWISE_HEADS(7) MLL_ROWWISE_HEADS(8)
+                default: grouped = false;
+            }
+#undef MLL_ROWWISE_HEADS
+        }
+    }
+    if (!grouped)
+        paged_attention_rowwise_kernel<T, 1, DIMS><<<dim3(n_tokens, heads, max_chunks), kWave, 0, stream>>>(
+            static_cast<const T*>(q), static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), block_table,
+            table_width, seq_of_token, positions, static_cast<T*>(out), part_o, part_ml, max_chunks, scale, window, heads,
+            kv_heads, head_dim, page_size);
     if (const int status = check_launch("paged_attention_rowwise")) return status;
     paged_attention_rowwise_merge_kernel<T, DIMS><<<dim3(n_tokens, heads), kWave, 0, stream>>>(
         part_o, part_ml, seq_of_token, positions, static_cast<T*>(out), max_chunks, window, heads, head_dim);
@@ -290,6 +459,14 @@ static int launch_rowwise(const void* q, const void* k_cache, const void* v_cach
 using namespace mll;
 
 extern "C" int mll_paged_attention_rowwise_chunk() { return kRowwiseChunk; }
+
+// From how many rows (tokens x waves a token) on a step's chunked row-wise attention lets a wave take several query
+// heads of a kv head; returns the value before. Both ways give the same bits.
+extern "C" int64_t mll_rowwise_heads_from(int64_t rows) {
+    const int64_t before = mll::grouped_from_rows;
+    mll::grouped_from_rows = rows;
+    return before;
+}
 
 // max_chunks 0: one wave per (token, head). Otherwise one wave per chunk, for rows whose keys span at most
 // max_chunks chunks (the caller's promise: a row with more would lose its last ones), with part_o

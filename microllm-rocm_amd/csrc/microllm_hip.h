@@ -61,6 +61,10 @@ int mll_qkv_rope_store(const void* qkv, int in_dtype, int n_partials, int64_t pa
 // max_chunks chunks (chunks lie at absolute positions), and part_o [n_tokens * heads * max_chunks * head_dim]
 // and part_ml [n_tokens * heads * max_chunks * 2] floats are the workspace.
 int mll_paged_attention_rowwise_chunk();
+// In float32 with head sizes up to 128 a wave of the chunked kernel takes several query heads of a kv head (their
+// keys and values read once) from this many rows (tokens x waves a token) on; returns the value before. The same bits
+// either way.
+int64_t mll_rowwise_heads_from(int64_t rows);
 int mll_paged_attention_rowwise(const void* q, int dtype, const void* k_cache, const void* v_cache,
                                 const int32_t* block_table, int table_width,
                                 const int32_t* seq_of_token, const int32_t* positions, void* out,

@@ -325,6 +325,14 @@ def _check_paged(q, k_cache, v_cache, block_table, heads, kv_heads, head_dim) ->
 ROWWISE_SPLIT_BELOW = 2048      # (token, head) rows: with fewer, a row's chunks of keys get a wave each
 
 
+def rowwise_heads_from(rows: int) -> int:
+    """From how many rows (tokens x waves a token) on the chunked row-wise attention lets one wave take several
+    query heads of a kv head (float32, head sizes up to 128); returns the value before. Both ways give the same bits."""
+    lib = library.load()
+    lib.mll_rowwise_heads_from.restype = ctypes.c_int64
+    return int(lib.mll_rowwise_heads_from(ctypes.c_int64(int(rows))))
+
+
 def rowwise_chunks(longest: int, window: int) -> int:
     """The most chunks of keys (at absolute positions) that a row's visible keys can span, for rows that see at
     most ``longest`` keys' positions (position < longest)."""

@@ -268,7 +268,8 @@ def test_rowwise_attention(dtype, heads, kv_heads, hd, page_size, window):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kv_heads,hd,page_size,window", [
-    (4, 2, 16, 16, 0), (3, 1, 40, 16, 130), (6, 3, 128, 32, 0), (2, 1, 72, 16, 257), (5, 5, 48, 48, 1), (2, 2, 24, 16, 128)])
+    (4, 2, 16, 16, 0), (3, 1, 40, 16, 130), (6, 3, 128, 32, 0), (2, 1, 72, 16, 257), (5, 5, 48, 48, 1), (2, 2, 24, 16, 128),
+    (28, 4, 128, 16, 0), (12, 2, 64, 16, 200), (10, 2, 32, 48, 0), (16, 1, 96, 16, 129), (9, 1, 16, 16, 0)])
 def test_rowwise_attention_a_wave_per_chunk_gives_the_same_bits(dtype, heads, kv_heads, hd, page_size, window):
     """The plain kernel walks a row's keys by one wave, or by a wave per chunk of 128 keys with a merge: the same
     result to the last bit, whatever the row's position (chunk edges, one key beyond, many chunks) and window,
@@ -285,6 +286,15 @@ def test_rowwise_attention_a_wave_per_chunk_gives_the_same_bits(dtype, heads, kv
     by_chunk = k.paged_attention_rowwise(*args, split=True, longest=max(lengths))
     generous = k.paged_attention_rowwise(*args, split=True)      # as many chunks as the table is wide
     assert torch.equal(whole, by_chunk) and torch.equal(whole, generous)
+    # in float32 a wave of the chunked kernel may take several query heads of a kv head: forced, and forbidden
+    usual = k.rowwise_heads_from(1)
+    try:
+        several_heads = k.paged_attention_rowwise(*args, split=True, longest=max(lengths))
+        k.rowwise_heads_from(1 << 60)
+        one_head = k.paged_attention_rowwise(*args, split=True, longest=max(lengths))
+    finally:
+        k.rowwise_heads_from(usual)
+    assert torch.equal(whole, several_heads) and torch.equal(whole, one_head)
     reference = reference_attention(q_exact, ek, ev, seq, pos, heads, kv_heads, hd, scale, window)
     np.testing.assert_allclose(whole.float().cpu().numpy(), reference, **tolerance(dtype))
     assert k.rowwise_chunks(700, 0) == 6 and k.rowwise_chunks(128, 0) == 1 and k.rowwise_chunks(129, 0) == 2
