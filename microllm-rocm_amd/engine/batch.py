@@ -20,10 +20,15 @@ from ..ops.transfers import copy_to_device, on_device
 
 @dataclass
 class StepEntry:
-    """One request's next tokens and the places among them whose logits are wanted."""
+    """One request's next tokens and the places among them whose logits are wanted.
+
+    ``token_from``: the entry's one token is not known on the host yet; it is row ``token_from`` of the
+    ``device_tokens`` that the step is given (ids chosen on the device by the step before), and ``tokens`` holds a
+    stand-in."""
     request_id: Hashable
     tokens: Sequence[int]
     want: Sequence[int] = ()
+    token_from: Optional[int] = None
 
 
 @dataclass

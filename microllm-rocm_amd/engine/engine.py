@@ -12,6 +12,7 @@ from __future__ import annotations
 import os
 from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Union
 
+import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, RequestCache, pages_of_group
@@ -245,6 +246,7 @@ class Engine:
         else:
             ctx = state.builder.build(requests, [entry.tokens for entry in entries], every_row, fixed_width=width)
         self._last_graph = state
+        self._tokens_from_device(ctx.tokens, entries, list(range(n)))
         if state.graph is None:
             self._capture(state, ctx)
             self._policy.decode.trim(keep=key)
@@ -275,9 +277,26 @@ class Engine:
     def _padded_step(self, shape: FixedShape, batch: HostBatch) -> Optional[torch.Tensor]:
         """The step in its fixed shape, run eagerly."""
         ctx = self._builder.upload(batch, fixed=shape)
+        self._tokens_from_device(ctx.tokens, self._entries, batch.step.cu[:-1].tolist())
         logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
         wanted = int(batch.want_rows.size)
         return logits[:wanted] if wanted else None
+
+    def _tokens_from_device(self, tokens: torch.Tensor, entries: Sequence[StepEntry], places: List[int]) -> None:
+        """Put the tokens that entries take from ``device_tokens`` into the step's token list on the device
+        (``places[i]`` is where entry ``i``'s first token lies in it), after the host's stand-ins were copied there."""
+        source = self._device_tokens
+        if source is None:
+            return
+        taking = [(places[index], entry.token_from) for index, entry in enumerate(entries) if entry.token_from is not None]
+        if not taking:
+            return
+        count = len(taking)
+        if [place for place, _ in taking] == list(range(count)) and [row for _, row in taking] == list(range(count)):
+            tokens[:count].copy_(source[:count])      # the same requests in the same order as the step before
+            return
+        both = on_device(np.asarray(taking, dtype=np.int64).T.copy(), self.device)
+        tokens.index_copy_(0, both[0], source.index_select(0, both[1]))
 
     def _mixed_graph_step(self, shape: FixedShape, batch: HostBatch) -> Optional[torch.Tensor]:
         key = shape.key()
@@ -286,6 +305,7 @@ class Engine:
             state = _DecodeGraph(self, shape.width)
             self._policy.mixed.put(key, state, self._policy.evicted_mixed)
         ctx = state.builder.upload(batch, fixed=shape)
+        self._tokens_from_device(ctx.tokens, self._entries, batch.step.cu[:-1].tolist())
         if state.graph is None:
             self._capture(state, ctx)
             self._policy.captured_mixed(key)
@@ -315,8 +335,14 @@ class Engine:
         self.graphs_captured += 1
 
     # ---- the step ------------------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry], reserved: bool = False, borrow_logits: bool = False) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], reserved: bool = False, borrow_logits: bool = False,
+             device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Run one batch; returns float32 logits ``[wanted, vocab]`` in the order of entries and of ``want``.
+
+        ``device_tokens`` (int32, on the device): where entries with ``token_from`` take their token from, so that
+        a step can be launched before the ids that the step before chose have reached the host. Such an id is not
+        checked against the vocabulary here; an id that is none (-1, from logits that were not finite) embeds as a
+        row that is not finite either.
 
         With ``reserved`` the caller (a scheduler) has already taken the pages for every portion. The result is the
         caller's to keep. With ``borrow_logits`` it may be the buffer that a captured decode step writes, which the
@@ -341,7 +367,11 @@ class Engine:
             count = len(entry.tokens)
             if count == 0:
                 raise ValueError(f"request {entry.request_id!r} brings no tokens")
-            if count == 1:
+            if entry.token_from is not None:
+                if count != 1 or device_tokens is None or not 0 <= entry.token_from < device_tokens.shape[0]:
+                    raise ValueError(f"request {entry.request_id!r}: a token from the device is one token, a row of device_tokens")
+                lowest = highest = 0
+            elif count == 1:
                 lowest = highest = int(entry.tokens[0])
             else:
                 lowest, highest = int(min(entry.tokens)), int(max(entry.tokens))
@@ -371,11 +401,13 @@ class Engine:
                 for request in taken:
                     self.cache.cancel_reservation(request)
                 raise
+        self._device_tokens = device_tokens if any(entry.token_from is not None for entry in entries) else None
         try:
             if self.use_graphs and len(entries) <= MAX_GRAPH_REQUESTS and all(len(entry.tokens) == 1 for entry in entries):
                 logits = self._graph_step(requests, entries)
             else:
                 self._last_graph = None
+                self._entries = entries
                 batch = self._builder.prepare(requests, [entry.tokens for entry in entries], [entry.want for entry in entries])
                 shape = self._fixed_shape(batch) if self.use_graphs and self.graph_mixed_steps else None
                 if shape is not None and self._policy.wants_mixed(shape.key()):
@@ -384,6 +416,7 @@ class Engine:
                     logits = self._padded_step(shape, batch)
                 else:
                     ctx = self._builder.upload(batch)
+                    self._tokens_from_device(ctx.tokens, entries, batch.step.cu[:-1].tolist())
                     logits = self.model.forward(ctx, self._bindings, ctx.want_rows)
         except BaseException:
             self._roll_back(requests)

@@ -33,14 +33,16 @@ def _params_list(params, count: int) -> List[SamplingParams]:
 def generate(engine: Engine, prompts: Sequence[Sequence[int]],
              params: Union[None, SamplingParams, Sequence[SamplingParams]] = None,
              max_batched_tokens: int = 2048, prefill_chunk: int = 512, max_requests: Optional[int] = None,
-             arrival_steps: Optional[Sequence[int]] = None, return_scheduler: bool = False):
-    """Prompt plus generated tokens for every prompt, in input order."""
+             arrival_steps: Optional[Sequence[int]] = None, return_scheduler: bool = False, lookahead: bool = True):
+    """Prompt plus generated tokens for every prompt, in input order. With ``lookahead`` (the default: nobody looks
+    at a token before the end) a step is launched before the host has seen the tokens of the step before
+    (``Scheduler``); the tokens are the same."""
     single = bool(prompts) and isinstance(prompts[0], int)
     if single:
         prompts = [prompts]
     param_list = _params_list(params, len(prompts))
     scheduler = Scheduler(engine, max_batched_tokens=max_batched_tokens, prefill_chunk=prefill_chunk,
-                          max_requests=max_requests)
+                          max_requests=max_requests, lookahead=lookahead)
     ids = []
     for index, (prompt, request_params) in enumerate(zip(prompts, param_list)):
         arrival = arrival_steps[index] if arrival_steps is not None else None

@@ -11,6 +11,11 @@ token or at its length. States and reasons are the reference's
 into fixed slots and reserves capacity up front, so it has neither a token budget
 nor a way to run out of cache.
 
+With ``lookahead`` a step does not wait for the tokens it selects: they stay on the device, the next step takes
+them from there (``StepEntry.token_from``), and the host learns them one step late, while the GPU is already at
+work on that next step; what the host must decide before then (who runs, who ends at its length, who gets
+pages) needs only counts, not ids. A request with stop tokens is waited for as before.
+
 When pages run out: the running request that was admitted last is preempted. Its
 pages and slot go back, it returns to the head of the waiting queue, and when it
 is admitted again its prompt and the tokens it had generated are run again in
@@ -27,8 +32,10 @@ from dataclasses import dataclass, field
 from typing import Deque, Dict, Hashable, List, Optional, Sequence
 
 from ..cache.pages import OutOfPages
-from ..sampling import Sampler, SamplingParams
+from ..sampling import NonFiniteLogits, Sampler, SamplingParams
 from .batch import StepEntry
+
+NOT_YET = -1      # in Request.generated: a token that was selected on the device and has not reached the host
 
 
 class RequestState(enum.Enum):
@@ -103,6 +110,21 @@ class SchedulerMetrics:
 
 
 @dataclass(eq=False)
+class Pending:
+    """The tokens a step selected, still on their way to the host: for whom, where each lies in its request's
+    ``generated``, and the selection to ask."""
+    requests: List[Request]
+    places: List[int]
+    selection: object
+
+    def row_of(self, request: Request) -> Optional[int]:
+        for row, candidate in enumerate(self.requests):
+            if candidate is request:
+                return row
+        return None
+
+
+@dataclass(eq=False)
 class Portion:
     """What one request brings to a step."""
     request: Request
@@ -113,7 +135,7 @@ class Portion:
 
 class Scheduler:
     def __init__(self, engine, max_batched_tokens: int = 2048, prefill_chunk: int = 512,
-                 max_requests: Optional[int] = None, sampler: Optional[Sampler] = None):
+                 max_requests: Optional[int] = None, sampler: Optional[Sampler] = None, lookahead: bool = False):
         if max_batched_tokens <= 0 or prefill_chunk <= 0:
             raise ValueError("max_batched_tokens and prefill_chunk must be positive")
         self.engine = engine
@@ -123,6 +145,8 @@ class Scheduler:
         self.prefill_chunk = min(prefill_chunk, getattr(self.cache, "max_portion", None) or prefill_chunk)
         self.max_requests = min(max_requests or self.cache.max_requests, self.cache.max_requests)
         self.sampler = sampler or Sampler()
+        self.lookahead = lookahead
+        self._pending: Optional[Pending] = None
         self.requests: Dict[int, Request] = {}
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []     # in admission order
@@ -265,42 +289,88 @@ class Scheduler:
         if self.cache.groups:
             self.metrics.peak_held_pages = max(self.metrics.peak_held_pages, max(self.cache.held_pages()))
         produced: List[int] = []
-        if portions:
-            entries = []
-            for portion in portions:
-                request = portion.request
-                tokens = request.tokens_between(portion.start, portion.start + portion.count)
-                entries.append(StepEntry(request.id, tokens, [portion.count - 1] if portion.wants_logits else []))
-            try:
-                logits = self.engine.step(entries, reserved=True, borrow_logits=True)
-            except Exception:
-                self._step_failed(portions)
-                raise
-            for portion in portions:
-                if portion.count == 1 and portion.request.state == RequestState.DECODING:
-                    self.metrics.decode_tokens += 1
-                else:
-                    self.metrics.prefill_tokens += portion.count
-                self.metrics.batched_tokens += portion.count
-            self.metrics.engine_steps += 1
-            for portion in portions:
-                portion.request.computed += portion.count
-            wanting = [portion.request for portion in portions if portion.wants_logits]
-            if wanting:
-                tokens = self.sampler.select(logits, [r.params for r in wanting], [len(r.generated) for r in wanting])
-                now = time.perf_counter()
-                for request, token in zip(wanting, tokens):
-                    request.generated.append(int(token))
-                    request.state = RequestState.DECODING
-                    if request.first_token_time < 0:
-                        request.first_token_time = now
-                    produced.append(request.id)
-                    if int(token) in request.params.stop_tokens:      # emitted, then stop
-                        self._complete(request, CompletionReason.STOP_TOKEN)
-                    elif len(request.generated) >= request.params.max_new_tokens:
-                        self._complete(request, CompletionReason.LENGTH)
+        before, self._pending = self._pending, None      # what the step before selected and the host has not seen
+        try:
+            if portions:
+                entries = []
+                for portion in portions:
+                    request = portion.request
+                    tokens = request.tokens_between(portion.start, portion.start + portion.count)
+                    token_from = None
+                    if NOT_YET in tokens:
+                        row = before.row_of(request) if before is not None else None
+                        if portion.count == 1 and row is not None:
+                            tokens, token_from = [0], row      # the step takes it from the device
+                        else:                                    # a longer portion needs it here: wait for it
+                            self._learn(before)
+                            before = None
+                            tokens = request.tokens_between(portion.start, portion.start + portion.count)
+                    entries.append(StepEntry(request.id, tokens, [portion.count - 1] if portion.wants_logits else [], token_from))
+                device_tokens = before.selection.device if before is not None and any(e.token_from is not None for e in entries) else None
+                try:
+                    if device_tokens is None:
+                        logits = self.engine.step(entries, reserved=True, borrow_logits=True)
+                    else:
+                        logits = self.engine.step(entries, reserved=True, borrow_logits=True, device_tokens=device_tokens)
+                except Exception:
+                    self._step_failed(portions)
+                    raise
+                for portion in portions:
+                    if portion.count == 1 and portion.request.state == RequestState.DECODING:
+                        self.metrics.decode_tokens += 1
+                    else:
+                        self.metrics.prefill_tokens += portion.count
+                    self.metrics.batched_tokens += portion.count
+                self.metrics.engine_steps += 1
+                for portion in portions:
+                    portion.request.computed += portion.count
+                wanting = [portion.request for portion in portions if portion.wants_logits]
+                if wanting and self.lookahead and not any(r.params.stop_tokens for r in wanting):
+                    # Selected, not waited for: what ends a request here is its length, which needs no id.
+                    selection = self.sampler.select_later(logits, [r.params for r in wanting], [len(r.generated) for r in wanting])
+                    self._pending = Pending(list(wanting), [len(r.generated) for r in wanting], selection)
+                    for request in wanting:
+                        request.generated.append(NOT_YET)
+                        request.state = RequestState.DECODING
+                        produced.append(request.id)
+                        if len(request.generated) >= request.params.max_new_tokens:
+                            self._complete(request, CompletionReason.LENGTH)
+                elif wanting:
+                    tokens = self.sampler.select(logits, [r.params for r in wanting], [len(r.generated) for r in wanting])
+                    now = time.perf_counter()
+                    for request, token in zip(wanting, tokens):
+                        request.generated.append(int(token))
+                        request.state = RequestState.DECODING
+                        if request.first_token_time < 0:
+                            request.first_token_time = now
+                        produced.append(request.id)
+                        if int(token) in request.params.stop_tokens:      # emitted, then stop
+                            self._complete(request, CompletionReason.STOP_TOKEN)
+                        elif len(request.generated) >= request.params.max_new_tokens:
+                            self._complete(request, CompletionReason.LENGTH)
+        finally:
+            if before is not None:
+                self._learn(before)      # its copy has long arrived: the GPU is busy with the step just launched
         self.current_step += 1
         return produced
+
+    def _learn(self, pending: Pending) -> None:
+        """The host takes the ids of a selection it did not wait for."""
+        tokens = pending.selection.tokens()
+        now = time.perf_counter()
+        for request, place, token in zip(pending.requests, pending.places, tokens):
+            if place < len(request.generated) and request.generated[place] == NOT_YET:
+                request.generated[place] = int(token)
+            if request.first_token_time < 0:
+                request.first_token_time = now
+            if request.state == RequestState.COMPLETED and request.completion_time < now and place == len(request.generated) - 1:
+                request.completion_time = now      # it ended at its length before its last id was known
+
+    def drain(self) -> None:
+        """Wait for what the last step selected (``lookahead``): every generated id is then known to the host."""
+        pending, self._pending = self._pending, None
+        if pending is not None:
+            self._learn(pending)
 
     def run_until_idle(self, maximum_steps: int = -1) -> None:
         """Step until nothing runs or waits; more than ``maximum_steps`` is an error
@@ -311,6 +381,7 @@ class Scheduler:
                 raise RuntimeError(f"scheduler did not become idle within {maximum_steps} steps")
             self.step()
             steps += 1
+        self.drain()
 
     # ---- endings -------------------------------------------------------------------------
     def _release(self, request: Request) -> None:

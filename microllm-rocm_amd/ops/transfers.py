@@ -65,6 +65,12 @@ def on_host(tensor: torch.Tensor) -> torch.Tensor:
     return tensor.detach().to("cpu")
 
 
+def count_copy_to_host(tensor: torch.Tensor) -> None:
+    """A copy to the host that the caller makes itself (into pinned memory, without waiting) still counts."""
+    _stats.device_to_host_calls += 1
+    _stats.device_to_host_bytes += _bytes(tensor)
+
+
 def device_copy(tensor: torch.Tensor) -> torch.Tensor:
     """A copy on the same device."""
     _stats.device_to_device_calls += 1

@@ -1,3 +1,3 @@
-from .sampler import NonFiniteLogits, Sampler, SamplingParams, uniform_for
+from .sampler import NonFiniteLogits, Sampler, SamplingParams, Selection, uniform_for
 
-__all__ = ["NonFiniteLogits", "Sampler", "SamplingParams", "uniform_for"]
+__all__ = ["NonFiniteLogits", "Sampler", "SamplingParams", "Selection", "uniform_for"]

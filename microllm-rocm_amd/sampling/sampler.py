@@ -20,7 +20,7 @@ import numpy as np
 import torch
 
 from ..ops import kernels
-from ..ops.transfers import on_device, on_host
+from ..ops.transfers import count_copy_to_host, on_device, on_host
 
 _MASK = (1 << 64) - 1
 
@@ -65,27 +65,58 @@ class NonFiniteLogits(RuntimeError):
     """A row of logits held NaN or infinity (the reference throws too, src/inference/scheduler.cpp:918-920)."""
 
 
+class Selection:
+    """Tokens that have been chosen on the device and are on their way to the host. ``device`` is the int32 tensor
+    of chosen ids (a row per row of logits), which a following step may take its tokens from without waiting;
+    ``tokens()`` waits for the copy and returns them, raising ``NonFiniteLogits`` for a row that held none."""
+
+    def __init__(self, device: torch.Tensor, host: torch.Tensor, copied: "torch.cuda.Event"):
+        self.device, self._host, self._copied = device, host, copied
+        self._tokens = None
+
+    def tokens(self) -> List[int]:
+        if self._tokens is None:
+            self._copied.synchronize()
+            self._tokens = self._host.tolist()
+            for row, token in enumerate(self._tokens):
+                if token < 0:
+                    raise NonFiniteLogits(f"row {row} of the logits is not finite")
+        return self._tokens
+
+
 class Sampler:
     """Selects one token per row of logits on the device; one transfer of the chosen ids back."""
 
-    def select(self, logits: torch.Tensor, params: Sequence[SamplingParams], draws: Sequence[int]) -> List[int]:
+    def _choose(self, logits: torch.Tensor, params: Sequence[SamplingParams], draws: Sequence[int]) -> torch.Tensor:
         if logits.shape[0] != len(params) or len(params) != len(draws):
             raise ValueError("one SamplingParams and one draw index per row of logits")
         if all(p.greedy for p in params):
-            chosen = kernels.argmax(logits)
-        else:
-            # one transfer for the three per-row values: temperatures, top-k counts (as int32 bits) and uniforms
-            packed = np.empty((3, len(params)), dtype=np.float32)
-            packed[0] = [0.0 if p.greedy else p.temperature for p in params]
-            packed[1].view(np.int32)[:] = [p.top_k for p in params]
-            packed[2] = [uniform_for(p.seed, d) for p, d in zip(params, draws)]
-            values = on_device(packed, logits.device)
-            temperature, top_k, uniform = values[0], values[1].view(torch.int32), values[2]
-            if all(p.top_k == 0 for p in params):
-                top_k = None      # no row is restricted: the kernel leaves its search for the k-th value out
-            chosen = kernels.sample(logits, temperature, top_k, uniform)
-        tokens = on_host(chosen).tolist()
+            return kernels.argmax(logits)
+        # one transfer for the three per-row values: temperatures, top-k counts (as int32 bits) and uniforms
+        packed = np.empty((3, len(params)), dtype=np.float32)
+        packed[0] = [0.0 if p.greedy else p.temperature for p in params]
+        packed[1].view(np.int32)[:] = [p.top_k for p in params]
+        packed[2] = [uniform_for(p.seed, d) for p, d in zip(params, draws)]
+        values = on_device(packed, logits.device)
+        temperature, top_k, uniform = values[0], values[1].view(torch.int32), values[2]
+        if all(p.top_k == 0 for p in params):
+            top_k = None      # no row is restricted: the kernel leaves its search for the k-th value out
+        return kernels.sample(logits, temperature, top_k, uniform)
+
+    def select(self, logits: torch.Tensor, params: Sequence[SamplingParams], draws: Sequence[int]) -> List[int]:
+        tokens = on_host(self._choose(logits, params, draws)).tolist()
         for row, token in enumerate(tokens):
             if token < 0:
                 raise NonFiniteLogits(f"row {row} of the logits is not finite")
         return tokens
+
+    def select_later(self, logits: torch.Tensor, params: Sequence[SamplingParams], draws: Sequence[int]) -> Selection:
+        """The same choice without waiting for it: the ids stay on the device for whoever steps next, and their
+        copy to pinned host memory is under way when this returns."""
+        chosen = self._choose(logits, params, draws)
+        host = torch.empty(chosen.shape, dtype=chosen.dtype, pin_memory=True)
+        host.copy_(chosen, non_blocking=True)
+        count_copy_to_host(chosen)
+        copied = torch.cuda.Event()
+        copied.record()
+        return Selection(chosen, host, copied)

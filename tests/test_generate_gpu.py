@@ -531,3 +531,26 @@ def test_a_step_copies_its_metadata_once_and_nothing_back(tmp_path, dtype):
     generate(engine, [prompts["b"]], GenerationConfig(max_new_tokens=6, temperature=0.0))
     moved = transfer_stats()
     assert moved.device_to_host_calls == 6 and moved.device_to_host_bytes == 6 * 4, "the chosen id of every step, nothing else"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_lookahead_generates_the_same_tokens(tmp_path, dtype):
+    """Steps launched before the host has seen the tokens of the step before (they take them from the device) give
+    what waiting for every token gives: greedy and sampled, prompts in portions beside decoding, arrivals at
+    different steps, and a pool so small that requests are preempted and run again from ids the host must have."""
+    from microllm_rocm_amd import GenerationConfig, generate
+    folder = make_folder(tmp_path, "B", SHARP)
+    config = CONFIGS["B"]
+    prompts = [random_tokens(80 + index, length, config.vocab_size) for index, length in enumerate((5, 17, 40, 64, 9, 33))]
+    params = [GenerationConfig(max_new_tokens=20 + index, temperature=(0.0, 0.8)[index % 2], seed=index, top_k=(0, 20, 0)[index % 3])
+              for index in range(len(prompts))]
+    for options in ({"max_tokens": 2048}, {"num_pages": 9, "max_tokens": None}):
+        engine = engine_for(folder, dtype, max_requests=4, **options)
+        common = dict(prefill_chunk=16, max_batched_tokens=32, arrival_steps=[0, 0, 2, 3, 9, 9], return_scheduler=True)
+        waited, slow = generate(engine, prompts, params, lookahead=False, **common)
+        ahead, fast = generate(engine, prompts, params, lookahead=True, **common)
+        assert ahead == waited
+        assert fast.metrics.preemptions == slow.metrics.preemptions and (fast.metrics.preemptions > 0) == ("num_pages" in options)
+        assert all(token >= 0 for output in ahead for token in output)
+        engine.cache.check()
+        assert not engine.cache.requests

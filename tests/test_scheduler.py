@@ -29,18 +29,25 @@ class FakeEngine:
         self.spec = SimpleNamespace(vocab_size=VOCAB, max_positions=max_positions)
         self.fed = {}
         self.batches = []
+        self.from_device = 0
 
-    def step(self, entries, reserved=False, borrow_logits=False):
+    def step(self, entries, reserved=False, borrow_logits=False, device_tokens=None):
         assert reserved
         rows = []
         self.batches.append([(entry.request_id, len(entry.tokens)) for entry in entries])
+        self.from_device += sum(entry.token_from is not None for entry in entries)
         for entry in entries:
             request = self.cache.get(entry.request_id)
             history = self.fed.setdefault(entry.request_id, [])
             if request.num_tokens == 0:
                 history.clear()               # run again after a preemption
             assert len(history) == request.num_tokens
-            history.extend(entry.tokens)
+            tokens = list(entry.tokens)
+            if entry.token_from is not None:  # an id the host has not seen: the step reads it where it was selected
+                assert len(tokens) == 1
+                tokens = [int(device_tokens[entry.token_from])]
+            assert all(0 <= token < VOCAB for token in tokens)
+            history.extend(tokens)
             for place in entry.want:
                 rows.append(logits_after(history[:request.num_tokens + place + 1]))
             self.cache.commit(request, len(entry.tokens))
@@ -52,6 +59,21 @@ class PlainSampler:
     def select(self, logits, params, draws):
         return [plain.sample(row.numpy().astype(np.float64), p.temperature, p.top_k, plain.uniform_for(p.seed, d))
                 for row, p, d in zip(logits, params, draws)]
+
+    def select_later(self, logits, params, draws):
+        """What ``Sampler.select_later`` returns: the ids where the next step can read them, and a way to ask for
+        them; asked, it counts, so that a test can tell whether the scheduler waited."""
+        chosen = self.select(logits, params, draws)
+        sampler = self
+
+        class Later:
+            device = torch.tensor(chosen, dtype=torch.int32)
+
+            def tokens(self):
+                sampler.asked_later = getattr(sampler, "asked_later", 0) + 1
+                return list(chosen)
+
+        return Later()
 
 
 def alone(prompt, params):
@@ -216,14 +238,14 @@ class FailingEngine(FakeEngine):
             from microllm_rocm_amd.parts import StateNeed
             self.cache = CacheManager([PagedKVNeed(1, 8, None), StateNeed((2,))], [None, None], 4, 16, 4, device=None)
 
-    def step(self, entries, reserved=False, borrow_logits=False):
+    def step(self, entries, reserved=False, borrow_logits=False, device_tokens=None):
         self.calls += 1
         if self.calls == self.fail_at:
             # what Engine.step does when the model raises: the step's reservations are given back
             for entry in entries:
                 self.cache.cancel_reservation(self.cache.get(entry.request_id))
             raise RuntimeError("a kernel refused its arguments")
-        return super().step(entries, reserved)
+        return super().step(entries, reserved, device_tokens=device_tokens)
 
 
 @pytest.mark.parametrize("state", [False, True])
@@ -263,18 +285,50 @@ def test_a_request_alone_always_fits_and_idle_limit_is_an_error():
         s.run_until_idle(maximum_steps=2)
 
 
-@pytest.mark.parametrize("seed", range(4))
-def test_random_workloads_match_requests_run_alone(seed):
+@pytest.mark.parametrize("lookahead", [False, True])
+@pytest.mark.parametrize("seed", range(6))
+def test_random_workloads_match_requests_run_alone(seed, lookahead):
+    """Also with ``lookahead``, where the host learns a step's tokens while the next step runs: the pool is small
+    enough for preemptions (recomputation needs the ids on the host), some requests have stop tokens (waited for
+    as ever), and every token must be what the request generates alone."""
     rng = np.random.default_rng(seed)
     engine = FakeEngine(num_pages=int(rng.integers(10, 24)), page_size=4, max_requests=3, window=None if seed % 2 else 12)
-    s = scheduler(engine, max_batched_tokens=int(rng.integers(4, 20)), prefill_chunk=int(rng.integers(2, 12)))
+    s = scheduler(engine, max_batched_tokens=int(rng.integers(4, 20)), prefill_chunk=int(rng.integers(2, 12)), lookahead=lookahead)
     jobs = []
     for index in range(8):
         prompt = rng.integers(0, VOCAB, size=int(rng.integers(1, 14))).tolist()
+        stops = tuple(rng.choice(VOCAB, size=3, replace=False).tolist()) if seed >= 4 and index % 3 == 0 else ()
         params = SamplingParams(max_new_tokens=int(rng.integers(1, 12)), temperature=float(rng.choice([0.0, 0.8])),
-                                top_k=int(rng.choice([0, 5])), seed=index)
+                                top_k=int(rng.choice([0, 5])), seed=index, stop_tokens=stops)
         jobs.append((s.submit(prompt, params, arrival_step=int(rng.integers(0, 10))), prompt, params))
     s.run_until_idle(maximum_steps=2000)
     for rid, prompt, params in jobs:
         assert s.request(rid).generated == alone(prompt, params)
+        assert s.request(rid).first_token_time > 0 and s.request(rid).completion_time >= s.request(rid).first_token_time
     assert engine.cache.free_pages() == [engine.cache.groups[0].pool.num_pages]
+    if not lookahead:
+        assert engine.from_device == 0
+    elif seed < 4:      # (a step that selects for a request with stop tokens waits, for all its requests)
+        assert engine.from_device > 0, "with lookahead steps take tokens that the host has not seen"
+
+
+def test_lookahead_learns_a_step_s_tokens_one_step_late_and_all_of_them_in_the_end():
+    engine = FakeEngine(num_pages=32, page_size=4)
+    sampler = PlainSampler()
+    s = Scheduler(engine, sampler=sampler, lookahead=True)
+    params = SamplingParams(max_new_tokens=6, temperature=0.0)
+    first, second = s.submit([1, 2, 3], params), s.submit([4, 5], params)
+    s.step()                                      # both prompts; their first tokens are selected, not waited for
+    assert s.request(first).generated == [-1] and getattr(sampler, "asked_later", 0) == 0
+    s.step()                                      # launched with ids from the device, then the first step's are learnt
+    assert sampler.asked_later == 1 and s.request(first).generated[0] >= 0 and s.request(first).generated[1] == -1
+    assert engine.from_device == 2
+    s.run_until_idle()
+    assert s.request(first).generated == alone([1, 2, 3], params) and s.request(second).generated == alone([4, 5], params)
+    assert all(token >= 0 for rid in (first, second) for token in s.request(rid).generated)
+    # a request with stop tokens is waited for in the step that selects for it
+    stopping = SamplingParams(max_new_tokens=6, temperature=0.0, stop_tokens=(alone([7, 8], params)[2],))
+    third = s.submit([7, 8], stopping)
+    s.run_until_idle()
+    assert s.request(third).generated == alone([7, 8], stopping) and len(s.request(third).generated) == 3
+    assert s.request(third).completion_reason.value == "stop_token"
