@@ -114,6 +114,9 @@ class Engine:
             raise RuntimeError("no GPU is visible; this engine has no CPU path")
         library.load()  # fail now, and loudly, if the kernels are missing and cannot be built
         self._ahead: Optional[_BuiltAhead] = None
+        self._borrow = False
+        self._entries: Sequence[StepEntry] = ()
+        self._device_tokens: Optional[torch.Tensor] = None     # of the step that is running, if it takes tokens from there
         self.steps_built_ahead = 0      # decode steps whose metadata was ready when they came
         self._last_graph: Optional[_DecodeGraph] = None
         if tune_library and not kernels.library_tuning():
