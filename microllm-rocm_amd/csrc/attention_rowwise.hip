@@ -221,12 +221,14 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_kernel(
 // attend_chunk: the dot products in ascending dims, the tile's maximum and sum over the wave, the values in the
 // order of the keys; only what is independent of the head (addresses, loads) is done once. Writes what MODE 1 writes,
 // bit for bit. Head sizes up to 64 * DIMS <= 128.
-template <typename T, int DIMS, int GW>
+// MODE as in the kernel for one head a wave: 0 walks all chunks of the row and merges as it goes (out), 1 takes the chunk
+// blockIdx.z and leaves its result in the workspace (part_o, part_ml).
+template <typename T, int MODE, int DIMS, int GW>
 __global__ __launch_bounds__(kWave) void paged_attention_rowwise_heads_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ seq_of_token,
-    const int32_t* __restrict__ positions, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks,
-    float scale, int window, int heads, int kv_heads, int head_dim, int page_size) {
+    const int32_t* __restrict__ positions, T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
+    int max_chunks, float scale, int window, int heads, int kv_heads, int head_dim, int page_size) {
     __shared__ float q_shared[GW][64 * DIMS];
     __shared__ float p_shared[GW][kWave];
     __shared__ int64_t v_shared[2][kWave];
@@ -242,7 +244,7 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_heads_kernel(
     const int position = positions[token];
     const int low = window > 0 ? max(0, position - window + 1) : 0;
     const int first_chunk = low / kRowwiseChunk, last_chunk = position / kRowwiseChunk;
-    if (first_chunk + static_cast<int>(blockIdx.z) > last_chunk) return;
+    if (MODE == 1 && first_chunk + static_cast<int>(blockIdx.z) > last_chunk) return;
     const int32_t* table = block_table + static_cast<int64_t>(seq) * table_width;
 #pragma unroll
     for (int g = 0; g < GW; ++g) {
@@ -251,9 +253,9 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_heads_kernel(
     }
     __syncthreads();
 
-    const int chunk = first_chunk + blockIdx.z;
-    const int first = max(low, chunk * kRowwiseChunk), last = min(position, chunk * kRowwiseChunk + kRowwiseChunk - 1);
     float acc[GW][DIMS], chunk_max[GW], chunk_sum[GW];
+    // The keys [first, last] of one chunk, from zero: attend_chunk for every head of the wave.
+    auto attend = [&](int first, int last) __attribute__((always_inline)) {
 #pragma unroll
     for (int g = 0; g < GW; ++g) {
         chunk_max[g] = -INFINITY;
@@ -331,17 +333,54 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_heads_kernel(
             }
         }
     }
+    };
+
+    if (MODE == 1) {
+        const int chunk = first_chunk + blockIdx.z;
+        attend(max(low, chunk * kRowwiseChunk), min(position, chunk * kRowwiseChunk + kRowwiseChunk - 1));
+#pragma unroll
+        for (int g = 0; g < GW; ++g) {
+            const int64_t slot = (static_cast<int64_t>(token) * heads + first_head + g) * max_chunks + blockIdx.z;
+#pragma unroll
+            for (int i = 0; i < DIMS; ++i) {
+                const int d = lane + i * kWave;
+                if (d < head_dim) part_o[slot * head_dim + d] = acc[g][i];
+            }
+            if (lane == 0) {
+                part_ml[slot * 2] = chunk_max[g];
+                part_ml[slot * 2 + 1] = chunk_sum[g];
+            }
+        }
+        return;
+    }
+    float total[GW][DIMS], total_max[GW], total_sum[GW];
 #pragma unroll
     for (int g = 0; g < GW; ++g) {
-        const int64_t slot = (static_cast<int64_t>(token) * heads + first_head + g) * max_chunks + blockIdx.z;
+        total_max[g] = -INFINITY;
+        total_sum[g] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < DIMS; ++i) total[g][i] = 0.0f;
+    }
+    for (int chunk = first_chunk; chunk <= last_chunk; ++chunk) {
+        attend(max(low, chunk * kRowwiseChunk), min(position, chunk * kRowwiseChunk + kRowwiseChunk - 1));
+#pragma unroll
+        for (int g = 0; g < GW; ++g) {
+            float new_max, keep, add;
+            merge_scales(total_max[g], chunk_max[g], new_max, keep, add);
+            total_sum[g] = merged(total_sum[g], keep, chunk_sum[g], add);
+#pragma unroll
+            for (int i = 0; i < DIMS; ++i) total[g][i] = merged(total[g][i], keep, acc[g][i], add);
+            total_max[g] = new_max;
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < GW; ++g) {
+        T* out_row = out + (static_cast<int64_t>(token) * heads + first_head + g) * head_dim;
+        const float inverse = 1.0f / total_sum[g];
 #pragma unroll
         for (int i = 0; i < DIMS; ++i) {
             const int d = lane + i * kWave;
-            if (d < head_dim) part_o[slot * head_dim + d] = acc[g][i];
-        }
-        if (lane == 0) {
-            part_ml[slot * 2] = chunk_max[g];
-            part_ml[slot * 2 + 1] = chunk_sum[g];
+            if (d < head_dim) out_row[d] = from_float<T>(__fmul_rn(total[g][i], inverse));
         }
     }
 }
@@ -397,7 +436,29 @@ static int launch_rowwise_dims(const void* q, const void* k_cache, const void* v
                           int table_width, const int32_t* seq_of_token, const int32_t* positions, void* out,
                           float* part_o, float* part_ml, int max_chunks, float scale, int window, int n_tokens,
                           int heads, int kv_heads, int head_dim, int page_size, hipStream_t stream) {
+    const int gw = (std::is_same<T, float>::value && DIMS <= 2) ? heads_a_wave(heads / kv_heads) : 1;
+    const bool several_heads = gw >= 2 && static_cast<int64_t>(n_tokens) * (heads / gw) >= grouped_from_rows;
+#define MLL_ROWWISE_HEADS(MODE, GW)                                                                                    \
+    case GW:                                                                                                           \
+        paged_attention_rowwise_heads_kernel<T, MODE, DIMS, GW><<<heads_grid, kWave, 0, stream>>>(                      \
+            static_cast<const T*>(q), static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), block_table,    \
+            table_width, seq_of_token, positions, static_cast<T*>(out), part_o, part_ml, max_chunks, scale, window,   \
+            heads, kv_heads, head_dim, page_size);                                                                     \
+        break;
+#define MLL_ROWWISE_HEADS_ALL(MODE)                                                                                    \
+    switch (gw) {                                                                                                      \
+        MLL_ROWWISE_HEADS(MODE, 2) MLL_ROWWISE_HEADS(MODE, 3) MLL_ROWWISE_HEADS(MODE, 4) MLL_ROWWISE_HEADS(MODE, 5)    \
+        MLL_ROWWISE_HEADS(MODE, 6) MLL_ROWWISE_HEADS(MODE, 7) MLL_ROWWISE_HEADS(MODE, 8)                               \
+        default: break;                                                                                                \
+    }
     if (max_chunks == 0) {
+        if constexpr (std::is_same<T, float>::value && DIMS <= 2) {
+            if (several_heads) {
+                const dim3 heads_grid(n_tokens, heads / gw);
+                MLL_ROWWISE_HEADS_ALL(0)
+                return check_launch("paged_attention_rowwise");
+            }
+        }
         paged_attention_rowwise_kernel<T, 0, DIMS><<<dim3(n_tokens, heads), kWave, 0, stream>>>(
             static_cast<const T*>(q), static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), block_table,
             table_width, seq_of_token, positions, static_cast<T*>(out), nullptr, nullptr, 0, scale, window, heads,
@@ -405,27 +466,13 @@ static int launch_rowwise_dims(const void* q, const void* k_cache, const void* v
         return check_launch("paged_attention_rowwise");
     }
     // Several query heads of a kv head in one wave where the step still has rows enough for the GPU that way
-    // (float32, head sizes up to 128: the path of the 32-bit engine; 64 requests of 4096 keys at 7B sizes).
-    const int gw = (std::is_same<T, float>::value && DIMS <= 2) ? heads_a_wave(heads / kv_heads) : 1;
-    const int64_t grouped_rows = static_cast<int64_t>(n_tokens) * (heads / gw);
+    // (float32, head sizes up to 128: the path of the 32-bit engine).
     bool grouped = false;
     if constexpr (std::is_same<T, float>::value && DIMS <= 2) {
-        if (gw >= 2 && grouped_rows >= grouped_from_rows) {
+        if (several_heads) {
             grouped = true;
-            const dim3 grid(n_tokens, heads / gw, max_chunks);
-#define MLL_ROWWISE_HEADS(GW)                                                                                          \
-    case GW:                                                                                                           \
-        paged_attention_rowwise_heads_kernel<T, DIMS, GW><<<grid, kWave, 0, stream>>>(                                 \
-            static_cast<const T*>(q), static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), block_table,    \
-            table_width, seq_of_token, positions, part_o, part_ml, max_chunks, scale, window, heads, kv_heads,        \
-            head_dim, page_size);                                                                                      \
-        break;
-            switch (gw) {
-                MLL_ROWWISE_HEADS(2) MLL_ROWWISE_HEADS(3) MLL_ROWWISE_HEADS(4) MLL_ROWWISE_HEADS(5)
-                MLL_ROWWISE_HEADS(6) MLL_ROWWISE_HEADS(7) MLL_ROWWISE_HEADS(8)
-                default: grouped = false;
-            }
-#undef MLL_ROWWISE_HEADS
+            const dim3 heads_grid(n_tokens, heads / gw, max_chunks);
+            MLL_ROWWISE_HEADS_ALL(1)
         }
     }
     if (!grouped)
@@ -437,6 +484,8 @@ static int launch_rowwise_dims(const void* q, const void* k_cache, const void* v
     paged_attention_rowwise_merge_kernel<T, DIMS><<<dim3(n_tokens, heads), kWave, 0, stream>>>(
         part_o, part_ml, seq_of_token, positions, static_cast<T*>(out), max_chunks, window, heads, head_dim);
     return check_launch("paged_attention_rowwise_merge");
+#undef MLL_ROWWISE_HEADS_ALL
+#undef MLL_ROWWISE_HEADS
 }
 
 template <typename T>

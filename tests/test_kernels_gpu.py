@@ -289,12 +289,12 @@ def test_rowwise_attention_a_wave_per_chunk_gives_the_same_bits(dtype, heads, kv
     # in float32 a wave of the chunked kernel may take several query heads of a kv head: forced, and forbidden
     usual = k.rowwise_heads_from(1)
     try:
-        several_heads = k.paged_attention_rowwise(*args, split=True, longest=max(lengths))
+        several_heads = [k.paged_attention_rowwise(*args, split=True, longest=max(lengths)), k.paged_attention_rowwise(*args, split=False)]
         k.rowwise_heads_from(1 << 60)
-        one_head = k.paged_attention_rowwise(*args, split=True, longest=max(lengths))
+        one_head = [k.paged_attention_rowwise(*args, split=True, longest=max(lengths)), k.paged_attention_rowwise(*args, split=False)]
     finally:
         k.rowwise_heads_from(usual)
-    assert torch.equal(whole, several_heads) and torch.equal(whole, one_head)
+    assert all(torch.equal(whole, other) for other in several_heads + one_head)
     reference = reference_attention(q_exact, ek, ev, seq, pos, heads, kv_heads, hd, scale, window)
     np.testing.assert_allclose(whole.float().cpu().numpy(), reference, **tolerance(dtype))
     assert k.rowwise_chunks(700, 0) == 6 and k.rowwise_chunks(128, 0) == 1 and k.rowwise_chunks(129, 0) == 2
