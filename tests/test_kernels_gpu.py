@@ -418,6 +418,37 @@ def test_gemm_f32_and_row_independence(m, n, k):
     assert torch.equal(alone[0], out[-1])
 
 
+@pytest.mark.parametrize("n,k,parts", [(3584, 3584, 8), (1152, 1792, 4), (896, 4864, 8), (37888, 512, 1), (640, 901, 2), (3000, 1026, 2), (200, 300, 1)])
+def test_gemm_f32_in_parts_gives_every_row_the_same_bits_in_every_batch(n, k, parts):
+    """The 32-bit product cuts the reduction of a weight with few rows of its own into parts by the weight's shape
+    alone; the parts, added in order, are the product, and a row's parts are the same bits whether it comes alone, with
+    15 others (one element a thread, or 2 x 2), with 40 (tiles of 16 x 32 or 32 x 64), 64 (64 x 64) or 600 (128 x 64):
+    every kernel sums an element in ascending k with one fused multiply-add a term. Reductions that are no multiple of 4
+    (no 16-byte loads) and of 2 mod 4 are among the shapes."""
+    ka = kernels()
+    assert ka.f32_splits(n, k) == parts
+    rng = np.random.default_rng(n + k)
+    a = rng.normal(size=(600, k)).astype(np.float32)
+    w = (rng.normal(size=(n, k)) * 0.05).astype(np.float32)
+    bias = rng.normal(size=n).astype(np.float32)
+    device_a, device_w, device_bias = (torch.from_numpy(x).to(DEVICE) for x in (a, w, bias))
+    whole = ka.gemm_f32(device_a, device_w, device_bias, partials=True)
+    assert tuple(whole.shape) == ((parts, 600, n) if parts > 1 else (600, n))
+    total = whole.double().sum(0) if parts > 1 else whole.double()
+    expected = a.astype(np.float64) @ w.astype(np.float64).T + bias
+    np.testing.assert_allclose(total.cpu().numpy(), expected, rtol=3e-5, atol=3e-5 * np.abs(expected).max())
+    if parts > 1:      # the bias is in the first part alone, and the parts are sums over consecutive ranges of k
+        part_length = -(-(-(-k // parts)) // 4) * 4
+        second = a[:3, part_length:2 * part_length].astype(np.float64) @ w[:, part_length:2 * part_length].astype(np.float64).T
+        np.testing.assert_allclose(whole[1, :3].double().cpu().numpy(), second, rtol=3e-5, atol=3e-5 * np.abs(second).max())
+    for rows in (1, 16, 40, 64):
+        fewer = ka.gemm_f32(device_a[:rows].contiguous(), device_w, device_bias, partials=True)
+        assert torch.equal(fewer, whole[..., :rows, :]), f"{rows} rows: other bits than the same rows among 600"
+    unsplit = ka.gemm_f32(device_a[:40].contiguous(), device_w, device_bias)      # one sum an element when the caller wants no parts
+    assert tuple(unsplit.shape) == (40, n)
+    np.testing.assert_allclose(unsplit.cpu().numpy(), expected[:40], rtol=3e-5, atol=3e-5 * np.abs(expected).max())
+
+
 @pytest.mark.parametrize("m", [1, 3, 8, 33, 64, 100])
 @pytest.mark.parametrize("n,k", [(331, 120), (1000, 96), (256, 3584), (4608, 512)])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
