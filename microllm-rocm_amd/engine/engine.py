@@ -268,14 +268,15 @@ class Engine:
         the padded step is then replayed from a graph or run eagerly is the policy's choice (most shapes of a
         changing workload come once); it is padded either way, so that the kernels' choices that follow the number
         of rows (which product, how a reduction is cut) are the same both times and a step gives the same bits
-        whether its shape happens to be captured or not."""
+        whether its shape happens to be captured or not. A planner's array that is empty stays empty: the kernel it
+        would feed (single tokens beside a prompt that has none) is then not launched at all."""
         step = batch.step
         wanted = int(batch.want_rows.size)
         if step.n_tokens > MAX_GRAPH_TOKENS or step.n_seqs > MAX_GRAPH_REQUESTS or wanted > MAX_GRAPH_WANTED:
             return None
         return FixedShape(tokens=_token_rows(step.n_tokens), requests=_power_of_two(step.n_seqs),
                           wanted=_wanted_rows(wanted), width=_power_of_two(batch.blocks_needed, MIN_GRAPH_WIDTH),
-                          planned={name: _power_of_two(rows) for name, rows in batch.planned_rows().items()})
+                          planned={name: _power_of_two(rows) if rows else 0 for name, rows in batch.planned_rows().items()})
 
     def _padded_step(self, shape: FixedShape, batch: HostBatch) -> Optional[torch.Tensor]:
         """The step in its fixed shape, run eagerly."""
