@@ -67,9 +67,10 @@ class Part:
 
     def flops(self, tokens: int) -> float:
         """Floating-point operations of this part over one request's prompt of ``tokens`` ids (2 per multiply-add);
-        by default those of its matrix products, found as attributes with ``out_features`` and ``in_features``."""
+        by default those of its matrix products: its attributes that are a ``linear.Weight``."""
+        from .linear import Weight      # (linear imports nothing of this module)
         return sum(2.0 * value.out_features * value.in_features * tokens for value in vars(self).values()
-                   if hasattr(value, "out_features") and hasattr(value, "in_features"))
+                   if isinstance(value, Weight))
 
     def name(self, role: str) -> str:
         try:
