@@ -21,6 +21,7 @@
 // XCD gets the same number of tiles.
 #include <utility>
 
+#include "cache_layout.h"
 #include "common.h"
 #include "microllm_hip.h"
 
@@ -97,12 +98,14 @@ __device__ __attribute__((always_inline)) inline void operands_arrived(TiledOper
                      :: "memory");
 }
 
-// EPILOGUE: 0 = float32 [M, N]; 1 = bfloat16 [M, N]; 2 = bfloat16 [M, N / 2] = silu(even rows of W) * (odd rows).
+// EPILOGUE: 0 = float32 [M, N]; 1 = bfloat16 [M, N]; 2 = bfloat16 [M, N / 2] = silu(even rows of W) * (odd rows);
+// 3 = queries, keys and values: bias, rotation, queries to `store.q_out`, keys and values into their pages (W's rows
+// in rotary pair order; see MllQkvStore).
 // With epilogue 0 the stages of k may be dealt to gridDim.y workgroups, each writing its own [M, N] of partial sums.
 template <int EPILOGUE>
 __global__ __launch_bounds__(kTiledThreads, 1) void gemm_tiled_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w_packed,
                                                                       void* __restrict__ out, int m, int n, int k, int n_tiles,
-                                                                      int k_steps, int m_blocks, int n_blocks) {
+                                                                      int k_steps, int m_blocks, int n_blocks, MllQkvStore store) {
     // Two slots. In a slot: A as [16 pieces of 16 rows][row][8 places of 16 bytes], the row's chunk c of 8 elements at
     // place c ^ (row / 2); then W as [16 tiles][2 k steps][1 KB in MFMA operand order]. Only the direct loads write
     // this memory and only the asm reads read it.
@@ -243,6 +246,79 @@ __global__ __launch_bounds__(kTiledThreads, 1) void gemm_tiled_kernel(const bf16
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
     }
 
+    if constexpr (EPILOGUE == 3) {
+        // The lane's 4 columns of a tile lie in one head (head_dim is a multiple of 16). In a query or key head
+        // columns 2p and 2p + 1 hold dims p and p + n_freq, the two that rotate together, so the lane's columns are
+        // dims p, p + n_freq, p + 1, p + 1 + n_freq with p even: two neighbours in each half, stored as one word
+        // each. Dims beyond the rotated ones, and values, are in place.
+        const CacheLayout layout(store.kv_heads, store.page_size, store.head_dim);
+#pragma unroll
+        for (int nt = 0; nt < kWaveTilesN; ++nt) {
+            const int column = (n_tile0 + wave_n * kWaveTilesN + nt) * 16 + quad * 4;
+            if (column >= n) continue;
+            const int head = column / store.head_dim, within = column % store.head_dim;
+            const bool is_query = head < store.heads;
+            const bool is_value = head >= store.heads + store.kv_heads;
+            const bool rotate = !is_value && within + 3 < 2 * store.n_freq;        // both pairs or, n_freq being even here, none
+            const int pair = within / 2;
+            // dims of the lane's four results, in the order of the accumulator
+            int dim[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dim[i] = rotate ? pair + i / 2 + (i % 2) * store.n_freq : within + i;
+            float bias[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (store.bias) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) bias[i] = store.bias[head * store.head_dim + dim[i]];
+            }
+#pragma unroll
+            for (int mt = 0; mt < kWaveTilesM; ++mt) {
+                const int row = m0 + wave_m * 128 + mt * 16 + col;
+                if (row >= m) continue;
+                float y[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) y[i] = acc[nt][mt][i] + bias[i];
+                if (rotate) {
+                    const floatx4 cs = *reinterpret_cast<const floatx4*>(store.cos_sin + (static_cast<int64_t>(row) * store.n_freq + pair) * 2);
+                    const float x0 = y[0], x1 = y[1], x2 = y[2], x3 = y[3];
+                    y[0] = rotate_first(x0, x1, cs[0], cs[1]);
+                    y[1] = rotate_second(x0, x1, cs[0], cs[1]);
+                    y[2] = rotate_first(x2, x3, cs[2], cs[3]);
+                    y[3] = rotate_second(x2, x3, cs[2], cs[3]);
+                }
+                // y[0], y[2] are neighbours in dim (dim[0], dim[0] + 1) when rotated, and so are y[1], y[3]
+                bf16x2 low, high;
+                if (rotate) {
+                    low[0] = static_cast<__bf16>(y[0]); low[1] = static_cast<__bf16>(y[2]);
+                    high[0] = static_cast<__bf16>(y[1]); high[1] = static_cast<__bf16>(y[3]);
+                } else {
+                    low[0] = static_cast<__bf16>(y[0]); low[1] = static_cast<__bf16>(y[1]);
+                    high[0] = static_cast<__bf16>(y[2]); high[1] = static_cast<__bf16>(y[3]);
+                }
+                const int low_dim = dim[0], high_dim = rotate ? dim[1] : dim[2];
+                if (is_query) {
+                    bf16* q_row = static_cast<bf16*>(store.q_out) + (static_cast<int64_t>(row) * store.heads + head) * store.head_dim;
+                    *reinterpret_cast<bf16x2*>(q_row + low_dim) = low;
+                    *reinterpret_cast<bf16x2*>(q_row + high_dim) = high;
+                    continue;
+                }
+                if (!store.slot_mapping) continue;
+                const int slot = store.slot_mapping[row];
+                if (slot < 0) continue;
+                const int page = slot / store.page_size, offset = slot % store.page_size;
+                if (!is_value) {
+                    bf16* pages = static_cast<bf16*>(store.k_cache);        // two neighbouring dims are neighbours in a page of keys
+                    *reinterpret_cast<bf16x2*>(pages + layout.k_at(page, head - store.heads, offset, low_dim)) = low;
+                    *reinterpret_cast<bf16x2*>(pages + layout.k_at(page, head - store.heads, offset, high_dim)) = high;
+                } else {
+                    bf16* pages = static_cast<bf16*>(store.v_cache);        // and 8 elements apart in a page of values
+                    const int kv_head = head - store.heads - store.kv_heads;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) pages[layout.v_at(page, kv_head, offset, within + i)] = from_float<bf16>(y[i]);
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int mt = 0; mt < kWaveTilesM; ++mt) {
         const int row = m0 + wave_m * 128 + mt * 16 + col;
@@ -289,12 +365,13 @@ __global__ __launch_bounds__(kTiledThreads, 1) void gemm_tiled_kernel(const bf16
 }
 
 template <int EPILOGUE>
-static int launch_tiled(const void* a, const void* w_packed, void* out, int m, int n, int k, int splits, hipStream_t stream) {
+static int launch_tiled(const void* a, const void* w_packed, void* out, int m, int n, int k, int splits, hipStream_t stream,
+                        const MllQkvStore& store = MllQkvStore{}) {
     const int n_tiles = (n + 15) / 16, k_steps = k / 32;
     const int m_blocks = (m + kTileM - 1) / kTileM, n_blocks = (n + kTileN - 1) / kTileN;
     const dim3 grid(8 * ((m_blocks * n_blocks + 7) / 8), splits);
     gemm_tiled_kernel<EPILOGUE><<<grid, kTiledThreads, 0, stream>>>(static_cast<const bf16*>(a), static_cast<const bf16*>(w_packed),
-                                                            out, m, n, k, n_tiles, k_steps, m_blocks, n_blocks);
+                                                            out, m, n, k, n_tiles, k_steps, m_blocks, n_blocks, store);
     return check_launch("gemm_tiled");
 }
 
@@ -317,4 +394,23 @@ extern "C" int mll_gemm_tiled(const void* a, const void* w_packed, void* out, in
         case 2: return launch_tiled<2>(a, w_packed, out, m, n, k, splits, stream);
         default: return fail("gemm_tiled: unknown epilogue");
     }
+}
+
+extern "C" int mll_gemm_tiled_qkv(const void* a, const void* w_packed, int m, int k, const MllQkvStore* store, hipStream_t stream) {
+    MLL_REQUIRE(store != nullptr, "gemm_tiled_qkv: no store");
+    MLL_REQUIRE(m >= 0 && k > 0 && k % 32 == 0, "gemm_tiled_qkv: k must be a positive multiple of 32");
+    MLL_REQUIRE(static_cast<int64_t>(kTileM) * k < (int64_t{1} << 30), "gemm_tiled_qkv: k is too long");
+    MLL_REQUIRE(store->heads > 0 && store->kv_heads >= 0 && store->head_dim > 0 && store->head_dim % 16 == 0,
+                "gemm_tiled_qkv: head_dim must be a multiple of 16");
+    MLL_REQUIRE(store->n_freq >= 0 && store->n_freq % 2 == 0 && 2 * store->n_freq <= store->head_dim,
+                "gemm_tiled_qkv: the number of rotary pairs must be even and at most head_dim / 2");
+    MLL_REQUIRE(store->n_freq == 0 || (store->cos_sin && reinterpret_cast<uintptr_t>(store->cos_sin) % 16 == 0),
+                "gemm_tiled_qkv: rotation needs a 16-byte aligned cos/sin table");
+    MLL_REQUIRE(store->q_out && reinterpret_cast<uintptr_t>(store->q_out) % 4 == 0, "gemm_tiled_qkv: no place for the queries");
+    MLL_REQUIRE(!store->slot_mapping || (store->k_cache && store->v_cache && store->page_size > 0 && store->page_size % 16 == 0),
+                "gemm_tiled_qkv: a slot mapping needs both caches and pages of a multiple of 16 positions");
+    MLL_REQUIRE(reinterpret_cast<uintptr_t>(a) % 16 == 0, "gemm_tiled_qkv: the activations must be 16-byte aligned");
+    if (m == 0) return 0;
+    const int n = (store->heads + 2 * store->kv_heads) * store->head_dim;
+    return launch_tiled<3>(a, w_packed, nullptr, m, n, k, 1, stream, *store);
 }

@@ -166,6 +166,10 @@ int mll_gemm_medium(const void* a, const void* w_packed, void* out, int epilogue
 // order alone.
 int mll_gemm_tiled(const void* a, const void* w_packed, void* out, int epilogue, int m, int n, int k,
                    int splits, hipStream_t stream);
+// Queries, keys and values of many rows: the tiled product finished as mll_gemm_skinny_qkv finishes its own (the
+// same MllQkvStore, the weight in rotary pair order). k a multiple of 32, store->n_freq even, no rows' factors; a
+// workgroup owns a 256 x 256 tile of the result and the reduction is never taken in parts.
+int mll_gemm_tiled_qkv(const void* a, const void* w_packed, int m, int k, const MllQkvStore* store, hipStream_t stream);
 
 // Calibration: a kernel that reads `bytes` of memory once with `blocks` workgroups, and one in which every wave of
 // `blocks` workgroups of 4 issues iterations * 16 independent v_mfma_f32_16x16x32_bf16 (16384 flops each). The caller

@@ -883,6 +883,43 @@ def gemm_tiled(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f
     return out
 
 
+def gemm_tiled_qkv(x: torch.Tensor, packed: torch.Tensor, bias: Optional[torch.Tensor],
+                   slot_mapping: Optional[torch.Tensor], cos_sin: Optional[torch.Tensor],
+                   k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                   heads: int, kv_heads: int, head_dim: int, page_size: int) -> torch.Tensor:
+    """Queries, keys and values of many bfloat16 rows in one kernel: ``gemm_tiled`` finished by the work of
+    ``qkv_rope_store`` (arguments as ``gemm_skinny_qkv``'s; ``k`` a multiple of 32 and an even number of rotary
+    pairs). The reduction is not taken in parts, so this pays where ``tiled_splits`` is 1. Returns the queries."""
+    lib = library.load()
+    _device_tensor(x, "gemm input", torch.bfloat16)
+    _device_tensor(packed, "packed weight", torch.bfloat16)
+    _need(x.dim() == 2, "gemm_tiled_qkv takes [m, k] activations")
+    m, k = x.shape
+    total = (heads + 2 * kv_heads) * head_dim
+    _need(k % 32 == 0 and head_dim % 16 == 0, "gemm_tiled_qkv needs k % 32 == 0 and head_dim % 16 == 0")
+    _need(packed.dim() == 5 and tuple(packed.shape[2:]) == (4, 16, 8) and packed.shape[0] == total // 16
+          and packed.shape[1] == k // 32, "the packed weight does not fit the heads and k")
+    if bias is not None:
+        _device_tensor(bias, "qkv bias", torch.float32)
+        _need(tuple(bias.shape) == (total,), "qkv bias has the wrong size")
+    n_freq = 0
+    if cos_sin is not None:
+        _device_tensor(cos_sin, "cos/sin table", torch.float32)
+        _need(cos_sin.dim() == 3 and cos_sin.shape[0] == m and cos_sin.shape[2] == 2, "the cos/sin table must be [rows, n_freq, 2]")
+        n_freq = cos_sin.shape[1]
+        _need(2 * n_freq <= head_dim and n_freq % 2 == 0, "gemm_tiled_qkv takes an even number of rotary pairs, at most head_dim / 2")
+    if slot_mapping is not None:
+        _device_tensor(slot_mapping, "slot mapping", torch.int32)
+        _need(tuple(slot_mapping.shape) == (m,), "slot mapping must hold one entry per token")
+        _need(k_cache is not None and v_cache is not None, "slot mapping needs both caches")
+        _check_pages(k_cache, v_cache, torch.bfloat16, kv_heads, head_dim, page_size)
+    q_out = torch.empty((m, heads * head_dim), dtype=torch.bfloat16, device=x.device)
+    store = _QkvStore(_ptr(bias), _ptr(slot_mapping), _ptr(cos_sin), n_freq, _ptr(q_out),
+                      _ptr(k_cache), _ptr(v_cache), heads, kv_heads, head_dim, page_size)
+    _check(lib.mll_gemm_tiled_qkv(_ptr(x), _ptr(packed), m, k, ctypes.byref(store), _stream()), lib)
+    return q_out
+
+
 def measured_peaks(device: Optional[torch.device] = None, read_bytes: int = 4 << 30) -> dict:
     """What this GPU reaches on a kernel that only reads memory once and on one that only issues bfloat16 MFMAs:
     ``{"hbm_read_GBps": ..., "mfma_bf16_TFLOPs": ...}`` (the best of a few launches each; well under a second)."""

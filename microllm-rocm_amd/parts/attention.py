@@ -18,7 +18,7 @@ import torch
 
 from ..ops import kernels
 from .base import MATRIX, Mixer, PagedKVNeed, Runtime, TensorDecl, VECTOR
-from .linear import SKINNY_ROWS, UnscaledRows, Weight, linear, linear_into_stream, takes_packed, takes_unscaled
+from .linear import MEDIUM_ROWS, SKINNY_ROWS, UnscaledRows, Weight, linear, linear_into_stream, takes_packed, takes_unscaled
 from .registry import build_part, register_part
 from .spec import PartSpec
 
@@ -134,6 +134,15 @@ class PagedAttention(Mixer):
     def takes_unscaled(self, rows: int) -> bool:
         return self.qkv_weight.row_order is not None and takes_unscaled(self.qkv_weight, rows)
 
+    @staticmethod
+    def _tiled_whole(weight: Weight, rows: int, cos_sin) -> bool:
+        """Whether the tiled product with the q/k/v epilogue takes these rows: only the packed copy is kept, the
+        rows are a prompt's, and the product's tiles fill the GPU without taking the reduction in parts (partial
+        sums cannot be rotated and stored by the workgroup that made them)."""
+        return (weight.tensor is None and rows > MEDIUM_ROWS and weight.in_features % 32 == 0
+                and (cos_sin is None or cos_sin.shape[1] % 2 == 0)
+                and kernels.tiled_splits(rows, weight.out_features, weight.in_features) == 1)
+
     def forward(self, x, ctx, cache, residual=None):
         view = ctx.paged[cache.group]
         scale = None
@@ -152,6 +161,9 @@ class PagedAttention(Mixer):
         if pair_order and x.shape[0] <= SKINNY_ROWS:
             q = kernels.gemm_skinny_qkv(x, weight.packed, bias, slot_mapping, cos_sin, k_pages, v_pages,
                                         self.heads, stored_heads, self.head_dim, view.page_size, scale=scale)
+        elif pair_order and scale is None and self._tiled_whole(weight, x.shape[0], cos_sin):
+            q = kernels.gemm_tiled_qkv(x, weight.packed, bias, slot_mapping, cos_sin, k_pages, v_pages,
+                                       self.heads, stored_heads, self.head_dim, view.page_size)
         else:
             if scale is not None:
                 raise TypeError("rows without their factors reached a q/k/v product that cannot apply them")

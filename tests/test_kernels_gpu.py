@@ -753,6 +753,81 @@ def test_gemm_tiled(m, n, k):
         ka.gemm_tiled(a[:, :k - 8].contiguous(), ka.pack_weight(w[:, :k - 8].contiguous()), n)
 
 
+@pytest.mark.parametrize("m", [65, 300, 600])
+@pytest.mark.parametrize("heads,kv_heads,hd,rotary,hidden,bias", [(4, 2, 16, 16, 64, True), (3, 1, 32, 32, 96, True), (28, 4, 128, 128, 512, True),
+                                                                   (5, 5, 48, 24, 160, False), (2, 0, 64, 64, 96, True), (7, 1, 80, 0, 32, True)])
+def test_gemm_tiled_qkv_is_product_then_rope_store(m, heads, kv_heads, hd, rotary, hidden, bias):
+    """The tiled product's q/k/v epilogue: against float64 numpy (bias, split-half rotation, pages read back), and
+    the same bits as the two kernels it replaces. Rows past a tile's edge, slots of -1 and pages filled before
+    show what is written where it should not be."""
+    rng = np.random.default_rng(m + heads)
+    ka = kernels()
+    total = (heads + 2 * kv_heads) * hd
+    theta = 1e4
+    x_ref, x = to_bf16_exact(rng.normal(size=(m, hidden)))
+    w_ref, w = to_bf16_exact(rng.normal(size=(total, hidden)) * 0.2)
+    b_ref = rng.normal(size=total).astype(np.float32) if bias else None
+    b = torch.from_numpy(b_ref).to(DEVICE) if bias else None
+    inv_freq = torch.from_numpy(theta ** -(np.arange(0, rotary, 2) / rotary)).to(DEVICE) if rotary else None
+    positions_host = rng.integers(0, 30000, size=m).astype(np.int32)
+    positions = torch.from_numpy(positions_host).to(DEVICE)
+    page_size = 32
+    n_pages = -(-m // page_size) + 2
+    slots_host = rng.permutation(page_size * n_pages)[:m].astype(np.int32)
+    slots_host[[3, m - 1]] = -1
+    slots = torch.from_numpy(slots_host).to(DEVICE) if kv_heads else None
+
+    def pages():
+        if not kv_heads:
+            return None, None
+        return (torch.full(key_page_shape(n_pages, kv_heads, page_size, hd), 7.0, dtype=torch.bfloat16, device=DEVICE),
+                torch.full(value_page_shape(n_pages, kv_heads, page_size, hd), 7.0, dtype=torch.bfloat16, device=DEVICE))
+
+    order = ka.rotary_pair_order(heads, kv_heads, hd, rotary // 2)
+    packed = ka.pack_weight(w, row_order=order)
+    table = ka.rope_table(positions, inv_freq) if rotary else None
+    k_one, v_one = pages()
+    q_one = ka.gemm_tiled_qkv(x, packed, b, slots, table, k_one, v_one, heads, kv_heads, hd, page_size)
+    assert q_one.shape == (m, heads * hd) and q_one.dtype == torch.bfloat16
+
+    q_ref, k_ref, v_ref = reference_qkv(x_ref @ w_ref.T, None if b_ref is None else b_ref.astype(np.float64), positions_host,
+                                        theta, heads, kv_heads, hd, rotary)
+    tol = dict(rtol=8e-3, atol=8e-3)
+    np.testing.assert_allclose(q_one.float().cpu().numpy().reshape(m, heads, hd), q_ref, **tol)
+    if kv_heads:
+        k_host = key_rows(k_one, hd).float().cpu().numpy()        # [page, kv_head, position, dim]
+        v_host = value_rows(v_one, hd).float().cpu().numpy()
+        written = np.zeros((n_pages, page_size), dtype=bool)
+        for token, slot in enumerate(slots_host):
+            if slot < 0:
+                continue
+            page, offset = divmod(int(slot), page_size)
+            written[page, offset] = True
+            np.testing.assert_allclose(k_host[page, :, offset, :], k_ref[token], **tol)
+            np.testing.assert_allclose(v_host[page, :, offset, :], v_ref[token], **tol)
+        assert np.all(k_host.transpose(0, 2, 1, 3)[~written] == 7.0) and np.all(v_host.transpose(0, 2, 1, 3)[~written] == 7.0)
+
+    k_two, v_two = pages()
+    q_two = ka.qkv_rope_store(ka.gemm_tiled(x, packed, total, "f32"), b, positions, slots, None, k_two, v_two,
+                              heads, kv_heads, hd, page_size, torch.bfloat16, pair_order=True, cos_sin=table)
+    assert torch.equal(q_one, q_two)
+    if kv_heads:
+        assert torch.equal(k_one, k_two) and torch.equal(v_one, v_two)
+
+
+def test_gemm_tiled_qkv_refuses_what_it_cannot_do():
+    ka = kernels()
+    x = torch.zeros((70, 40), dtype=torch.bfloat16, device=DEVICE)
+    w = torch.zeros((2 * 16, 40), dtype=torch.bfloat16, device=DEVICE)
+    with pytest.raises(Exception, match="k % 32"):
+        ka.gemm_tiled_qkv(x, ka.pack_weight(w), None, None, None, None, None, 2, 0, 16, 16)
+    x = torch.zeros((70, 64), dtype=torch.bfloat16, device=DEVICE)
+    w = torch.zeros((2 * 48, 64), dtype=torch.bfloat16, device=DEVICE)
+    odd = torch.zeros((70, 3, 2), dtype=torch.float32, device=DEVICE)       # three rotary pairs
+    with pytest.raises(Exception, match="even number of rotary pairs"):
+        ka.gemm_tiled_qkv(x, ka.pack_weight(w), None, None, odd, None, None, 2, 0, 48, 16)
+
+
 @pytest.mark.parametrize("m,width,k", [(20, 203, 96), (64, 176, 64), (33, 1000, 520)])
 def test_gemm_medium_gated_epilogue(m, width, k):
     rng = np.random.default_rng(width + 1)
