@@ -164,12 +164,16 @@ int mll_gemm_medium(const void* a, const void* w_packed, void* out, int epilogue
 // mll_gemm_skinny. With epilogue 0, `splits` > 1 deals the stages of 64 of k to that many workgroups per tile:
 // out is then [splits, m, n] partial sums for the caller to add in order. For weights that are kept in the packed
 // order alone.
+// tile_rows: the rows of a workgroup's tile of the result, 256, 192, 160 or 128, or 0 for mll_tiled_tile_rows's
+// choice; the result's bits do not depend on it.
 int mll_gemm_tiled(const void* a, const void* w_packed, void* out, int epilogue, int m, int n, int k,
-                   int splits, hipStream_t stream);
+                   int splits, int tile_rows, hipStream_t stream);
+int mll_tiled_tile_rows(int m, int n, int splits);
 // Queries, keys and values of many rows: the tiled product finished as mll_gemm_skinny_qkv finishes its own (the
 // same MllQkvStore, the weight in rotary pair order). k a multiple of 32, store->n_freq even, no rows' factors; a
-// workgroup owns a 256 x 256 tile of the result and the reduction is never taken in parts.
-int mll_gemm_tiled_qkv(const void* a, const void* w_packed, int m, int k, const MllQkvStore* store, hipStream_t stream);
+// workgroup owns a whole tile of the result and the reduction is never taken in parts.
+int mll_gemm_tiled_qkv(const void* a, const void* w_packed, int m, int k, const MllQkvStore* store, int tile_rows,
+                       hipStream_t stream);
 
 // Calibration: a kernel that reads `bytes` of memory once with `blocks` workgroups, and one in which every wave of
 // `blocks` workgroups of 4 issues iterations * 16 independent v_mfma_f32_16x16x32_bf16 (16384 flops each). The caller

@@ -841,7 +841,8 @@ def gemm_medium(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "
     return out
 
 
-TILED_TILE = 256            # gemm_tiled works in tiles of 256 x 256, stages of 64 of the reduction
+TILED_TILE = 256            # gemm_tiled works in tiles of up to 256 x 256, stages of 64 of the reduction
+COMPUTE_UNITS = 256         # of an MI355X: a workgroup of gemm_tiled has one to itself
 TILED_SPLIT_STAGES = 8      # a part of the reduction keeps at least this many stages
 
 
@@ -856,7 +857,22 @@ def tiled_splits(m: int, n: int, k: int) -> int:
     return splits
 
 
-def gemm_tiled(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f32", splits: int = 1) -> torch.Tensor:
+def tiled_tile_rows(m: int, n: int, splits: int = 1) -> int:
+    """The rows of a workgroup's tile that ``gemm_tiled`` chooses for this product: 256, or fewer where that fills
+    the compute units better. The result's bits do not depend on it."""
+    return int(library.load().mll_tiled_tile_rows(m, n, splits))
+
+
+def tiled_fill(m: int, n: int, splits: int = 1) -> float:
+    """How much of the compute units' time ``gemm_tiled``'s workgroups fill for this product: workgroups over the
+    places of the rounds of ``COMPUTE_UNITS`` they take (0.91 for 2048 x 4608 in tiles of 160 rows, 0.56 in tiles
+    of 256)."""
+    blocks = -(-m // tiled_tile_rows(m, n, splits)) * -(-n // TILED_TILE) * splits
+    return blocks / (-(-blocks // COMPUTE_UNITS) * COMPUTE_UNITS)
+
+
+def gemm_tiled(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f32", splits: int = 1,
+               tile_rows: int = 0) -> torch.Tensor:
     """``x @ W.T`` for many bfloat16 rows and a packed weight, on this package's tiled MFMA kernel (0.9 to 1.1 of
     the library's untuned rate at 2048 rows and more, 1.1 to 1.4 PFLOP/s: for weights that are kept in the packed
     order alone). ``k`` must be
@@ -879,14 +895,14 @@ def gemm_tiled(x: torch.Tensor, packed: torch.Tensor, n: int, epilogue: str = "f
         code, out = 2, torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
     else:
         raise KernelLibraryError(f"unknown epilogue {epilogue!r}")
-    _check(lib.mll_gemm_tiled(_ptr(x), _ptr(packed), _ptr(out), code, m, n, k, splits, _stream()), lib)
+    _check(lib.mll_gemm_tiled(_ptr(x), _ptr(packed), _ptr(out), code, m, n, k, splits, tile_rows, _stream()), lib)
     return out
 
 
 def gemm_tiled_qkv(x: torch.Tensor, packed: torch.Tensor, bias: Optional[torch.Tensor],
                    slot_mapping: Optional[torch.Tensor], cos_sin: Optional[torch.Tensor],
                    k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                   heads: int, kv_heads: int, head_dim: int, page_size: int) -> torch.Tensor:
+                   heads: int, kv_heads: int, head_dim: int, page_size: int, tile_rows: int = 0) -> torch.Tensor:
     """Queries, keys and values of many bfloat16 rows in one kernel: ``gemm_tiled`` finished by the work of
     ``qkv_rope_store`` (arguments as ``gemm_skinny_qkv``'s; ``k`` a multiple of 32 and an even number of rotary
     pairs). The reduction is not taken in parts, so this pays where ``tiled_splits`` is 1. Returns the queries."""
@@ -916,7 +932,7 @@ def gemm_tiled_qkv(x: torch.Tensor, packed: torch.Tensor, bias: Optional[torch.T
     q_out = torch.empty((m, heads * head_dim), dtype=torch.bfloat16, device=x.device)
     store = _QkvStore(_ptr(bias), _ptr(slot_mapping), _ptr(cos_sin), n_freq, _ptr(q_out),
                       _ptr(k_cache), _ptr(v_cache), heads, kv_heads, head_dim, page_size)
-    _check(lib.mll_gemm_tiled_qkv(_ptr(x), _ptr(packed), m, k, ctypes.byref(store), _stream()), lib)
+    _check(lib.mll_gemm_tiled_qkv(_ptr(x), _ptr(packed), m, k, ctypes.byref(store), tile_rows, _stream()), lib)
     return q_out
 
 

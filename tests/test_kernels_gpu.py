@@ -749,6 +749,14 @@ def test_gemm_tiled(m, n, k):
     # the same in every run, and a row's result does not depend on the other rows of the call
     assert torch.equal(ka.gemm_tiled(a, packed, n, "f32"), full)
     assert torch.equal(ka.gemm_tiled(a[m - 70:].contiguous(), packed, n, "f32"), full[m - 70:]) if m > 70 else True
+    # nor on how many rows a workgroup's tile has
+    assert ka.tiled_tile_rows(m, n) in (256, 192, 160, 128)
+    for tile_rows in (256, 192, 160, 128):
+        assert torch.equal(ka.gemm_tiled(a, packed, n, "f32", tile_rows=tile_rows), full), tile_rows
+        assert torch.equal(ka.gemm_tiled(a, packed, n, "bf16", tile_rows=tile_rows), out), tile_rows
+        assert torch.equal(ka.gemm_tiled(a, packed, n, "f32", splits=3, tile_rows=tile_rows), ka.gemm_tiled(a, packed, n, "f32", splits=3))
+    with pytest.raises(Exception, match="256, 192, 160 or 128"):
+        ka.gemm_tiled(a, packed, n, "f32", tile_rows=64)
     with pytest.raises(Exception, match="multiple of 32"):
         ka.gemm_tiled(a[:, :k - 8].contiguous(), ka.pack_weight(w[:, :k - 8].contiguous()), n)
 
@@ -813,6 +821,20 @@ def test_gemm_tiled_qkv_is_product_then_rope_store(m, heads, kv_heads, hd, rotar
     assert torch.equal(q_one, q_two)
     if kv_heads:
         assert torch.equal(k_one, k_two) and torch.equal(v_one, v_two)
+    for tile_rows in (256, 192, 160, 128):
+        k_three, v_three = pages()
+        q_three = ka.gemm_tiled_qkv(x, packed, b, slots, table, k_three, v_three, heads, kv_heads, hd, page_size, tile_rows=tile_rows)
+        assert torch.equal(q_three, q_one), tile_rows
+        if kv_heads:
+            assert torch.equal(k_three, k_one) and torch.equal(v_three, v_one), tile_rows
+
+
+def test_tiles_of_fewer_rows_where_they_fill_the_compute_units():
+    ka = kernels()
+    assert ka.tiled_tile_rows(2048, 4608) == 160       # 144 tiles of 256 rows, 234 of 160
+    assert ka.tiled_tile_rows(2048, 37888) == 256      # many rounds either way: the tile that loads least a product
+    assert ka.tiled_tile_rows(2048, 3584, 2) == 256    # 224 workgroups in one round
+    assert ka.tiled_tile_rows(100, 512) == 128         # one round whatever the height: the cheapest tile
 
 
 def test_gemm_tiled_qkv_refuses_what_it_cannot_do():
