@@ -25,36 +25,58 @@ def _fill_random(engine: Engine) -> None:
                 tensor.normal_(0.0, 1.0)
 
 
-def decode_throughput(engine: Engine, batch: int, context: int, steps: int, warmup: int, seed: int = 0) -> Dict[str, float]:
-    """``batch`` requests that each hold ``context`` positions decode ``warmup + steps`` tokens, greedily."""
+def decode_throughput(engine: Engine, batch: int, context: int, steps: int, warmup: int, seed: int = 0,
+                      lookahead: bool = True) -> Dict[str, float]:
+    """``batch`` requests that each hold ``context`` positions decode ``warmup + steps`` tokens, greedily.
+
+    With ``lookahead`` the loop is generation's (``Scheduler(lookahead=True)``): a step takes its tokens from the
+    ids that the step before chose on the device, and the host reads a step's ids while the next one runs. Without
+    it the host waits for every step's ids before it builds the next step."""
     rng = np.random.default_rng(seed)
     sampler = Sampler()
     params = [SamplingParams(temperature=0.0)] * batch
+    draws = [0] * batch
     ids = [("bench", batch, index) for index in range(batch)]
     for request_id in ids:
         request = engine.open(request_id)
         engine.cache.reserve(request, context)
         engine.cache.commit(request, context)
     _fill_random(engine)
-    tokens = rng.integers(0, engine.spec.vocab_size, size=batch).tolist()
+    first = rng.integers(0, engine.spec.vocab_size, size=batch).tolist()
 
     def one_step(current):
         logits = engine.step([StepEntry(request_id, [token], [0]) for request_id, token in zip(ids, current)], borrow_logits=True)
-        return sampler.select(logits, params, [0] * batch)
+        return sampler.select(logits, params, draws)
+
+    def one_step_ahead(before):
+        """Launches the step after ``before`` (a Selection; None: the first step), then learns ``before``'s ids."""
+        if before is None:
+            logits = engine.step([StepEntry(request_id, [token], [0]) for request_id, token in zip(ids, first)], borrow_logits=True)
+        else:
+            entries = [StepEntry(request_id, [0], [0], token_from=row) for row, request_id in enumerate(ids)]
+            logits = engine.step(entries, borrow_logits=True, device_tokens=before.device)
+        selection = sampler.select_later(logits, params, draws)
+        if before is not None:
+            before.tokens()
+        return selection
+
+    def run(count, state):
+        for _ in range(count):
+            state = one_step_ahead(state) if lookahead else one_step(state)
+        return state
 
     try:
-        for _ in range(warmup):
-            tokens = one_step(tokens)
+        state = run(warmup, None if lookahead else first)
         torch.cuda.synchronize()
         started = time.perf_counter()
-        for _ in range(steps):
-            tokens = one_step(tokens)
+        state = run(steps, state)
+        last = state.tokens() if lookahead else state
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - started
     finally:
         for request_id in ids:
             engine.close(request_id)
-    return {"tokens_per_second": batch * steps / elapsed, "ms_per_step": elapsed / steps * 1e3}
+    return {"tokens_per_second": batch * steps / elapsed, "ms_per_step": elapsed / steps * 1e3, "last_tokens": list(last)}
 
 
 def prefill_throughput(engine: Engine, tokens: int, repeats: int = 3, seed: int = 0) -> Dict[str, float]:

@@ -554,3 +554,21 @@ def test_lookahead_generates_the_same_tokens(tmp_path, dtype):
         assert all(token >= 0 for output in ahead for token in output)
         engine.cache.check()
         assert not engine.cache.requests
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_timed_decode_loop_gives_the_same_tokens_with_and_without_lookahead(tmp_path, dtype):
+    """The benchmark's decode loop, which takes a step's tokens from the ids that the step before left on the
+    device, decodes what the loop that waits for every step's ids decodes, and leaves the cache as it found it."""
+    from microllm_rocm_amd.engine.benchmark import decode_throughput
+    folder = make_folder(tmp_path, "A", SHARP)
+    results = []
+    for lookahead, warmup in ((False, 2), (True, 2), (True, 0), (False, 0)):
+        engine = engine_for(folder, dtype, max_tokens=4 * 128, max_requests=4)      # the same pages for the same requests
+        torch.manual_seed(5)       # the caches are filled with random keys and values
+        results.append(decode_throughput(engine, 3, 40, steps=9, warmup=warmup, seed=1, lookahead=lookahead))
+        engine.cache.check()
+        assert not engine.cache.requests
+    assert results[0]["last_tokens"] == results[1]["last_tokens"] and len(results[0]["last_tokens"]) == 3
+    assert results[2]["last_tokens"] == results[3]["last_tokens"]
+    assert all(result["tokens_per_second"] > 0 for result in results)
