@@ -19,10 +19,10 @@ namespace mll {
 
 constexpr int kRowwiseMaxHeadDim = 512;
 constexpr int kRowwiseChunk = 128;      // keys; a multiple of the tiles of 64
-// Rows of (token, wave's heads) a step must still have when a wave takes several query heads of a kv head: 64, e.g. 16
-// requests of 4 kv heads (measured at 7B sizes and 4096 keys: 16 requests 159 -> 146 us, 64 requests 544 -> 413; 8
-// requests 89 -> 130). mll_rowwise_heads_from sets it: tests force either way with it.
-static int64_t grouped_from_rows = 64;
+// How many query heads of a kv head a wave takes in the float32 kernels: 0 lets the launch choose by how many waves
+// the step then still has (rowwise_heads_a_wave); tests and measurements force 1 to 8 with mll_rowwise_heads_a_wave.
+static int forced_heads_a_wave = 0;
+constexpr int64_t kRowwiseWavesWanted = 4096;      // four a SIMD: fewer leave the loads' latency in the open
 
 __device__ inline void load_eight(const float* from, float (&to)[8]) {
     const float4 low = *reinterpret_cast<const float4*>(from);
@@ -236,9 +236,11 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_heads_kernel(
     const int token = blockIdx.x;
     const int lane = threadIdx.x;
     const int group = heads / kv_heads;
-    const int waves_of_group = group / GW;                       // GW divides the group
+    const int waves_of_group = (group + GW - 1) / GW;            // the group's last wave may have fewer heads
     const int kv_head = blockIdx.y / waves_of_group;
-    const int first_head = kv_head * group + (blockIdx.y % waves_of_group) * GW;
+    const int first_in_group = (blockIdx.y % waves_of_group) * GW;
+    const int first_head = kv_head * group + first_in_group;
+    const int heads_here = min(GW, group - first_in_group);      // heads past them repeat the last one and write nothing
     const int seq = seq_of_token[token];
     if (seq < 0) return;
     const int position = positions[token];
@@ -248,7 +250,7 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_heads_kernel(
     const int32_t* table = block_table + static_cast<int64_t>(seq) * table_width;
 #pragma unroll
     for (int g = 0; g < GW; ++g) {
-        const T* q_row = q + (static_cast<int64_t>(token) * heads + first_head + g) * head_dim;
+        const T* q_row = q + (static_cast<int64_t>(token) * heads + first_head + min(g, heads_here - 1)) * head_dim;
         for (int d = lane; d < head_dim; d += kWave) q_shared[g][d] = to_float(q_row[d]);
     }
     __syncthreads();
@@ -278,6 +280,7 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_heads_kernel(
             v_place = v_tile + ((offset % 16) / 8) * 256;
             v_place_last = v_tile + ((offset % 16) / 8) * 128;
             const int whole = head_dim / 8 * 8;
+#pragma unroll 4
             for (int d = 0; d < whole; d += 8) {
                 float k[8];
                 load_eight(k_tile + (d / 8) * 128, k);
@@ -340,6 +343,7 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_heads_kernel(
         attend(max(low, chunk * kRowwiseChunk), min(position, chunk * kRowwiseChunk + kRowwiseChunk - 1));
 #pragma unroll
         for (int g = 0; g < GW; ++g) {
+            if (g >= heads_here) break;
             const int64_t slot = (static_cast<int64_t>(token) * heads + first_head + g) * max_chunks + blockIdx.z;
 #pragma unroll
             for (int i = 0; i < DIMS; ++i) {
@@ -375,6 +379,7 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_heads_kernel(
     }
 #pragma unroll
     for (int g = 0; g < GW; ++g) {
+        if (g >= heads_here) break;
         T* out_row = out + (static_cast<int64_t>(token) * heads + first_head + g) * head_dim;
         const float inverse = 1.0f / total_sum[g];
 #pragma unroll
@@ -385,10 +390,17 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_heads_kernel(
     }
 }
 
-// The most query heads of a kv head that one wave of the kernel above takes: the largest divisor of the group up to 8.
-static int heads_a_wave(int group) {
-    for (int count = group < 8 ? group : 8; count >= 2; --count)
-        if (group % count == 0) return count;
+// How many query heads of a kv head one wave of the kernel above takes in a step of `rows` (token, kv head, chunk)
+// items: as many as leave the GPU its waves, of the counts that fill the group's waves evenly (7 heads: 7, or 4
+// and 3, or 2, 2, 2 and 1; not 5 and 2). One: the kernel for one head a wave.
+static int rowwise_heads_a_wave(int group, int64_t rows) {
+    const int most = group < 8 ? group : 8;
+    if (forced_heads_a_wave > 0) return forced_heads_a_wave < most ? forced_heads_a_wave : most;
+    for (int count = most; count >= 2; --count) {
+        const int waves = (group + count - 1) / count;
+        if (waves * count - group > 1) continue;      // the group's last wave would have much less than the others
+        if (rows * waves >= kRowwiseWavesWanted) return count;
+    }
     return 1;
 }
 
@@ -409,18 +421,32 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_merge_kernel(
 #pragma unroll
     for (int i = 0; i < DIMS; ++i) total[i] = 0.0f;
     float total_max = -INFINITY, total_sum = 0.0f;
-    for (int slot = 0; slot < chunks; ++slot) {
-        const float chunk_max = part_ml[(first_slot + slot) * 2];
-        const float chunk_sum = part_ml[(first_slot + slot) * 2 + 1];
-        float new_max, keep, add;
-        merge_scales(total_max, chunk_max, new_max, keep, add);
-        total_sum = merged(total_sum, keep, chunk_sum, add);
+    // Eight chunks' results are asked for at once and then merged one after the other: the loads of a chunk do not
+    // wait for the merge of the chunk before.
+    constexpr int kAtOnce = 8;
+    for (int base = 0; base < chunks; base += kAtOnce) {
+        float chunk_max[kAtOnce], chunk_sum[kAtOnce], chunk_o[kAtOnce][DIMS];
 #pragma unroll
-        for (int i = 0; i < DIMS; ++i) {
-            const int d = lane + i * kWave;
-            if (d < head_dim) total[i] = merged(total[i], keep, part_o[(first_slot + slot) * head_dim + d], add);
+        for (int u = 0; u < kAtOnce; ++u) {
+            const int64_t slot = first_slot + min(base + u, chunks - 1);
+            chunk_max[u] = part_ml[slot * 2];
+            chunk_sum[u] = part_ml[slot * 2 + 1];
+#pragma unroll
+            for (int i = 0; i < DIMS; ++i) {
+                const int d = lane + i * kWave;
+                chunk_o[u][i] = d < head_dim ? part_o[slot * head_dim + d] : 0.0f;
+            }
         }
-        total_max = new_max;
+#pragma unroll
+        for (int u = 0; u < kAtOnce; ++u) {
+            if (base + u >= chunks) break;
+            float new_max, keep, add;
+            merge_scales(total_max, chunk_max[u], new_max, keep, add);
+            total_sum = merged(total_sum, keep, chunk_sum[u], add);
+#pragma unroll
+            for (int i = 0; i < DIMS; ++i) total[i] = merged(total[i], keep, chunk_o[u][i], add);
+            total_max = new_max;
+        }
     }
     T* out_row = out + (static_cast<int64_t>(token) * heads + head) * head_dim;
     const float inverse = 1.0f / total_sum;
@@ -434,10 +460,13 @@ __global__ __launch_bounds__(kWave) void paged_attention_rowwise_merge_kernel(
 template <typename T, int DIMS>
 static int launch_rowwise_dims(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
                           int table_width, const int32_t* seq_of_token, const int32_t* positions, void* out,
-                          float* part_o, float* part_ml, int max_chunks, float scale, int window, int n_tokens,
+                          float* part_o, float* part_ml, int max_chunks, int usual_chunks, float scale, int window, int n_tokens,
                           int heads, int kv_heads, int head_dim, int page_size, hipStream_t stream) {
-    const int gw = (std::is_same<T, float>::value && DIMS <= 2) ? heads_a_wave(heads / kv_heads) : 1;
-    const bool several_heads = gw >= 2 && static_cast<int64_t>(n_tokens) * (heads / gw) >= grouped_from_rows;
+    const int group = heads / kv_heads;
+    const int64_t rows = static_cast<int64_t>(n_tokens) * kv_heads * (max_chunks > 0 ? (usual_chunks > 0 ? usual_chunks : max_chunks) : 1);
+    const int gw = (std::is_same<T, float>::value && DIMS <= 2) ? rowwise_heads_a_wave(group, rows) : 1;
+    const bool several_heads = gw >= 2;
+    const int group_waves = kv_heads * ((group + gw - 1) / gw);
 #define MLL_ROWWISE_HEADS(MODE, GW)                                                                                    \
     case GW:                                                                                                           \
         paged_attention_rowwise_heads_kernel<T, MODE, DIMS, GW><<<heads_grid, kWave, 0, stream>>>(                      \
@@ -454,7 +483,7 @@ static int launch_rowwise_dims(const void* q, const void* k_cache, const void* v
     if (max_chunks == 0) {
         if constexpr (std::is_same<T, float>::value && DIMS <= 2) {
             if (several_heads) {
-                const dim3 heads_grid(n_tokens, heads / gw);
+                const dim3 heads_grid(n_tokens, group_waves);
                 MLL_ROWWISE_HEADS_ALL(0)
                 return check_launch("paged_attention_rowwise");
             }
@@ -471,7 +500,7 @@ static int launch_rowwise_dims(const void* q, const void* k_cache, const void* v
     if constexpr (std::is_same<T, float>::value && DIMS <= 2) {
         if (several_heads) {
             grouped = true;
-            const dim3 heads_grid(n_tokens, heads / gw, max_chunks);
+            const dim3 heads_grid(n_tokens, group_waves, max_chunks);
             MLL_ROWWISE_HEADS_ALL(1)
         }
     }
@@ -491,11 +520,11 @@ static int launch_rowwise_dims(const void* q, const void* k_cache, const void* v
 template <typename T>
 static int launch_rowwise(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
                           int table_width, const int32_t* seq_of_token, const int32_t* positions, void* out,
-                          float* part_o, float* part_ml, int max_chunks, float scale, int window, int n_tokens,
+                          float* part_o, float* part_ml, int max_chunks, int usual_chunks, float scale, int window, int n_tokens,
                           int heads, int kv_heads, int head_dim, int page_size, hipStream_t stream) {
 #define MLL_ROWWISE_DIMS(D)                                                                                            \
     return launch_rowwise_dims<T, D>(q, k_cache, v_cache, block_table, table_width, seq_of_token, positions, out, part_o, \
-                                     part_ml, max_chunks, scale, window, n_tokens, heads, kv_heads, head_dim, page_size, stream)
+                                     part_ml, max_chunks, usual_chunks, scale, window, n_tokens, heads, kv_heads, head_dim, page_size, stream)
     if (head_dim <= kWave) MLL_ROWWISE_DIMS(1);
     if (head_dim <= 2 * kWave) MLL_ROWWISE_DIMS(2);
     if (head_dim <= 4 * kWave) MLL_ROWWISE_DIMS(4);
@@ -509,22 +538,24 @@ using namespace mll;
 
 extern "C" int mll_paged_attention_rowwise_chunk() { return kRowwiseChunk; }
 
-// From how many rows (tokens x waves a token) on a step's chunked row-wise attention lets a wave take several query
-// heads of a kv head; returns the value before. Both ways give the same bits.
-extern "C" int64_t mll_rowwise_heads_from(int64_t rows) {
-    const int64_t before = mll::grouped_from_rows;
-    mll::grouped_from_rows = rows;
+// Forces how many query heads of a kv head a wave of the float32 kernels takes (1 to 8; more than the group has:
+// the group), or with 0 gives the choice back to the launch; returns the value before. Every count gives the same bits.
+extern "C" int mll_rowwise_heads_a_wave(int count) {
+    const int before = mll::forced_heads_a_wave;
+    mll::forced_heads_a_wave = count < 0 ? 0 : count;
     return before;
 }
 
 // max_chunks 0: one wave per (token, head). Otherwise one wave per chunk, for rows whose keys span at most
 // max_chunks chunks (the caller's promise: a row with more would lose its last ones), with part_o
 // [n_tokens * heads * max_chunks * head_dim] and part_ml [n_tokens * heads * max_chunks * 2] floats as workspace.
+// usual_chunks (0: max_chunks): how many chunks the step's rows have now, where max_chunks leaves room for later
+// steps of the same shape; only how many heads a wave takes follows from it.
 extern "C" int mll_paged_attention_rowwise(const void* q, int dtype, const void* k_cache, const void* v_cache,
                                            const int32_t* block_table, int table_width,
                                            const int32_t* seq_of_token, const int32_t* positions, void* out,
-                                           float* part_o, float* part_ml, int max_chunks, float scale, int window,
-                                           int n_tokens, int heads, int kv_heads, int head_dim, int page_size,
+                                           float* part_o, float* part_ml, int max_chunks, int usual_chunks, float scale,
+                                           int window, int n_tokens, int heads, int kv_heads, int head_dim, int page_size,
                                            hipStream_t stream) {
     MLL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "paged_attention: heads must divide into kv_heads groups");
     MLL_REQUIRE(head_dim > 0 && head_dim <= kRowwiseMaxHeadDim, "paged_attention: head_dim must be in [1, 512]");
@@ -536,9 +567,9 @@ extern "C" int mll_paged_attention_rowwise(const void* q, int dtype, const void*
     if (n_tokens == 0) return 0;
     if (dtype == kF32)
         return launch_rowwise<float>(q, k_cache, v_cache, block_table, table_width, seq_of_token, positions, out, part_o,
-                                     part_ml, max_chunks, scale, window, n_tokens, heads, kv_heads, head_dim, page_size, stream);
+                                     part_ml, max_chunks, usual_chunks, scale, window, n_tokens, heads, kv_heads, head_dim, page_size, stream);
     if (dtype == kBF16)
         return launch_rowwise<bf16>(q, k_cache, v_cache, block_table, table_width, seq_of_token, positions, out, part_o,
-                                    part_ml, max_chunks, scale, window, n_tokens, heads, kv_heads, head_dim, page_size, stream);
+                                    part_ml, max_chunks, usual_chunks, scale, window, n_tokens, heads, kv_heads, head_dim, page_size, stream);
     return fail("paged_attention: unknown dtype");
 }

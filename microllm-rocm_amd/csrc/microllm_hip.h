@@ -60,15 +60,17 @@ int mll_qkv_rope_store(const void* qkv, int in_dtype, int n_partials, int64_t pa
 // the same arithmetic (the same bits), for steps with few rows; no row's visible keys may then span more than
 // max_chunks chunks (chunks lie at absolute positions), and part_o [n_tokens * heads * max_chunks * head_dim]
 // and part_ml [n_tokens * heads * max_chunks * 2] floats are the workspace.
+// usual_chunks (0: max_chunks): how many chunks the rows have in this step, where max_chunks leaves room for later
+// steps of the same shape; it only decides how many heads a wave takes.
 int mll_paged_attention_rowwise_chunk();
-// In float32 with head sizes up to 128 a wave of the chunked kernel takes several query heads of a kv head (their
-// keys and values read once) from this many rows (tokens x waves a token) on; returns the value before. The same bits
-// either way.
-int64_t mll_rowwise_heads_from(int64_t rows);
+// In float32 with head sizes up to 128 a wave takes several query heads of a kv head (their keys and values read
+// once) where the step still has waves enough for the GPU that way. This forces the count (1 to 8; 0: the launch
+// chooses again) and returns the value before. The same bits whatever the count.
+int mll_rowwise_heads_a_wave(int count);
 int mll_paged_attention_rowwise(const void* q, int dtype, const void* k_cache, const void* v_cache,
                                 const int32_t* block_table, int table_width,
                                 const int32_t* seq_of_token, const int32_t* positions, void* out,
-                                float* part_o, float* part_ml, int max_chunks, float scale, int window,
+                                float* part_o, float* part_ml, int max_chunks, int usual_chunks, float scale, int window,
                                 int n_tokens, int heads, int kv_heads, int head_dim, int page_size,
                                 hipStream_t stream);
 

@@ -325,12 +325,11 @@ def _check_paged(q, k_cache, v_cache, block_table, heads, kv_heads, head_dim) ->
 ROWWISE_SPLIT_BELOW = 2048      # (token, head) rows: with fewer, a row's chunks of keys get a wave each
 
 
-def rowwise_heads_from(rows: int) -> int:
-    """From how many rows (tokens x waves a token) on the chunked row-wise attention lets one wave take several
-    query heads of a kv head (float32, head sizes up to 128); returns the value before. Both ways give the same bits."""
-    lib = library.load()
-    lib.mll_rowwise_heads_from.restype = ctypes.c_int64
-    return int(lib.mll_rowwise_heads_from(ctypes.c_int64(int(rows))))
+def rowwise_heads_a_wave(count: int) -> int:
+    """Forces how many query heads of a kv head one wave of the float32 row-wise attention takes (1 to 8; 0 gives
+    the choice back to the launch, which goes by the waves the step then has); returns the value before. Every
+    count gives the same bits."""
+    return int(library.load().mll_rowwise_heads_a_wave(int(count)))
 
 
 def rowwise_chunks(longest: int, window: int) -> int:
@@ -346,10 +345,12 @@ def paged_attention_rowwise(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
                             block_table: torch.Tensor, seq_of_token: torch.Tensor, positions: torch.Tensor,
                             scale: float, window: int, heads: int, kv_heads: int, head_dim: int,
                             out: Optional[torch.Tensor] = None, longest: Optional[int] = None,
-                            split: Optional[bool] = None) -> torch.Tensor:
+                            split: Optional[bool] = None, usual: Optional[int] = None) -> torch.Tensor:
     """The plain attention kernel (any dtype, any head size). ``longest``: no position of the step reaches it
     (default: what the block table can hold). ``split``: a wave per chunk of keys and a merge, or a wave per row;
-    by default by the number of rows. Both give the same bits."""
+    by default by the number of rows. Both give the same bits. ``usual``: how far the step's rows reach now
+    (default ``longest``, which may leave room for later steps of the same shape): how many query heads a wave
+    of the float32 kernel takes goes by it, nothing else."""
     lib = library.load()
     page_size = _check_paged(q, k_cache, v_cache, block_table, heads, kv_heads, head_dim)
     n_tokens = q.shape[0]
@@ -366,6 +367,7 @@ def paged_attention_rowwise(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     if split is None:
         split = n_tokens * heads < ROWWISE_SPLIT_BELOW
     chunks = rowwise_chunks(max(longest, 1), window) if split else 0
+    usual_chunks = rowwise_chunks(max(min(int(usual), longest), 1), window) if split and usual is not None else 0
     part_o = part_ml = None
     if chunks > 1:
         part_o = torch.empty((n_tokens, heads, chunks, head_dim), dtype=torch.float32, device=q.device)
@@ -374,7 +376,7 @@ def paged_attention_rowwise(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         chunks = 0      # one chunk a row: the wave per row is the wave per chunk
     _check(lib.mll_paged_attention_rowwise(_ptr(q), _code(q.dtype), _ptr(k_cache), _ptr(v_cache), _ptr(block_table),
                                            block_table.shape[1], _ptr(seq_of_token), _ptr(positions), _ptr(out),
-                                           _ptr(part_o), _ptr(part_ml), chunks, ctypes.c_float(scale), int(window),
+                                           _ptr(part_o), _ptr(part_ml), chunks, usual_chunks, ctypes.c_float(scale), int(window),
                                            n_tokens, heads, kv_heads, head_dim, page_size, _stream()), lib)
     return out
 
@@ -724,7 +726,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                    scale, window, heads, kv_heads, head_dim, splits, out=out, token_ids=plan.single_tokens)
         return out
     return paged_attention_rowwise(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
-                                   scale, window, heads, kv_heads, head_dim, longest=max(ctx.planned_total, ctx.max_total))
+                                   scale, window, heads, kv_heads, head_dim, longest=max(ctx.planned_total, ctx.max_total),
+                                   usual=ctx.max_total)
 
 
 def pack_weight(weight: torch.Tensor, interleave_halves: bool = False,

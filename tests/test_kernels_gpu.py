@@ -286,14 +286,16 @@ def test_rowwise_attention_a_wave_per_chunk_gives_the_same_bits(dtype, heads, kv
     by_chunk = k.paged_attention_rowwise(*args, split=True, longest=max(lengths))
     generous = k.paged_attention_rowwise(*args, split=True)      # as many chunks as the table is wide
     assert torch.equal(whole, by_chunk) and torch.equal(whole, generous)
-    # in float32 a wave of the chunked kernel may take several query heads of a kv head: forced, and forbidden
-    usual = k.rowwise_heads_from(1)
+    # in float32 a wave may take several query heads of a kv head, the group's last wave fewer: every count, forced
+    usual = k.rowwise_heads_a_wave(1)
+    several_heads, one_head = [], []
     try:
-        several_heads = [k.paged_attention_rowwise(*args, split=True, longest=max(lengths)), k.paged_attention_rowwise(*args, split=False)]
-        k.rowwise_heads_from(1 << 60)
         one_head = [k.paged_attention_rowwise(*args, split=True, longest=max(lengths)), k.paged_attention_rowwise(*args, split=False)]
+        for count in range(2, 9):
+            k.rowwise_heads_a_wave(count)
+            several_heads += [k.paged_attention_rowwise(*args, split=True, longest=max(lengths)), k.paged_attention_rowwise(*args, split=False)]
     finally:
-        k.rowwise_heads_from(usual)
+        k.rowwise_heads_a_wave(usual)
     assert all(torch.equal(whole, other) for other in several_heads + one_head)
     reference = reference_attention(q_exact, ek, ev, seq, pos, heads, kv_heads, hd, scale, window)
     np.testing.assert_allclose(whole.float().cpu().numpy(), reference, **tolerance(dtype))
