@@ -200,26 +200,29 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float* __rest
 // Where W has few rows the kernel above stays at 1.8 to 2.0 TB/s: a wave an element's worth of lanes is all the
 // parallelism there is, and its reads from LDS (512 KB for 16 KB of W) are what a compute unit can give; neither four
 // sums an element instead of one, nor two chunks in flight instead of one, nor reading LDS a batch ahead changes that.
-constexpr int kWideColumns = 32;
 constexpr int kWideThreads = 128;
 constexpr int kWideDepth = 128;                      // of k in a chunk
 constexpr int kWideQuads = kWideDepth / 4;           // float4 in a row of a chunk
-constexpr int kWideLoadsA = 16 * kWideQuads / kWideThreads;
-constexpr int kWideLoadsW = kWideColumns * kWideQuads / kWideThreads;
-constexpr int kWideFrom = 16384;                     // columns of C from which this kernel is taken: 512 workgroups
+constexpr int kWideFrom = 16384;                     // columns of C from which this kernel is taken whatever the parts
 
-template <bool VECTOR>
+// TR x TC elements a thread: rows r (+ 8), columns c, c + 16, ... of the workgroup's 8 TR rows and 16 TC columns. Per
+// four k a thread reads TR + TC times from LDS for 4 TR TC multiply-adds, and every element of W is read by 8 threads:
+// with 2 x 2 that is 16 reads an element of W, which is what bounds the kernel (4.1 TB/s of W for gate/up at 8 rows,
+// where half of the 16 rows are empty); 1 x 4 for at most 8 rows makes it 10 (4.8 TB/s; the head 4.95 -> 5.4).
+template <bool VECTOR, int TR, int TC>
 __global__ __launch_bounds__(kWideThreads) void gemm_f32_small_wide_kernel(const float* __restrict__ a, const float* __restrict__ w,
                                                                            const float* __restrict__ bias, float* __restrict__ c,
                                                                            int m, int n, int k, int k_split) {
     MLL_F32_SPLIT_RANGE
-    __shared__ __align__(16) float a_tile[16][kWideDepth + 4];
-    __shared__ __align__(16) float w_tile[kWideColumns][kWideDepth + 4];
-    const int col0 = blockIdx.x * kWideColumns;
-    const int column = threadIdx.x % 16;      // this thread's outputs: rows `row`, row + 8; columns col0 + `column`, + 16
+    constexpr int ROWS = 8 * TR, COLUMNS = 16 * TC;
+    constexpr int LOADS_A = ROWS * kWideQuads / kWideThreads, LOADS_W = COLUMNS * kWideQuads / kWideThreads;
+    __shared__ __align__(16) float a_tile[ROWS][kWideDepth + 4];
+    __shared__ __align__(16) float w_tile[COLUMNS][kWideDepth + 4];
+    const int col0 = blockIdx.x * COLUMNS;
+    const int column = threadIdx.x % 16;      // this thread's outputs: rows `row` (+ 8); columns col0 + `column` + 16 j
     const int row = threadIdx.x / 16;
-    // What a thread brings in of a chunk: float4 number threadIdx.x + j * 128 of the chunk's rows of A (16 rows of
-    // kWideQuads) and of W (32 rows).
+    // What a thread brings in of a chunk: float4 number threadIdx.x + j * 128 of the chunk's rows of A (ROWS rows of
+    // kWideQuads) and of W (COLUMNS rows).
     auto load4 = [&](const float* matrix, int rows, int first_row, int index, int k0) {
         const int r = index / kWideQuads, kk = k0 + (index % kWideQuads) * 4;
         const bool live = first_row + r < rows;
@@ -230,23 +233,27 @@ __global__ __launch_bounds__(kWideThreads) void gemm_f32_small_wide_kernel(const
         for (int e = 0; e < 4; ++e) v[e] = (live && kk + e < k) ? source[e] : 0.0f;
         return make_float4(v[0], v[1], v[2], v[3]);
     };
-    float4 a_next[kWideLoadsA], w_next[kWideLoadsW];
+    float4 a_next[LOADS_A], w_next[LOADS_W];
     auto fetch = [&](int k0) {
 #pragma unroll
-        for (int j = 0; j < kWideLoadsA; ++j) a_next[j] = load4(a, m, 0, threadIdx.x + j * kWideThreads, k0);
+        for (int j = 0; j < LOADS_A; ++j) a_next[j] = load4(a, m, 0, threadIdx.x + j * kWideThreads, k0);
 #pragma unroll
-        for (int j = 0; j < kWideLoadsW; ++j) w_next[j] = load4(w, n, col0, threadIdx.x + j * kWideThreads, k0);
+        for (int j = 0; j < LOADS_W; ++j) w_next[j] = load4(w, n, col0, threadIdx.x + j * kWideThreads, k0);
     };
-    float acc[2][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}};
+    float acc[TR][TC];
+#pragma unroll
+    for (int i = 0; i < TR; ++i)
+#pragma unroll
+        for (int j = 0; j < TC; ++j) acc[i][j] = 0.0f;
     fetch(k_lo);
     for (int k0 = k_lo; k0 < k; k0 += kWideDepth) {
 #pragma unroll
-        for (int j = 0; j < kWideLoadsA; ++j) {
+        for (int j = 0; j < LOADS_A; ++j) {
             const int index = threadIdx.x + j * kWideThreads;
             *reinterpret_cast<float4*>(&a_tile[index / kWideQuads][(index % kWideQuads) * 4]) = a_next[j];
         }
 #pragma unroll
-        for (int j = 0; j < kWideLoadsW; ++j) {
+        for (int j = 0; j < LOADS_W; ++j) {
             const int index = threadIdx.x + j * kWideThreads;
             *reinterpret_cast<float4*>(&w_tile[index / kWideQuads][(index % kWideQuads) * 4]) = w_next[j];
         }
@@ -255,28 +262,45 @@ __global__ __launch_bounds__(kWideThreads) void gemm_f32_small_wide_kernel(const
         // Four k a read, added one after the other in ascending k.
 #pragma unroll
         for (int kk = 0; kk < kWideDepth; kk += 4) {
-            const float4 a0 = *reinterpret_cast<const float4*>(&a_tile[row][kk]);
-            const float4 a1 = *reinterpret_cast<const float4*>(&a_tile[row + 8][kk]);
-            const float4 w0 = *reinterpret_cast<const float4*>(&w_tile[column][kk]);
-            const float4 w1 = *reinterpret_cast<const float4*>(&w_tile[column + 16][kk]);
-            acc[0][0] = fmaf(a0.x, w0.x, acc[0][0]); acc[0][1] = fmaf(a0.x, w1.x, acc[0][1]);
-            acc[1][0] = fmaf(a1.x, w0.x, acc[1][0]); acc[1][1] = fmaf(a1.x, w1.x, acc[1][1]);
-            acc[0][0] = fmaf(a0.y, w0.y, acc[0][0]); acc[0][1] = fmaf(a0.y, w1.y, acc[0][1]);
-            acc[1][0] = fmaf(a1.y, w0.y, acc[1][0]); acc[1][1] = fmaf(a1.y, w1.y, acc[1][1]);
-            acc[0][0] = fmaf(a0.z, w0.z, acc[0][0]); acc[0][1] = fmaf(a0.z, w1.z, acc[0][1]);
-            acc[1][0] = fmaf(a1.z, w0.z, acc[1][0]); acc[1][1] = fmaf(a1.z, w1.z, acc[1][1]);
-            acc[0][0] = fmaf(a0.w, w0.w, acc[0][0]); acc[0][1] = fmaf(a0.w, w1.w, acc[0][1]);
-            acc[1][0] = fmaf(a1.w, w0.w, acc[1][0]); acc[1][1] = fmaf(a1.w, w1.w, acc[1][1]);
+            float4 av[TR], wv[TC];
+#pragma unroll
+            for (int i = 0; i < TR; ++i) av[i] = *reinterpret_cast<const float4*>(&a_tile[row + 8 * i][kk]);
+#pragma unroll
+            for (int j = 0; j < TC; ++j) wv[j] = *reinterpret_cast<const float4*>(&w_tile[column + 16 * j][kk]);
+#pragma unroll
+            for (int i = 0; i < TR; ++i)
+#pragma unroll
+                for (int j = 0; j < TC; ++j) acc[i][j] = fmaf(av[i].x, wv[j].x, acc[i][j]);
+#pragma unroll
+            for (int i = 0; i < TR; ++i)
+#pragma unroll
+                for (int j = 0; j < TC; ++j) acc[i][j] = fmaf(av[i].y, wv[j].y, acc[i][j]);
+#pragma unroll
+            for (int i = 0; i < TR; ++i)
+#pragma unroll
+                for (int j = 0; j < TC; ++j) acc[i][j] = fmaf(av[i].z, wv[j].z, acc[i][j]);
+#pragma unroll
+            for (int i = 0; i < TR; ++i)
+#pragma unroll
+                for (int j = 0; j < TC; ++j) acc[i][j] = fmaf(av[i].w, wv[j].w, acc[i][j]);
         }
         __syncthreads();
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TR; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < TC; ++j) {
             const int r = row + 8 * i, col = col0 + column + 16 * j;
             if (r < m && col < n) c[static_cast<int64_t>(r) * n + col] = acc[i][j] + (bias ? bias[col] : 0.0f);
         }
+}
+
+template <int TR, int TC>
+static void launch_small_wide(const float* a, const float* w, const float* bias, float* c, int m, int n, int k, int k_split,
+                              unsigned parts, bool vector, hipStream_t stream) {
+    const dim3 grid((n + 16 * TC - 1) / (16 * TC), 1, parts);
+    if (vector) gemm_f32_small_wide_kernel<true, TR, TC><<<grid, kWideThreads, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
+    else gemm_f32_small_wide_kernel<false, TR, TC><<<grid, kWideThreads, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
 }
 
 }  // namespace mll
@@ -286,6 +310,13 @@ using namespace mll;
 // Into how many parts the reduction over k is cut for a weight [n, k]: a function of the weight's shape alone. A
 // weight with few rows of its own (q/k/v, o, down) gives the GPU too few tiles of C; its parts go to workgroups of
 // their own. Parts are at least 448 terms long and at most 8.
+static int f32_wide_columns = 4;      // 2: the kernel of 2 x 2 elements a thread wherever one of 4 columns would be taken
+extern "C" int mll_gemm_f32_wide_columns(int columns) {      // for measurements and tests: the same bits either way
+    const int before = f32_wide_columns;
+    f32_wide_columns = columns == 2 ? 2 : 4;
+    return before;
+}
+
 extern "C" int mll_gemm_f32_splits(int n, int k) {
     if (n >= kWideFrom) return 1;
     int splits = 1;
@@ -304,10 +335,17 @@ extern "C" int mll_gemm_f32(const float* a, const float* w, const float* bias, f
     const unsigned parts = static_cast<unsigned>(splits);
     const bool vector = k % 4 == 0 && reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
     if (m <= 16) {
-        if (n >= kWideFrom || static_cast<int64_t>((n + kWideColumns - 1) / kWideColumns) * splits >= 512) {
-            const dim3 grid((n + kWideColumns - 1) / kWideColumns, 1, parts);
-            if (vector) gemm_f32_small_wide_kernel<true><<<grid, kWideThreads, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
-            else gemm_f32_small_wide_kernel<false><<<grid, kWideThreads, 0, stream>>>(a, w, bias, c, m, n, k, k_split);
+        // Up to 8 rows: one row and four columns a thread where that still gives the GPU its workgroups (weights of
+        // many rows; the others with their parts). Else two rows and two columns where that does, else the kernel of
+        // one element a thread. (Two rows and four columns for 9 to 16 rows are slower than two and two: gate/up at
+        // 7B sizes 131 -> 156 us.)
+        const int64_t quads = static_cast<int64_t>((n + 63) / 64) * splits, pairs = static_cast<int64_t>((n + 31) / 32) * splits;
+        if (m <= 8 && f32_wide_columns != 2 && (n >= kWideFrom || quads >= 384)) {
+            launch_small_wide<1, 4>(a, w, bias, c, m, n, k, k_split, parts, vector, stream);
+            return check_launch("gemm_f32");
+        }
+        if (n >= kWideFrom || pairs >= 512) {
+            launch_small_wide<2, 2>(a, w, bias, c, m, n, k, k_split, parts, vector, stream);
             return check_launch("gemm_f32");
         }
         const dim3 grid((n + kSmallColumns - 1) / kSmallColumns, 1, parts);

@@ -402,6 +402,12 @@ def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
     return out
 
 
+def f32_wide_columns(columns: int) -> int:
+    """For measurements and tests: 2 makes ``gemm_f32`` take its kernel of two columns a thread wherever it would
+    take four (at most 16 rows), 4 gives the choice back; returns the value before. The same bits either way."""
+    return int(library.load().mll_gemm_f32_wide_columns(int(columns)))
+
+
 def f32_splits(n: int, k: int) -> int:
     """Into how many parts ``gemm_f32`` may cut the reduction of a weight ``[n, k]``: the weight's shape decides,
     never the rows of a call, so that a row's bits are the same in every batch."""

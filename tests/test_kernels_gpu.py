@@ -443,9 +443,17 @@ def test_gemm_f32_in_parts_gives_every_row_the_same_bits_in_every_batch(n, k, pa
         part_length = -(-(-(-k // parts)) // 4) * 4
         second = a[:3, part_length:2 * part_length].astype(np.float64) @ w[:, part_length:2 * part_length].astype(np.float64).T
         np.testing.assert_allclose(whole[1, :3].double().cpu().numpy(), second, rtol=3e-5, atol=3e-5 * np.abs(second).max())
-    for rows in (1, 16, 40, 64):
+    for rows in (1, 7, 8, 9, 16, 40, 64):
         fewer = ka.gemm_f32(device_a[:rows].contiguous(), device_w, device_bias, partials=True)
         assert torch.equal(fewer, whole[..., :rows, :]), f"{rows} rows: other bits than the same rows among 600"
+    # up to 16 rows a thread takes four columns of the weight where that fills the GPU, or two: the same bits
+    usual = ka.f32_wide_columns(2)
+    try:
+        for rows in (1, 8, 13, 16):
+            two = ka.gemm_f32(device_a[:rows].contiguous(), device_w, device_bias, partials=True)
+            assert torch.equal(two, whole[..., :rows, :]), f"{rows} rows, two columns a thread"
+    finally:
+        ka.f32_wide_columns(usual)
     unsplit = ka.gemm_f32(device_a[:40].contiguous(), device_w, device_bias)      # one sum an element when the caller wants no parts
     assert tuple(unsplit.shape) == (40, n)
     np.testing.assert_allclose(unsplit.cpu().numpy(), expected[:40], rtol=3e-5, atol=3e-5 * np.abs(expected).max())
