@@ -310,10 +310,12 @@ using namespace mll;
 // Into how many parts the reduction over k is cut for a weight [n, k]: a function of the weight's shape alone. A
 // weight with few rows of its own (q/k/v, o, down) gives the GPU too few tiles of C; its parts go to workgroups of
 // their own. Parts are at least 448 terms long and at most 8.
-static int f32_wide_columns = 4;      // 2: the kernel of 2 x 2 elements a thread wherever one of 4 columns would be taken
-extern "C" int mll_gemm_f32_wide_columns(int columns) {      // for measurements and tests: the same bits either way
-    const int before = f32_wide_columns;
-    f32_wide_columns = columns == 2 ? 2 : 4;
+// Which kernel takes a product of at most 16 rows: 0 the choice below; for measurements and tests 1 (an element a
+// thread), 2 (2 x 2) or 4 (1 x 4, at most 8 rows). The same bits whichever.
+static int f32_small_variant = 0;
+extern "C" int mll_gemm_f32_small_variant(int variant) {
+    const int before = f32_small_variant;
+    f32_small_variant = (variant == 1 || variant == 2 || variant == 4) ? variant : 0;
     return before;
 }
 
@@ -336,15 +338,24 @@ extern "C" int mll_gemm_f32(const float* a, const float* w, const float* bias, f
     const bool vector = k % 4 == 0 && reinterpret_cast<uintptr_t>(a) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
     if (m <= 16) {
         // Up to 8 rows: one row and four columns a thread where that still gives the GPU its workgroups (weights of
-        // many rows; the others with their parts). Else two rows and two columns where that does, else the kernel of
+        // many rows; the others with their parts); else two rows and two columns where that does, else the kernel of
         // one element a thread. (Two rows and four columns for 9 to 16 rows are slower than two and two: gate/up at
-        // 7B sizes 131 -> 156 us.)
+        // 7B sizes 131 -> 156 us. A column a thread with all rows, which reads an element of W from LDS once, is
+        // faster for one row alone (q/k/v 20 -> 16.5 us, down 60 -> 51) and 1 % in the step; from two rows on the
+        // rows of A, read by all lanes at one address, cost more than is saved: 8 rows 115 -> 310 us.)
         const int64_t quads = static_cast<int64_t>((n + 63) / 64) * splits, pairs = static_cast<int64_t>((n + 31) / 32) * splits;
-        if (m <= 8 && f32_wide_columns != 2 && (n >= kWideFrom || quads >= 384)) {
+        int variant = f32_small_variant;
+        if (variant == 4 && m > 8) variant = 2;
+        if (variant == 0) {
+            if (m <= 8 && (n >= kWideFrom || quads >= 384)) variant = 4;
+            else if (n >= kWideFrom || pairs >= 512) variant = 2;
+            else variant = 1;
+        }
+        if (variant == 4) {
             launch_small_wide<1, 4>(a, w, bias, c, m, n, k, k_split, parts, vector, stream);
             return check_launch("gemm_f32");
         }
-        if (n >= kWideFrom || pairs >= 512) {
+        if (variant == 2) {
             launch_small_wide<2, 2>(a, w, bias, c, m, n, k, k_split, parts, vector, stream);
             return check_launch("gemm_f32");
         }

@@ -95,10 +95,9 @@ int mll_silu_mul(const void* gate, const void* up, int64_t in_stride, void* out,
 // (only the number mll_gemm_f32_splits gives for the weight's shape) C is [splits, m, n]: sums over
 // consecutive ranges of k, the bias in the first, for the reader to add in order.
 int mll_gemm_f32_splits(int n, int k);
-// For at most 16 rows a thread of the product takes four columns of a weight where that leaves the GPU its workgroups;
-// 2 makes it take the kernel of two columns there (0 or 4: the choice above again). Returns the value before. The same
-// bits either way.
-int mll_gemm_f32_wide_columns(int columns);
+// Which kernel takes a product of at most 16 rows: 0 gives the choice back to the launch; 1 (an element a thread), 2
+// (two rows and two columns) and 4 (one row and four columns; at most 8 rows) force one, for measurements and tests. Returns the value before. The same bits whichever.
+int mll_gemm_f32_small_variant(int variant);
 int mll_gemm_f32(const float* a, const float* w, const float* bias, float* c,
                  int m, int n, int k, int splits, hipStream_t stream);
 

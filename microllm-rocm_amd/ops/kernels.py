@@ -402,10 +402,11 @@ def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
     return out
 
 
-def f32_wide_columns(columns: int) -> int:
-    """For measurements and tests: 2 makes ``gemm_f32`` take its kernel of two columns a thread wherever it would
-    take four (at most 16 rows), 4 gives the choice back; returns the value before. The same bits either way."""
-    return int(library.load().mll_gemm_f32_wide_columns(int(columns)))
+def f32_small_variant(variant: int) -> int:
+    """For measurements and tests: which kernel ``gemm_f32`` takes for at most 16 rows: 1 (an element a thread), 2
+    (2 x 2 elements) or 4 (1 x 4; at most 8 rows); 0 gives the choice back. Returns the value before. The same
+    bits whichever."""
+    return int(library.load().mll_gemm_f32_small_variant(int(variant)))
 
 
 def f32_splits(n: int, k: int) -> int:

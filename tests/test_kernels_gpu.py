@@ -446,14 +446,16 @@ def test_gemm_f32_in_parts_gives_every_row_the_same_bits_in_every_batch(n, k, pa
     for rows in (1, 7, 8, 9, 16, 40, 64):
         fewer = ka.gemm_f32(device_a[:rows].contiguous(), device_w, device_bias, partials=True)
         assert torch.equal(fewer, whole[..., :rows, :]), f"{rows} rows: other bits than the same rows among 600"
-    # up to 16 rows a thread takes four columns of the weight where that fills the GPU, or two: the same bits
-    usual = ka.f32_wide_columns(2)
+    # up to 16 rows any of three kernels may take the product: the same bits
+    usual = ka.f32_small_variant(0)
     try:
-        for rows in (1, 8, 13, 16):
-            two = ka.gemm_f32(device_a[:rows].contiguous(), device_w, device_bias, partials=True)
-            assert torch.equal(two, whole[..., :rows, :]), f"{rows} rows, two columns a thread"
+        for variant in (1, 2, 4):
+            ka.f32_small_variant(variant)
+            for rows in (1, 2, 3, 5, 8, 13, 16):
+                forced = ka.gemm_f32(device_a[:rows].contiguous(), device_w, device_bias, partials=True)
+                assert torch.equal(forced, whole[..., :rows, :]), f"{rows} rows, kernel {variant}"
     finally:
-        ka.f32_wide_columns(usual)
+        ka.f32_small_variant(usual)
     unsplit = ka.gemm_f32(device_a[:40].contiguous(), device_w, device_bias)      # one sum an element when the caller wants no parts
     assert tuple(unsplit.shape) == (40, n)
     np.testing.assert_allclose(unsplit.cpu().numpy(), expected[:40], rtol=3e-5, atol=3e-5 * np.abs(expected).max())
